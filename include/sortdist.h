@@ -1,0 +1,167 @@
+/*
+ * sortdist -- plain C ABI of the MI355X (gfx950) distance-neuron kernels.
+ *
+ * Every entry point replaces one static launcher of the reference extension
+ * (core/cuda/norm_dist.h, cited per function) one level below its pybind layer
+ * (core/cuda/norm_dist.cpp:294-317): raw device pointers and sizes in, nothing returned
+ * but a status.  Differences from the reference launchers, all additive:
+ *   - a trailing `stream` argument (a hipStream_t passed as void*; NULL = the null stream);
+ *     the reference always used the legacy default stream;
+ *   - an int status instead of void: 0 = ok, SD_ERR_ARG = rejected arguments,
+ *     SD_ERR_HIP = a HIP call or kernel launch failed; sd_last_error() returns the message
+ *     of the calling thread's last failure.
+ *
+ * Conventions (same as the reference): all tensors are contiguous fp32 device memory,
+ * indices are int32.  input is (B, CI, HW), weight is (W_CO, W_CI / G), output is
+ * (B, CO, HW); CI and CO count all groups.  B, CO, CI, HW are what the reference's pybind
+ * layer derives from the tensor sizes.  The optional index lists w_index_ci (S, G, CI/G) and
+ * w_index_co (S, G, CO/G), S = ceil(B/32), select for each 32-sample sub-batch the rows and
+ * columns of weight that the (already compacted) input and output refer to; pass NULL for
+ * the dense case, in which W_CO, W_CI are ignored.  The callee zero-fills every buffer it
+ * scatters into (grad_input, grad_weight), as the reference launchers do, and owns no
+ * caller-visible memory.  pos packs the arg-max input index in bits 0..30 and a branch/sign
+ * flag in bit 31.
+ */
+#ifndef SORTDIST_H
+#define SORTDIST_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SD_OK 0
+#define SD_ERR_ARG 1
+#define SD_ERR_HIP 2
+
+#define SD_MASK_TERM 0      /* independent Bernoulli draw for every (b, m, n) term */
+#define SD_MASK_FACTORED 1  /* keep(b,m,n) = keep_x(b,n) & keep_w(m,n), each with probability sqrt(q) */
+
+typedef void* sd_stream_t;
+
+/* library / error reporting (no reference counterpart) */
+int sd_version(void);
+const char* sd_last_error(void);
+
+/* ---- l-inf distance: struct inf_dist, core/cuda/norm_dist.h:20-31 ---- */
+
+/* inf_dist::forward_nograd (norm_dist.h:21-22; core/cuda/inf_dist_cuda.cu:277-304):
+ * output = max(1e-10, max_n |input - weight|). */
+int sd_inf_dist_forward_nograd(const float* input, const float* weight,
+                               int B, int CO, int CI, int G, int HW, float* output, sd_stream_t stream);
+
+/* inf_dist::forward (norm_dist.h:23-25; inf_dist_cuda.cu:306-323): as above plus
+ * pos = lowest arg-max index | (input - weight < 0) << 31; optional index lists. */
+int sd_inf_dist_forward(const float* input, const float* weight,
+                        int B, int CO, int CI, int G, int HW, float* output, int* pos,
+                        const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI, sd_stream_t stream);
+
+/* inf_dist::backward_input (norm_dist.h:26-27; inf_dist_cuda.cu:325-336). */
+int sd_inf_dist_backward_input(const float* grad_output, const int* pos,
+                               int B, int CO, int CI, int G, int HW, float* grad_input, sd_stream_t stream);
+
+/* inf_dist::backward_input_weight (norm_dist.h:28-30; inf_dist_cuda.cu:338-354).
+ * With index lists grad_weight has the full (W_CO, W_CI / G) shape. */
+int sd_inf_dist_backward_input_weight(const float* grad_output, const int* pos,
+                                      int B, int CO, int CI, int G, int HW, float* grad_input, float* grad_weight,
+                                      const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
+                                      sd_stream_t stream);
+
+/* ---- interval bounds through the l-inf layer: struct bound_inf_dist, norm_dist.h:33-45 ---- */
+
+/* bound_inf_dist::forward_nograd (norm_dist.h:34-35; core/cuda/bound_inf_dist_cuda.cu:314-328). */
+int sd_bound_inf_dist_forward_nograd(const float* inputL, const float* inputU, const float* weight,
+                                     int B, int CO, int CI, int G, int HW, float* outputL, float* outputU,
+                                     sd_stream_t stream);
+
+/* bound_inf_dist::forward (norm_dist.h:36-37; bound_inf_dist_cuda.cu:330-346). */
+int sd_bound_inf_dist_forward(const float* inputL, const float* inputU, const float* weight,
+                              int B, int CO, int CI, int G, int HW, float* outputL, float* outputU,
+                              int* posL, int* posU, sd_stream_t stream);
+
+/* bound_inf_dist::backward_input (norm_dist.h:38-40; bound_inf_dist_cuda.cu:362-371). */
+int sd_bound_inf_dist_backward_input(const float* grad_outputL, const float* grad_outputU,
+                                     const int* posL, const int* posU, int B, int CO, int CI, int G, int HW,
+                                     float* grad_inputL, float* grad_inputU, sd_stream_t stream);
+
+/* bound_inf_dist::backward_input_weight (norm_dist.h:41-44; bound_inf_dist_cuda.cu:373-383). */
+int sd_bound_inf_dist_backward_input_weight(const float* grad_outputL, const float* grad_outputU,
+                                            const int* posL, const int* posU, int B, int CO, int CI, int G, int HW,
+                                            float* grad_inputL, float* grad_inputU, float* grad_weight,
+                                            sd_stream_t stream);
+
+/* ---- sort neuron: struct sort_neuron, norm_dist.h:47-57; K in 2..25 ---- */
+
+/* sort_neuron::forward_nograd (norm_dist.h:48-49; core/cuda/sort_neuron.cu:387-434). */
+int sd_sort_neuron_forward_nograd(const float* input, const float* weight,
+                                  int B, int CO, int CI, int G, int HW, float* output, float q, int K,
+                                  sd_stream_t stream);
+
+/* sort_neuron::forward (norm_dist.h:50-51; sort_neuron.cu:437-485); pos is (K, B, CO, HW). */
+int sd_sort_neuron_forward(const float* input, const float* weight,
+                           int B, int CO, int CI, int G, int HW, float* output, int* pos, float q, int K,
+                           sd_stream_t stream);
+
+/* sort_neuron::backward_input (norm_dist.h:52-53; sort_neuron.cu:536-547). */
+int sd_sort_neuron_backward_input(const float* grad_output, const int* pos,
+                                  int B, int CO, int CI, int G, int HW, float* grad_input, float q, int K,
+                                  sd_stream_t stream);
+
+/* sort_neuron::backward_input_weight (norm_dist.h:54-56; sort_neuron.cu:549-562). */
+int sd_sort_neuron_backward_input_weight(const float* grad_output, const int* pos,
+                                         int B, int CO, int CI, int G, int HW, float* grad_input,
+                                         float* grad_weight, float q, int K, sd_stream_t stream);
+
+/* bound_sort_neuron_forward_cuda (norm_dist.h:60-61; sort_neuron.cu:487-534). */
+int sd_bound_sort_neuron_forward(const float* inputL, const float* inputU, const float* weight,
+                                 int B, int CO, int CI, int G, int HW, float* outputL, float* outputU,
+                                 float q, int K, sd_stream_t stream);
+
+/* ---- l-p norm distance: template struct norm_dist<ip>, norm_dist.h:4-18.  The dispatch on p
+ * that the reference does in its pybind layer (norm_dist.cpp:4,17-38,51-60) happens inside. ---- */
+
+/* norm_dist<ip>::forward / forward_with_max(max_output = nullptr) as selected by
+ * norm_dist_forward (core/cuda/norm_dist.cpp:43-61; norm_dist_cuda.cu:512-552). */
+int sd_norm_dist_forward(const float* input, const float* weight,
+                         int B, int CO, int CI, int G, int HW, float* output, float p,
+                         const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI, sd_stream_t stream);
+
+/* norm_dist<ip>::forward_with_max with a caller-supplied max_output (norm_dist.h:8-10;
+ * norm_dist.cpp:67-80). */
+int sd_norm_dist_forward_with_max(const float* input, const float* weight, const float* max_output,
+                                  int B, int CO, int CI, int G, int HW, float* output, float p,
+                                  const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
+                                  sd_stream_t stream);
+
+/* norm_dist<ip>::backward_input (norm_dist.h:11-13; norm_dist.cpp:86-102). */
+int sd_norm_dist_backward_input(const float* grad_output, const float* input, const float* weight,
+                                const float* output, int B, int CO, int CI, int G, int HW,
+                                float* grad_input, float p,
+                                const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
+                                sd_stream_t stream);
+
+/* norm_dist<ip>::backward_input_weight (norm_dist.h:14-17; norm_dist.cpp:108-125). */
+int sd_norm_dist_backward_input_weight(const float* grad_output, const float* input, const float* weight,
+                                       const float* output, int B, int CO, int CI, int G, int HW,
+                                       float* grad_input, float* grad_weight, float p,
+                                       const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
+                                       sd_stream_t stream);
+
+/* ---- masked order-statistic neuron (no reference launcher: the reference builds its training
+ * mask on the host, core/models/norm_dist.py:14-17, and hands index lists to inf_dist::forward).
+ * output = max(1e-10, max over kept n of |input - weight|) where term (b, m, n) is kept with
+ * probability q, decided by a stateless counter RNG of (seed, b, m, n); pos may be NULL. ---- */
+int sd_masked_inf_dist_forward(const float* input, const float* weight,
+                               int B, int CO, int CI, int G, int HW, float* output, int* pos,
+                               float q, uint32_t seed, int mode, sd_stream_t stream);
+
+/* The counter RNG and the thresholds it is compared with, exposed for verification. */
+uint32_t sd_rng_word(uint32_t seed, uint32_t stream_id, uint32_t row, uint32_t col);
+uint32_t sd_mask_threshold8(float q);
+uint32_t sd_mask_threshold16(float q);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SORTDIST_H */

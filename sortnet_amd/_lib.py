@@ -1,0 +1,79 @@
+"""ctypes binding of libsortdist.so (declarations: include/sortdist.h).
+
+There is no fallback: if the library has not been built, importing anything that needs it
+raises.  Build it with `make -C sortnet_amd/csrc` (or `__graft_entry__.build()`).
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libsortdist.so")
+
+_F = ctypes.c_void_p          # device pointer to float
+_I = ctypes.c_void_p          # device pointer to int32
+_S = ctypes.c_void_p          # hipStream_t
+_i = ctypes.c_int
+_f = ctypes.c_float
+_u = ctypes.c_uint32
+
+# name -> argument types, in the order of include/sortdist.h
+SIGNATURES = {
+    "sd_inf_dist_forward_nograd": [_F, _F, _i, _i, _i, _i, _i, _F, _S],
+    "sd_inf_dist_forward": [_F, _F, _i, _i, _i, _i, _i, _F, _I, _I, _I, _i, _i, _S],
+    "sd_inf_dist_backward_input": [_F, _I, _i, _i, _i, _i, _i, _F, _S],
+    "sd_inf_dist_backward_input_weight": [_F, _I, _i, _i, _i, _i, _i, _F, _F, _I, _I, _i, _i, _S],
+    "sd_bound_inf_dist_forward_nograd": [_F, _F, _F, _i, _i, _i, _i, _i, _F, _F, _S],
+    "sd_bound_inf_dist_forward": [_F, _F, _F, _i, _i, _i, _i, _i, _F, _F, _I, _I, _S],
+    "sd_bound_inf_dist_backward_input": [_F, _F, _I, _I, _i, _i, _i, _i, _i, _F, _F, _S],
+    "sd_bound_inf_dist_backward_input_weight": [_F, _F, _I, _I, _i, _i, _i, _i, _i, _F, _F, _F, _S],
+    "sd_sort_neuron_forward_nograd": [_F, _F, _i, _i, _i, _i, _i, _F, _f, _i, _S],
+    "sd_sort_neuron_forward": [_F, _F, _i, _i, _i, _i, _i, _F, _I, _f, _i, _S],
+    "sd_sort_neuron_backward_input": [_F, _I, _i, _i, _i, _i, _i, _F, _f, _i, _S],
+    "sd_sort_neuron_backward_input_weight": [_F, _I, _i, _i, _i, _i, _i, _F, _F, _f, _i, _S],
+    "sd_bound_sort_neuron_forward": [_F, _F, _F, _i, _i, _i, _i, _i, _F, _F, _f, _i, _S],
+    "sd_norm_dist_forward": [_F, _F, _i, _i, _i, _i, _i, _F, _f, _I, _I, _i, _i, _S],
+    "sd_norm_dist_forward_with_max": [_F, _F, _F, _i, _i, _i, _i, _i, _F, _f, _I, _I, _i, _i, _S],
+    "sd_norm_dist_backward_input": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _f, _I, _I, _i, _i, _S],
+    "sd_norm_dist_backward_input_weight": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _F, _f, _I, _I, _i, _i, _S],
+    "sd_masked_inf_dist_forward": [_F, _F, _i, _i, _i, _i, _i, _F, _I, _f, _u, _i, _S],
+}
+_OTHER = {
+    "sd_version": ([], _i),
+    "sd_last_error": ([], ctypes.c_char_p),
+    "sd_rng_word": ([_u, _u, _u, _u], _u),
+    "sd_mask_threshold8": ([_f], _u),
+    "sd_mask_threshold16": ([_f], _u),
+}
+
+_lib = None
+
+
+def load():
+    """Loads libsortdist.so once; raises RuntimeError if it is missing or incomplete."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "sortnet_amd: %s not found - build the HIP library first (make -C sortnet_amd/csrc); "
+            "there is no fallback path" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, args in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = _i
+    for name, (args, res) in _OTHER.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = res
+    _lib = lib
+    return lib
+
+
+def call(name, *args):
+    """Calls an entry point and turns a non-zero status into RuntimeError."""
+    lib = load()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        msg = lib.sd_last_error()
+        raise RuntimeError("%s failed (status %d): %s" % (name, rc, msg.decode() if msg else "?"))

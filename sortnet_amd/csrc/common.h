@@ -1,0 +1,69 @@
+// Shared definitions of the gfx950 distance-neuron kernels: argument block, counter RNG,
+// error reporting and small utility kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/sortdist.h"
+
+namespace sd {
+
+constexpr float kEps = 1e-10f;            // floor of every distance (core/cuda/inf_dist_cuda.cu:14)
+constexpr uint32_t kSign = 0x80000000u;   // bit 31 of pos
+constexpr uint32_t kNanId = 0xffffffffu;  // "no lower-bound gradient" sentinel (bound_inf_dist_cuda.cu:12)
+constexpr int kSubBatch = 32;             // samples sharing one index list (inf_dist_cuda.cu:8)
+
+// ---- counter RNG: word = mix(mix((seed ^ stream * C1) + row) + (col + 1) * C2) ------------------
+__host__ __device__ __forceinline__ uint32_t rng_mix(uint32_t h) {
+    h ^= h >> 16; h *= 0x21f0aaadu;
+    h ^= h >> 15; h *= 0x735a2d97u;
+    h ^= h >> 15;
+    return h;
+}
+__host__ __device__ __forceinline__ uint32_t rng_row_key(uint32_t seed, uint32_t stream, uint32_t row) {
+    return rng_mix((seed ^ (stream * 0x9e3779b9u)) + row);
+}
+__host__ __device__ __forceinline__ uint32_t rng_word(uint32_t key, uint32_t col) {
+    return rng_mix(key + (col + 1u) * 0x85ebca6bu);
+}
+
+// ---- arguments shared by every forward tile kernel -------------------------------------------
+struct FwdArgs {
+    const float* x0;      // input, or lower bound
+    const float* x1;      // upper bound (interval kernels)
+    const float* w;
+    const float* aux;     // max_output of the with-max l-p forward
+    float* y0;            // output, or lower output
+    float* y1;            // upper output
+    int* p0;              // pos / posL / sort pos (K, B, CO, HW)
+    int* p1;              // posU
+    const int* ci_idx;    // (S, G, CIg) or null
+    const int* co_idx;    // (S, G, COg) or null
+    int B, R, HW, G;      // R = B * HW rows of the batch tile
+    int COg, CIg;         // per-group output / input channels (compact sizes with index lists)
+    int W_COg, W_CIg;     // per-group rows / row length of the weight tensor
+    int nsplit;           // number of slices the reduction range is cut in (grid.z = G * nsplit)
+    int fast_x, fast_w;   // 128-bit loads allowed for the x / w tiles
+    float p, inv_p, q;
+    uint32_t seed, t8, t16;
+    int mask_mode;        // -1 none, SD_MASK_TERM, SD_MASK_FACTORED
+};
+
+// ---- error reporting ---------------------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int check_launch(const char* what);
+
+#define SD_REQUIRE(cond, ...)                                   \
+    do {                                                        \
+        if (!(cond)) { sd::set_error(__VA_ARGS__); return SD_ERR_ARG; } \
+    } while (0)
+
+// number of compute units of the current device (cached)
+int num_cus();
+
+// zero-fill n floats on `stream` with a kernel (graph-capture friendly, no memset node)
+int fill_zero(void* ptr, size_t n_words, hipStream_t stream);
+
+}  // namespace sd

@@ -1,0 +1,526 @@
+// Register/LDS-tiled forward kernel shared by every distance-neuron forward op, and the
+// per-op policies plugged into it.
+//
+// One workgroup = 256 work-items laid out 16 (output channel) x 16 (batch row).  It owns a
+// (16*TB) x (16*TM) tile of outputs; each work-item keeps a TB x TM block of accumulators in
+// registers (rows tb + 16*i, channels tm + 16*j).  The reduction axis is walked in chunks of
+// KT = 32 inputs: the x tile (one or two of them for interval kernels) and the w tile of a
+// chunk are staged in LDS with 128-bit global loads, rows padded to 36 floats so that the
+// 128-bit LDS reads of the 16 distinct rows of a wavefront fall on distinct banks, and are then
+// consumed four inputs at a time.  grid.z carries the group and, for ops whose result can be
+// merged with an atomic max, a slice of the reduction range (split-N) so that small batches
+// still fill 256 compute units.
+#pragma once
+#include <float.h>
+#include "common.h"
+
+namespace sd {
+
+constexpr int KT = 32;        // inputs per LDS chunk
+constexpr int LDP = KT + 4;   // padded LDS row length in floats
+
+// -------------------------------------------------------------------------------------------
+// tile loaders
+// -------------------------------------------------------------------------------------------
+__device__ __forceinline__ float mask_value(float v, uint32_t key, uint32_t n, uint32_t t16) {
+    return (rng_word(key, n) >> 16) < t16 ? v : __builtin_nanf("");
+}
+
+// NX = 1: one input tile.  NX = 2: lower/upper tiles with the inverted-interval repair
+// (core/cuda/bound_inf_dist_cuda.cu:63).
+template <int NX, int BB>
+__device__ __forceinline__ void load_x_tiles(float (*xs0)[LDP], float (*xs1)[LDP], const FwdArgs& a,
+                                             int g, int r0, int k0, int n_end) {
+    const int tid = threadIdx.x;
+    const bool masked = (NX == 1) && a.mask_mode == SD_MASK_FACTORED;
+    if (a.fast_x) {
+        constexpr int NV = BB * (KT / 4);
+        #pragma unroll
+        for (int e0 = 0; e0 < NV; e0 += 256) {
+            int e = e0 + tid;
+            if (NV % 256 != 0 && e >= NV) break;
+            int row = e >> 3, c4 = (e & 7) * 4;
+            int r = r0 + row, n = k0 + c4;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f), u = v;
+            if (r < a.R && n < n_end) {
+                size_t off = (size_t)(r * a.G + g) * a.CIg + n;
+                v = *reinterpret_cast<const float4*>(a.x0 + off);
+                if (NX == 2) {
+                    u = *reinterpret_cast<const float4*>(a.x1 + off);
+                    if (v.x > u.x) v.x = u.x = (v.x + u.x) * 0.5f;
+                    if (v.y > u.y) v.y = u.y = (v.y + u.y) * 0.5f;
+                    if (v.z > u.z) v.z = u.z = (v.z + u.z) * 0.5f;
+                    if (v.w > u.w) v.w = u.w = (v.w + u.w) * 0.5f;
+                }
+                if (masked) {
+                    uint32_t key = rng_row_key(a.seed, 1u, (uint32_t)(r * a.G + g));
+                    v.x = mask_value(v.x, key, n, a.t16);
+                    v.y = mask_value(v.y, key, n + 1, a.t16);
+                    v.z = mask_value(v.z, key, n + 2, a.t16);
+                    v.w = mask_value(v.w, key, n + 3, a.t16);
+                }
+            }
+            *reinterpret_cast<float4*>(&xs0[row][c4]) = v;
+            if (NX == 2) *reinterpret_cast<float4*>(&xs1[row][c4]) = u;
+        }
+    } else {
+        for (int e = tid; e < BB * KT; e += 256) {
+            int row, c;
+            if (a.HW > 1) { c = e / BB; row = e - c * BB; }   // neighbouring rows are contiguous in memory
+            else { row = e / KT; c = e - row * KT; }
+            int r = r0 + row, n = k0 + c;
+            float v = 0.f, u = 0.f;
+            if (r < a.R && n < n_end) {
+                int b = r / a.HW, hw = r - b * a.HW;
+                size_t off = ((size_t)(b * a.G + g) * a.CIg + n) * a.HW + hw;
+                v = a.x0[off];
+                if (NX == 2) {
+                    u = a.x1[off];
+                    if (v > u) v = u = (v + u) * 0.5f;
+                }
+                if (masked) v = mask_value(v, rng_row_key(a.seed, 1u, (uint32_t)((b * a.G + g) * a.HW + hw)), n, a.t16);
+            }
+            xs0[row][c] = v;
+            if (NX == 2) xs1[row][c] = u;
+        }
+    }
+}
+
+template <int BM>
+__device__ __forceinline__ void load_w_tile(float (*ws)[LDP], const FwdArgs& a,
+                                            int g, int s, int m0, int k0, int n_end) {
+    const int tid = threadIdx.x;
+    const bool masked = a.mask_mode == SD_MASK_FACTORED;
+    if (a.fast_w) {
+        constexpr int NV = BM * (KT / 4);
+        #pragma unroll
+        for (int e0 = 0; e0 < NV; e0 += 256) {
+            int e = e0 + tid;
+            if (NV % 256 != 0 && e >= NV) break;
+            int row = e >> 3, c4 = (e & 7) * 4;
+            int m = m0 + row, n = k0 + c4;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (m < a.COg && n < n_end) {
+                int wrow = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + m] : m;
+                v = *reinterpret_cast<const float4*>(a.w + (size_t)(g * a.W_COg + wrow) * a.W_CIg + n);
+                if (masked) {
+                    uint32_t key = rng_row_key(a.seed, 2u, (uint32_t)(g * a.COg + m));
+                    v.x = mask_value(v.x, key, n, a.t16);
+                    v.y = mask_value(v.y, key, n + 1, a.t16);
+                    v.z = mask_value(v.z, key, n + 2, a.t16);
+                    v.w = mask_value(v.w, key, n + 3, a.t16);
+                }
+            }
+            *reinterpret_cast<float4*>(&ws[row][c4]) = v;
+        }
+    } else {
+        for (int e = tid; e < BM * KT; e += 256) {
+            int row = e / KT, c = e - row * KT;
+            int m = m0 + row, n = k0 + c;
+            float v = 0.f;
+            if (m < a.COg && n < n_end) {
+                int wrow = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + m] : m;
+                int wcol = a.ci_idx ? a.ci_idx[(s * a.G + g) * a.CIg + n] : n;
+                v = a.w[(size_t)(g * a.W_COg + wrow) * a.W_CIg + wcol];
+                if (masked) v = mask_value(v, rng_row_key(a.seed, 2u, (uint32_t)(g * a.COg + m)), n, a.t16);
+            }
+            ws[row][c] = v;
+        }
+    }
+}
+
+// -------------------------------------------------------------------------------------------
+// the kernel
+// -------------------------------------------------------------------------------------------
+template <class P, int TB, int TM>
+__global__ void __launch_bounds__(256) fwd_kernel(FwdArgs a) {
+    constexpr int BB = 16 * TB, BM = 16 * TM, NX = P::NX;
+    __shared__ __attribute__((aligned(16))) float xs[NX][BB][LDP];
+    __shared__ __attribute__((aligned(16))) float ws[BM][LDP];
+
+    const int tid = threadIdx.x, tm = tid & 15, tb = tid >> 4;
+    const int g = blockIdx.z % a.G, split = blockIdx.z / a.G;
+    const int r0 = blockIdx.y * BB, m0 = blockIdx.x * BM;
+    const int s = (r0 / a.HW) / kSubBatch;
+
+    const int nchunks = (a.CIg + KT - 1) / KT;
+    const int n_begin = (int)((long long)split * nchunks / a.nsplit) * KT;
+    int n_end = (int)((long long)(split + 1) * nchunks / a.nsplit) * KT;
+    if (n_end > a.CIg) n_end = a.CIg;
+
+    typename P::Acc acc[TB][TM];
+    #pragma unroll
+    for (int i = 0; i < TB; i++) {
+        #pragma unroll
+        for (int j = 0; j < TM; j++) {
+            int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
+            int b = r / a.HW, hw = r - b * a.HW;
+            size_t o = ((size_t)(b * a.G + g) * a.COg + m) * a.HW + hw;
+            P::init(acc[i][j], a, o, r < a.R && m < a.COg);
+        }
+    }
+
+    for (int k0 = n_begin; k0 < n_end; k0 += KT) {
+        load_x_tiles<NX, BB>(xs[0], xs[NX - 1], a, g, r0, k0, n_end);
+        load_w_tile<BM>(ws, a, g, s, m0, k0, n_end);
+        __syncthreads();
+        #pragma unroll
+        for (int pass = 0; pass < P::PASSES; pass++) {
+            #pragma unroll 2
+            for (int n4 = 0; n4 < KT; n4 += 4) {
+                float4 wv[TM];
+                #pragma unroll
+                for (int j = 0; j < TM; j++) wv[j] = *reinterpret_cast<const float4*>(&ws[tm + 16 * j][n4]);
+                #pragma unroll
+                for (int i = 0; i < TB; i++) {
+                    float4 xl = *reinterpret_cast<const float4*>(&xs[0][tb + 16 * i][n4]);
+                    float4 xu = (NX == 2) ? *reinterpret_cast<const float4*>(&xs[NX - 1][tb + 16 * i][n4]) : xl;
+                    #pragma unroll
+                    for (int j = 0; j < TM; j++) P::step4(acc[i][j], a, xl, xu, wv[j], k0 + n4, pass);
+                }
+            }
+            #pragma unroll
+            for (int i = 0; i < TB; i++) {
+                #pragma unroll
+                for (int j = 0; j < TM; j++) P::chunk_end(acc[i][j], a, pass);
+            }
+        }
+        __syncthreads();
+    }
+
+    #pragma unroll
+    for (int i = 0; i < TB; i++) {
+        #pragma unroll
+        for (int j = 0; j < TM; j++) {
+            int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
+            if (r < a.R && m < a.COg) {
+                int b = r / a.HW, hw = r - b * a.HW;
+                size_t o = ((size_t)(b * a.G + g) * a.COg + m) * a.HW + hw;
+                P::store(acc[i][j], a, o);
+            }
+        }
+    }
+}
+
+// host-side launcher; the caller has validated shapes
+template <class P, int TB, int TM>
+int launch_fwd(const FwdArgs& a, hipStream_t stream) {
+    dim3 grid((a.COg + 16 * TM - 1) / (16 * TM), (a.R + 16 * TB - 1) / (16 * TB), a.G * a.nsplit);
+    hipLaunchKernelGGL((fwd_kernel<P, TB, TM>), grid, dim3(256), 0, stream, a);
+    return check_launch("fwd_kernel");
+}
+
+// -------------------------------------------------------------------------------------------
+// policies.  step4 consumes inputs n .. n+3 of one (row, channel) pair.
+// -------------------------------------------------------------------------------------------
+struct PolicyBase {
+    static constexpr int NX = 1;
+    static constexpr int PASSES = 1;
+    template <class A> static __device__ __forceinline__ void chunk_end(A&, const FwdArgs&, int) {}
+};
+
+// l-inf forward without indices (core/cuda/inf_dist_cuda.cu:17-107)
+struct LinfNograd : PolicyBase {
+    struct Acc { float v; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.v = kEps; }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
+                                                 const float4& w, int, int) {
+        float v = A.v;
+        v = fmaxf(fmaxf(v, fabsf(x.x - w.x)), fabsf(x.y - w.y));
+        v = fmaxf(fmaxf(v, fabsf(x.z - w.z)), fabsf(x.w - w.w));
+        A.v = v;
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+        // partial maxima are >= 1e-10 > 0, so their bit patterns order like integers
+        if (a.nsplit > 1) atomicMax(reinterpret_cast<int*>(a.y0 + o), __float_as_int(A.v));
+        else a.y0[o] = A.v;
+    }
+};
+
+// l-inf forward with arg-max index and sign (core/cuda/inf_dist_cuda.cu:110-212): the signed
+// difference of the current winner is kept, a later term replaces it only if strictly larger in
+// magnitude, so the lowest index wins ties and NaN terms never win.
+struct LinfPos : PolicyBase {
+    struct Acc { float bd; int bn; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.bd = kEps; A.bn = 0; }
+    static __device__ __forceinline__ void term(Acc& A, float x, float w, int n) {
+        float d = x - w;
+        if (fabsf(d) > fabsf(A.bd)) { A.bd = d; A.bn = n; }
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
+                                                 const float4& w, int n, int) {
+        term(A, x.x, w.x, n); term(A, x.y, w.y, n + 1); term(A, x.z, w.z, n + 2); term(A, x.w, w.w, n + 3);
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+        a.y0[o] = fabsf(A.bd);
+        a.p0[o] = A.bn | (A.bd < 0.f ? (int)kSign : 0);
+    }
+};
+
+// masked neuron, independent draw per term: byte (n & 3) of word(key(output), n >> 2) < t8 keeps
+template <bool POS>
+struct MaskedTerm : PolicyBase {
+    struct Acc { float bd; int bn; uint32_t key; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool) {
+        A.bd = kEps; A.bn = 0; A.key = rng_row_key(a.seed, 0u, (uint32_t)o);
+    }
+    static __device__ __forceinline__ void term(Acc& A, float x, float w, int n, bool keep) {
+        float d = x - w;
+        if (POS) { if (keep && fabsf(d) > fabsf(A.bd)) { A.bd = d; A.bn = n; } }
+        else A.bd = fmaxf(A.bd, keep ? fabsf(d) : 0.f);
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
+                                                 const float4& w, int n, int) {
+        uint32_t word = rng_word(A.key, (uint32_t)n >> 2);
+        term(A, x.x, w.x, n, (word & 0xffu) < a.t8);
+        term(A, x.y, w.y, n + 1, ((word >> 8) & 0xffu) < a.t8);
+        term(A, x.z, w.z, n + 2, ((word >> 16) & 0xffu) < a.t8);
+        term(A, x.w, w.w, n + 3, (word >> 24) < a.t8);
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+        a.y0[o] = fabsf(A.bd);
+        if (POS) a.p0[o] = A.bn | (A.bd < 0.f ? (int)kSign : 0);
+    }
+};
+
+// interval bounds, values only (core/cuda/bound_inf_dist_cuda.cu:15-118)
+struct BoundNograd : PolicyBase {
+    static constexpr int NX = 2;
+    struct Acc { float lo, hi; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.lo = -kEps; A.hi = kEps; }
+    static __device__ __forceinline__ void term(Acc& A, float l, float u, float w) {
+        float t1 = w - l, t2 = u - w;
+        A.lo = fminf(fminf(A.lo, t1), t2);
+        A.hi = fmaxf(fmaxf(A.hi, t1), t2);
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& l, const float4& u,
+                                                 const float4& w, int, int) {
+        term(A, l.x, u.x, w.x); term(A, l.y, u.y, w.y); term(A, l.z, u.z, w.z); term(A, l.w, u.w, w.w);
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+        if (a.nsplit > 1) {
+            atomicMax(reinterpret_cast<int*>(a.y0 + o), __float_as_int(-A.lo));
+            atomicMax(reinterpret_cast<int*>(a.y1 + o), __float_as_int(A.hi));
+        } else { a.y0[o] = -A.lo; a.y1[o] = A.hi; }
+    }
+};
+
+// interval bounds with indices (core/cuda/bound_inf_dist_cuda.cu:121-238)
+struct BoundPos : PolicyBase {
+    static constexpr int NX = 2;
+    struct Acc { float lo, hi; uint32_t pl, pu; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
+        A.lo = -kEps; A.hi = kEps; A.pl = kNanId; A.pu = 0u;
+    }
+    static __device__ __forceinline__ void term(Acc& A, float l, float u, float w, int n) {
+        float t1 = w - l, t2 = u - w;
+        float mn = fminf(t1, t2), mx = fmaxf(t1, t2);
+        uint32_t p = (uint32_t)n | (t1 <= t2 ? 0u : kSign);
+        if (mn < A.lo) { A.lo = mn; A.pl = p; }
+        if (mx > A.hi) { A.hi = mx; A.pu = p; }
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& l, const float4& u,
+                                                 const float4& w, int n, int) {
+        term(A, l.x, u.x, w.x, n); term(A, l.y, u.y, w.y, n + 1);
+        term(A, l.z, u.z, w.z, n + 2); term(A, l.w, u.w, w.w, n + 3);
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+        a.y0[o] = -A.lo; a.y1[o] = A.hi;
+        a.p0[o] = (int)A.pl; a.p1[o] = (int)A.pu;
+    }
+};
+
+// ---- sort neuron -------------------------------------------------------------------------
+// res[] ascending (res[K-1] largest), slots start at 0.  A value v > res[0] is inserted above
+// equal values: new[k] = clamp(v, res[k], res[k+1]), new[K-1] = max(res[K-1], v); the index
+// array follows the same comparisons (core/cuda/sort_neuron.cu:73-77,176-185).
+template <int K>
+__device__ __forceinline__ void topk_insert_values(float (&res)[K], float v) {
+    #pragma unroll
+    for (int k = 0; k < K - 1; k++) res[k] = __builtin_amdgcn_fmed3f(res[k], v, res[k + 1]);
+    res[K - 1] = fmaxf(res[K - 1], v);
+}
+template <int K>
+__device__ __forceinline__ void topk_insert(float (&res)[K], int (&idx)[K], float v, int p) {
+    #pragma unroll
+    for (int k = 0; k < K - 1; k++) {
+        bool below_next = v < res[k + 1], above_cur = v >= res[k];
+        idx[k] = below_next ? (above_cur ? p : idx[k]) : idx[k + 1];
+        res[k] = below_next ? (above_cur ? v : res[k]) : res[k + 1];
+    }
+    bool top = v >= res[K - 1];
+    idx[K - 1] = top ? p : idx[K - 1];
+    res[K - 1] = top ? v : res[K - 1];
+}
+// y = (init + sum_j t_j c_j q) / (1 - c_K), largest first, every product rounded separately
+template <int K>
+__device__ __forceinline__ float geo_sum(const float (&res)[K], float q) {
+    float ans = kEps, c = 1.f;
+    #pragma unroll
+    for (int k = K - 1; k >= 0; k--) { ans += res[k] * c * q; c *= 1.f - q; }
+    return ans / (1.f - c);
+}
+
+template <int K>
+struct SortNograd : PolicyBase {
+    struct Acc { float res[K]; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
+        #pragma unroll
+        for (int k = 0; k < K; k++) A.res[k] = 0.f;
+    }
+    static __device__ __forceinline__ void term(Acc& A, float x, float w) {
+        float v = fabsf(x - w);
+        if (v > A.res[0]) topk_insert_values<K>(A.res, v);
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
+                                                 const float4& w, int, int) {
+        term(A, x.x, w.x); term(A, x.y, w.y); term(A, x.z, w.z); term(A, x.w, w.w);
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) { a.y0[o] = geo_sum<K>(A.res, a.q); }
+};
+
+template <int K>
+struct SortPos : PolicyBase {
+    struct Acc { float res[K]; int idx[K]; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
+        #pragma unroll
+        for (int k = 0; k < K; k++) { A.res[k] = 0.f; A.idx[k] = 0; }
+    }
+    static __device__ __forceinline__ void term(Acc& A, float x, float w, int n) {
+        float d = x - w, v = fabsf(d);
+        if (v > A.res[0]) topk_insert<K>(A.res, A.idx, v, n | (d >= 0.f ? 0 : (int)kSign));
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
+                                                 const float4& w, int n, int) {
+        term(A, x.x, w.x, n); term(A, x.y, w.y, n + 1); term(A, x.z, w.z, n + 2); term(A, x.w, w.w, n + 3);
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+        a.y0[o] = geo_sum<K>(A.res, a.q);
+        size_t size = (size_t)a.B * a.G * a.COg * a.HW;
+        #pragma unroll
+        for (int k = K - 1; k >= 0; k--) a.p0[(size_t)(K - 1 - k) * size + o] = A.idx[k];
+    }
+};
+
+// interval bounds of the sort neuron (core/cuda/sort_neuron.cu:216-314).  The lower side keeps
+// the negated K most negative values of min(t1,t2), so both sides share the insertion routine.
+template <int K>
+struct BoundSort : PolicyBase {
+    static constexpr int NX = 2;
+    struct Acc { float lo[K], hi[K]; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
+        #pragma unroll
+        for (int k = 0; k < K; k++) { A.lo[k] = 0.f; A.hi[k] = 0.f; }
+    }
+    static __device__ __forceinline__ void term(Acc& A, float l, float u, float w) {
+        float t1 = w - l, t2 = u - w;
+        float nl = -fminf(t1, t2), hu = fmaxf(t1, t2);
+        if (nl > A.lo[0]) topk_insert_values<K>(A.lo, nl);
+        if (hu > A.hi[0]) topk_insert_values<K>(A.hi, hu);
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& l, const float4& u,
+                                                 const float4& w, int, int) {
+        term(A, l.x, u.x, w.x); term(A, l.y, u.y, w.y); term(A, l.z, u.z, w.z); term(A, l.w, u.w, w.w);
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+        a.y0[o] = geo_sum<K>(A.lo, a.q);
+        a.y1[o] = geo_sum<K>(A.hi, a.q);
+    }
+};
+
+// ---- l-p norm distance ---------------------------------------------------------------------
+// a^ip for a >= 0 by multiply chains for ip = 1..8 (core/cuda/fast_pow.cuh:1-12), otherwise
+// exp2(p log2 a) on the hardware transcendental units.
+template <int IP>
+__device__ __forceinline__ float pow_pos(float a, float p) {
+    float t1;
+    switch (IP) {
+        case 0: return 1.f;
+        case 1: return a;
+        case 2: return a * a;
+        case 3: return a * a * a;
+        case 4: t1 = a * a; return t1 * t1;
+        case 5: t1 = a * a; return a * t1 * t1;
+        case 6: t1 = a * a; return t1 * t1 * t1;
+        case 7: t1 = a * a; return a * t1 * t1 * t1;
+        case 8: t1 = a * a; t1 = t1 * t1; return t1 * t1;
+        default: return __builtin_amdgcn_exp2f(p * __builtin_amdgcn_logf(a));
+    }
+}
+
+// p <= 10: y = max(sum |d|^p, FLT_MIN)^(1/p)   (core/cuda/norm_dist_cuda.cu:163-259, no max)
+template <int IP>
+struct LpPlain : PolicyBase {
+    struct Acc { float s; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.s = 0.f; }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
+                                                 const float4& w, int, int) {
+        A.s += pow_pos<IP>(fabsf(x.x - w.x), a.p);
+        A.s += pow_pos<IP>(fabsf(x.y - w.y), a.p);
+        A.s += pow_pos<IP>(fabsf(x.z - w.z), a.p);
+        A.s += pow_pos<IP>(fabsf(x.w - w.w), a.p);
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+        a.y0[o] = powf(fmaxf(A.s, FLT_MIN), a.inv_p);
+    }
+};
+
+// p > 10: running maximum M with rescaling, two passes over every LDS chunk
+// (core/cuda/norm_dist_cuda.cu:36-160): y = M (sum (|d|/M)^p + (1e-10/M)^p)^(1/p).
+template <int IP>
+struct LpOnline : PolicyBase {
+    static constexpr int PASSES = 2;
+    struct Acc { float s, M, rinv, cm; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
+        A.s = 1.f; A.M = kEps; A.rinv = 1.f / kEps; A.cm = 0.f;
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
+                                                 const float4& w, int, int pass) {
+        if (pass == 0) {
+            float v = A.cm;
+            v = fmaxf(fmaxf(v, fabsf(x.x - w.x)), fabsf(x.y - w.y));
+            v = fmaxf(fmaxf(v, fabsf(x.z - w.z)), fabsf(x.w - w.w));
+            A.cm = v;
+        } else {
+            A.s += pow_pos<IP>(fabsf(x.x - w.x) * A.rinv, a.p);
+            A.s += pow_pos<IP>(fabsf(x.y - w.y) * A.rinv, a.p);
+            A.s += pow_pos<IP>(fabsf(x.z - w.z) * A.rinv, a.p);
+            A.s += pow_pos<IP>(fabsf(x.w - w.w) * A.rinv, a.p);
+        }
+    }
+    static __device__ __forceinline__ void chunk_end(Acc& A, const FwdArgs& a, int pass) {
+        if (pass == 0) {
+            if (A.cm > A.M) {
+                A.s *= __builtin_amdgcn_exp2f(a.p * __builtin_amdgcn_logf(A.M / A.cm));
+                A.M = A.cm;
+                A.rinv = 1.f / A.cm;
+            }
+            A.cm = 0.f;
+        }
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+        a.y0[o] = powf(A.s, a.inv_p) * A.M;
+    }
+};
+
+// caller-supplied maximum (core/cuda/norm_dist_cuda.cu:163-259 with has_max)
+template <int IP>
+struct LpWithMax : PolicyBase {
+    struct Acc { float s, rinv; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool valid) {
+        A.rinv = valid ? 1.f / a.aux[o] : 1.f;
+        A.s = __builtin_amdgcn_exp2f(a.p * __builtin_amdgcn_logf(kEps * A.rinv));
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
+                                                 const float4& w, int, int) {
+        A.s += pow_pos<IP>(fabsf(x.x - w.x) * A.rinv, a.p);
+        A.s += pow_pos<IP>(fabsf(x.y - w.y) * A.rinv, a.p);
+        A.s += pow_pos<IP>(fabsf(x.z - w.z) * A.rinv, a.p);
+        A.s += pow_pos<IP>(fabsf(x.w - w.w) * A.rinv, a.p);
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+        a.y0[o] = powf(A.s, a.inv_p) / A.rinv;
+    }
+};
+
+}  // namespace sd

@@ -1,0 +1,87 @@
+// Library runtime: error reporting, device queries, fill kernel and the verification exports.
+#include <cmath>
+#include "common.h"
+
+namespace sd {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("%s: %s", what, hipGetErrorString(e));
+        return SD_ERR_HIP;
+    }
+    return SD_OK;
+}
+
+int num_cus() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+__global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t* __restrict__ p, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * 256;
+    size_t n4 = n / 4;
+    uint4* p4 = reinterpret_cast<uint4*>(p);
+    for (size_t k = i; k < n4; k += stride) p4[k] = make_uint4(0u, 0u, 0u, 0u);
+    for (size_t k = n4 * 4 + i; k < n; k += stride) p[k] = 0u;
+}
+
+int fill_zero(void* ptr, size_t n_words, hipStream_t stream) {
+    if (n_words == 0) return SD_OK;
+    if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) {
+        set_error("fill_zero: buffer must be 16-byte aligned");
+        return SD_ERR_ARG;
+    }
+    size_t blocks = (n_words / 4 + 255) / 256;
+    size_t cap = (size_t)num_cus() * 16;
+    if (blocks > cap) blocks = cap;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                       reinterpret_cast<uint32_t*>(ptr), n_words);
+    return check_launch("fill_zero");
+}
+
+}  // namespace sd
+
+extern "C" {
+
+int sd_version(void) { return 100; }
+
+const char* sd_last_error(void) { return sd::g_err; }
+
+uint32_t sd_rng_word(uint32_t seed, uint32_t stream_id, uint32_t row, uint32_t col) {
+    return sd::rng_word(sd::rng_row_key(seed, stream_id, row), col);
+}
+
+uint32_t sd_mask_threshold8(float q) {
+    double t = std::floor((double)q * 256.0 + 0.5);
+    if (t < 0) t = 0;
+    if (t > 256) t = 256;
+    return (uint32_t)t;
+}
+
+uint32_t sd_mask_threshold16(float q) {
+    double t = std::floor(std::sqrt((double)q) * 65536.0 + 0.5);
+    if (t < 0) t = 0;
+    if (t > 65536) t = 65536;
+    return (uint32_t)t;
+}
+
+}  // extern "C"

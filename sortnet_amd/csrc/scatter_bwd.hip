@@ -1,0 +1,193 @@
+// Backward of the arg-max style ops (l-inf, sort neuron, interval bounds): every output sends its
+// upstream gradient to the saved input position(s) of grad_input and grad_weight
+// (core/cuda/inf_dist_cuda.cu:214-271, sort_neuron.cu:316-375, bound_inf_dist_cuda.cu:240-299).
+// Both targets are zero-filled here and accumulated with hardware fp32 atomic adds.
+#include <cmath>
+#include "common.h"
+
+namespace sd {
+
+struct BwdArgs {
+    const float* g0; const float* g1;    // upstream gradient (lower / upper for the interval op)
+    const int* p0; const int* p1;        // saved positions
+    float* gx0; float* gx1; float* gw;   // gw may be null
+    const int* ci_idx; const int* co_idx;
+    int B, HW, G, COg, CIg, W_COg, W_CIg;
+    int K;                               // slots per output (1 for l-inf)
+    float q, coef0;                      // sort neuron: first coefficient 1/(1-(1-q)^K) and ratio
+    long long total;                     // B * CO * HW
+};
+
+// l-inf (K = 1, unit coefficient) and sort neuron (K slots, geometric coefficients)
+template <bool SORT, bool HAS_W>
+__global__ void __launch_bounds__(256) scatter_bwd_kernel(BwdArgs a) {
+    long long o = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (o >= a.total) return;
+    int hw = (int)(o % a.HW);
+    long long t = o / a.HW;
+    int c = (int)(t % (a.G * a.COg));
+    int b = (int)(t / (a.G * a.COg));
+    int g = c / a.COg, m = c - g * a.COg;
+    int s = b / kSubBatch;
+    float grad = a.g0[o];
+    float coef = a.coef0;
+    size_t xbase = ((size_t)(b * a.G + g) * a.CIg) * a.HW + hw;
+    size_t wrow = 0;
+    if (HAS_W) {
+        int mm = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + m] : m;
+        wrow = (size_t)(g * a.W_COg + mm) * a.W_CIg;
+    }
+    const int K = SORT ? a.K : 1;
+    for (int k = 0; k < K; k++) {
+        int pr = a.p0[(size_t)k * a.total + o];
+        int n = pr & 0x7fffffff;
+        float v = pr >= 0 ? grad : -grad;
+        if (SORT) { v = v * coef * a.q; coef *= 1.f - a.q; }
+        unsafeAtomicAdd(a.gx0 + xbase + (size_t)n * a.HW, v);
+        if (HAS_W) {
+            int nn = a.ci_idx ? a.ci_idx[(s * a.G + g) * a.CIg + n] : n;
+            unsafeAtomicAdd(a.gw + wrow + nn, -v);
+        }
+    }
+}
+
+template <bool HAS_W>
+__global__ void __launch_bounds__(256) bound_bwd_kernel(BwdArgs a) {
+    long long o = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (o >= a.total) return;
+    int hw = (int)(o % a.HW);
+    long long t = o / a.HW;
+    int c = (int)(t % (a.G * a.COg));
+    int b = (int)(t / (a.G * a.COg));
+    int g = c / a.COg;
+    size_t xbase = ((size_t)(b * a.G + g) * a.CIg) * a.HW + hw;
+    size_t wrow = (size_t)c * a.CIg;
+    int pl = a.p0[o], pu = a.p1[o];
+    float gl = a.g0[o], gu = a.g1[o];
+    int nl = pl & 0x7fffffff, nu = pu & 0x7fffffff;
+    float vl = pl >= 0 ? gl : -gl, vu = pu >= 0 ? gu : -gu;
+    if ((uint32_t)pl != kNanId) {
+        unsafeAtomicAdd((pl >= 0 ? a.gx0 : a.gx1) + xbase + (size_t)nl * a.HW, vl);
+        if (HAS_W) unsafeAtomicAdd(a.gw + wrow + nl, -vl);
+    }
+    unsafeAtomicAdd((pu >= 0 ? a.gx1 : a.gx0) + xbase + (size_t)nu * a.HW, vu);
+    if (HAS_W) unsafeAtomicAdd(a.gw + wrow + nu, -vu);
+}
+
+static int make_bwd_args(BwdArgs& a, const char* who, int B, int CO, int CI, int G, int HW,
+                         const int* ci_idx, const int* co_idx, int W_CO, int W_CI) {
+    SD_REQUIRE(B > 0 && CO > 0 && CI > 0 && G > 0 && HW > 0, "%s: sizes must be positive", who);
+    SD_REQUIRE(CO % G == 0 && CI % G == 0, "%s: CO=%d and CI=%d must be multiples of G=%d", who, CO, CI, G);
+    SD_REQUIRE((long long)B * CO * HW < (1ll << 31) && (long long)B * CI * HW < (1ll << 31),
+               "%s: tensor too large for 32-bit indexing", who);
+    a = BwdArgs{};
+    a.B = B; a.HW = HW; a.G = G; a.COg = CO / G; a.CIg = CI / G;
+    a.ci_idx = ci_idx; a.co_idx = co_idx;
+    if (co_idx) { SD_REQUIRE(W_CO > 0 && W_CO % G == 0, "%s: bad W_CO=%d", who, W_CO); a.W_COg = W_CO / G; }
+    else a.W_COg = a.COg;
+    if (ci_idx) { SD_REQUIRE(W_CI > 0 && W_CI % G == 0, "%s: bad W_CI=%d", who, W_CI); a.W_CIg = W_CI / G; }
+    else a.W_CIg = a.CIg;
+    a.K = 1; a.q = 1.f; a.coef0 = 1.f;
+    a.total = (long long)B * CO * HW;
+    return SD_OK;
+}
+
+template <bool SORT>
+static int run_scatter(BwdArgs& a, hipStream_t st) {
+    int rc;
+    if ((rc = fill_zero(a.gx0, (size_t)a.B * a.G * a.CIg * a.HW, st))) return rc;
+    if (a.gw && (rc = fill_zero(a.gw, (size_t)a.G * a.W_COg * a.W_CIg, st))) return rc;
+    dim3 grid((unsigned)((a.total + 255) / 256));
+    if (a.gw) hipLaunchKernelGGL((scatter_bwd_kernel<SORT, true>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((scatter_bwd_kernel<SORT, false>), grid, dim3(256), 0, st, a);
+    return check_launch("scatter_bwd_kernel");
+}
+
+}  // namespace sd
+
+using namespace sd;
+
+extern "C" int sd_inf_dist_backward_input(const float* grad_output, const int* pos,
+                                          int B, int CO, int CI, int G, int HW, float* grad_input, sd_stream_t stream) {
+    BwdArgs a;
+    int rc = make_bwd_args(a, "inf_dist_backward_input", B, CO, CI, G, HW, nullptr, nullptr, 0, 0);
+    if (rc) return rc;
+    SD_REQUIRE(grad_output && pos && grad_input, "inf_dist_backward_input: null pointer");
+    a.g0 = grad_output; a.p0 = pos; a.gx0 = grad_input;
+    return run_scatter<false>(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int sd_inf_dist_backward_input_weight(const float* grad_output, const int* pos,
+                                                 int B, int CO, int CI, int G, int HW, float* grad_input,
+                                                 float* grad_weight, const int* w_index_ci, const int* w_index_co,
+                                                 int W_CO, int W_CI, sd_stream_t stream) {
+    BwdArgs a;
+    int rc = make_bwd_args(a, "inf_dist_backward_input_weight", B, CO, CI, G, HW, w_index_ci, w_index_co, W_CO, W_CI);
+    if (rc) return rc;
+    SD_REQUIRE(grad_output && pos && grad_input && grad_weight, "inf_dist_backward_input_weight: null pointer");
+    a.g0 = grad_output; a.p0 = pos; a.gx0 = grad_input; a.gw = grad_weight;
+    return run_scatter<false>(a, static_cast<hipStream_t>(stream));
+}
+
+static int sort_bwd(const char* who, const float* grad_output, const int* pos, int B, int CO, int CI, int G, int HW,
+                    float* grad_input, float* grad_weight, float q, int K, sd_stream_t stream) {
+    BwdArgs a;
+    int rc = make_bwd_args(a, who, B, CO, CI, G, HW, nullptr, nullptr, 0, 0);
+    if (rc) return rc;
+    SD_REQUIRE(grad_output && pos && grad_input, "%s: null pointer", who);
+    SD_REQUIRE(K >= 1 && K <= 25, "%s: K=%d outside 1..25", who, K);
+    SD_REQUIRE(q > 0.f && q <= 1.f, "%s: q=%g outside (0, 1]", who, (double)q);
+    a.g0 = grad_output; a.p0 = pos; a.gx0 = grad_input; a.gw = grad_weight;
+    a.K = K; a.q = q;
+    float r = powf(1.f - q, (float)K);          // core/cuda/sort_neuron.cu:322
+    a.coef0 = 1.f + r / (1.f - r);
+    return run_scatter<true>(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int sd_sort_neuron_backward_input(const float* grad_output, const int* pos,
+                                             int B, int CO, int CI, int G, int HW, float* grad_input,
+                                             float q, int K, sd_stream_t stream) {
+    return sort_bwd("sort_neuron_backward_input", grad_output, pos, B, CO, CI, G, HW, grad_input, nullptr, q, K, stream);
+}
+
+extern "C" int sd_sort_neuron_backward_input_weight(const float* grad_output, const int* pos,
+                                                    int B, int CO, int CI, int G, int HW, float* grad_input,
+                                                    float* grad_weight, float q, int K, sd_stream_t stream) {
+    SD_REQUIRE(grad_weight, "sort_neuron_backward_input_weight: null grad_weight");
+    return sort_bwd("sort_neuron_backward_input_weight", grad_output, pos, B, CO, CI, G, HW, grad_input, grad_weight,
+                    q, K, stream);
+}
+
+static int bound_bwd(const char* who, const float* gL, const float* gU, const int* posL, const int* posU,
+                     int B, int CO, int CI, int G, int HW, float* gxL, float* gxU, float* gw, sd_stream_t stream) {
+    BwdArgs a;
+    int rc = make_bwd_args(a, who, B, CO, CI, G, HW, nullptr, nullptr, 0, 0);
+    if (rc) return rc;
+    SD_REQUIRE(gL && gU && posL && posU && gxL && gxU, "%s: null pointer", who);
+    a.g0 = gL; a.g1 = gU; a.p0 = posL; a.p1 = posU; a.gx0 = gxL; a.gx1 = gxU; a.gw = gw;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    size_t nx = (size_t)B * CI * HW;
+    if ((rc = fill_zero(gxL, nx, st))) return rc;
+    if ((rc = fill_zero(gxU, nx, st))) return rc;
+    if (gw && (rc = fill_zero(gw, (size_t)CO * a.CIg, st))) return rc;
+    dim3 grid((unsigned)((a.total + 255) / 256));
+    if (gw) hipLaunchKernelGGL((bound_bwd_kernel<true>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((bound_bwd_kernel<false>), grid, dim3(256), 0, st, a);
+    return check_launch("bound_bwd_kernel");
+}
+
+extern "C" int sd_bound_inf_dist_backward_input(const float* grad_outputL, const float* grad_outputU,
+                                                const int* posL, const int* posU, int B, int CO, int CI, int G, int HW,
+                                                float* grad_inputL, float* grad_inputU, sd_stream_t stream) {
+    return bound_bwd("bound_inf_dist_backward_input", grad_outputL, grad_outputU, posL, posU, B, CO, CI, G, HW,
+                     grad_inputL, grad_inputU, nullptr, stream);
+}
+
+extern "C" int sd_bound_inf_dist_backward_input_weight(const float* grad_outputL, const float* grad_outputU,
+                                                       const int* posL, const int* posU, int B, int CO, int CI, int G,
+                                                       int HW, float* grad_inputL, float* grad_inputU,
+                                                       float* grad_weight, sd_stream_t stream) {
+    SD_REQUIRE(grad_weight, "bound_inf_dist_backward_input_weight: null grad_weight");
+    return bound_bwd("bound_inf_dist_backward_input_weight", grad_outputL, grad_outputU, posL, posU, B, CO, CI, G, HW,
+                     grad_inputL, grad_inputU, grad_weight, stream);
+}

@@ -1,0 +1,283 @@
+"""Functional / autograd front-end of the distance-neuron kernels.
+
+Public names, positional order, defaults, return shapes and dtypes follow the reference's
+core/norm_dist.py (file:line cited per symbol) so that its layers (core/models/norm_dist.py)
+run unmodified on top of this module.  Inputs are 3-D (B, C, HW) fp32 tensors on the GPU,
+weight is (CO, CI / groups); outputs are fp32 on the input's device, positions are int32.
+
+Every function dispatches to the HIP kernels through `sortnet_amd.ext`; there is no pure-torch
+path, so `use_custom_cuda_func=False` (which selects one in the reference) is rejected.
+"""
+import math
+
+import torch
+
+from . import ext as _C
+
+__all__ = [
+    "NormDistF", "NormDistDropoutF", "SortNeuronF", "BoundInfDistF", "MaskedInfDistF",
+    "norm_dist", "norm_dist_dropout", "sort_neuron", "bound_sort_neuron", "bound_inf_dist", "masked_inf_dist",
+]
+
+
+def _new_out(x, channels):
+    return torch.empty(x.size(0), channels, x.size(2), device=x.device, dtype=torch.float32)
+
+
+def _want_grad(*tensors):
+    return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+
+
+def _no_fallback(flag, name):
+    if not flag:
+        raise NotImplementedError(
+            "%s: use_custom_cuda_func=False selects a pure-torch path in the reference; this library "
+            "only runs its HIP kernels" % name)
+
+
+class NormDistF(torch.autograd.Function):
+    """l-p (finite p) or l-inf (p = inf) distance layer.  Mirrors core/norm_dist.py:6-51."""
+
+    @staticmethod
+    def forward(ctx, x, weight, group, p, need_grad, tag):
+        assert weight.size(1) * group == x.size(1)
+        y = _new_out(x, weight.size(0))
+        ctx.group, ctx.p, ctx.tag = group, p, tag
+        if math.isinf(p):
+            if need_grad:
+                pos = torch.empty_like(y, dtype=torch.int)
+                _C.inf_dist_forward(x, weight, y, pos, group)
+                ctx.save_for_backward(x, weight, pos)
+            else:
+                _C.inf_dist_forward_nograd(x, weight, y, group)
+        elif p > 0:
+            _C.norm_dist_forward(x, weight, y, group, p)
+            ctx.save_for_backward(x, weight, y)
+        else:
+            raise NotImplementedError
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        grad_output = grad_output.contiguous()
+        want_x, want_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        grad_weight = None
+        if math.isinf(ctx.p):
+            x, weight, pos = ctx.saved_tensors
+            grad_input = torch.empty_like(x)
+            if want_w:
+                grad_weight = torch.empty_like(weight)
+                _C.inf_dist_backward_input_weight(grad_output, pos, grad_input, grad_weight, ctx.group)
+            elif want_x:
+                _C.inf_dist_backward_input(grad_output, pos, grad_input, ctx.group)
+        else:
+            x, weight, y = ctx.saved_tensors
+            grad_input = torch.empty_like(x)
+            if want_w:
+                grad_weight = torch.empty_like(weight)
+                _C.norm_dist_backward_input_weight(grad_output, x, weight, y, grad_input, grad_weight,
+                                                   ctx.group, ctx.p)
+            elif want_x:
+                _C.norm_dist_backward_input(grad_output, x, weight, y, grad_input, ctx.group, ctx.p)
+        return (grad_input if want_x else None), grad_weight, None, None, None, None
+
+
+class NormDistDropoutF(torch.autograd.Function):
+    """Distance layer on index-list sub-matrices of the weight, one list per 32-sample sub-batch.
+    Mirrors core/norm_dist.py:54-99."""
+
+    @staticmethod
+    def forward(ctx, x, weight, w_index_ci, w_index_co, group, p, tag):
+        channels = weight.size(0) if w_index_co is None else w_index_co.size(-1) * group
+        assert weight.size(1) * group == x.size(1) or w_index_ci.size(-1) * group == x.size(1)
+        y = _new_out(x, channels)
+        ctx.group, ctx.p, ctx.tag = group, p, tag
+        if math.isinf(p):
+            pos = torch.empty_like(y, dtype=torch.int)
+            _C.inf_dist_forward(x, weight, y, pos, group, w_index_ci, w_index_co)
+            ctx.save_for_backward(x, weight, pos, w_index_ci, w_index_co)
+        elif p > 0:
+            _C.norm_dist_forward(x, weight, y, group, p, w_index_ci, w_index_co)
+            ctx.save_for_backward(x, weight, y, w_index_ci, w_index_co)
+        else:
+            raise NotImplementedError
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        grad_output = grad_output.contiguous()
+        want_x, want_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        grad_weight = None
+        if math.isinf(ctx.p):
+            x, weight, pos, w_index_ci, w_index_co = ctx.saved_tensors
+            grad_input = torch.empty_like(x)
+            if want_w:
+                grad_weight = torch.empty_like(weight)
+                _C.inf_dist_backward_input_weight(grad_output, pos, grad_input, grad_weight, ctx.group,
+                                                  w_index_ci, w_index_co)
+            elif want_x:
+                _C.inf_dist_backward_input(grad_output, pos, grad_input, ctx.group)
+        else:
+            x, weight, y, w_index_ci, w_index_co = ctx.saved_tensors
+            grad_input = torch.empty_like(x)
+            if want_w:
+                grad_weight = torch.empty_like(weight)
+                _C.norm_dist_backward_input_weight(grad_output, x, weight, y, grad_input, grad_weight,
+                                                   ctx.group, ctx.p, w_index_ci, w_index_co)
+            elif want_x:
+                _C.norm_dist_backward_input(grad_output, x, weight, y, grad_input, ctx.group, ctx.p,
+                                            w_index_ci, w_index_co)
+        return (grad_input if want_x else None), grad_weight, None, None, None, None, None
+
+
+class SortNeuronF(torch.autograd.Function):
+    """Geometric-weighted sum of the top-`truncate` values of |x - w|.  Mirrors core/norm_dist.py:102-133."""
+
+    @staticmethod
+    def forward(ctx, x, weight, group, q, truncate, need_grad, tag):
+        assert weight.size(1) * group == x.size(1)
+        y = _new_out(x, weight.size(0))
+        ctx.group, ctx.q, ctx.truncate, ctx.tag = group, q, truncate, tag
+        if need_grad:
+            pos = torch.empty(truncate, x.size(0), weight.size(0), x.size(2), device=x.device, dtype=torch.int)
+            _C.sort_neuron_forward(x, weight, y, pos, group, q, truncate)
+            ctx.save_for_backward(x, weight, pos)
+        else:
+            _C.sort_neuron_forward_nograd(x, weight, y, group, q, truncate)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, weight, pos = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        want_x, want_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        grad_input = torch.empty_like(x)
+        grad_weight = None
+        if want_w:
+            grad_weight = torch.empty_like(weight)
+            _C.sort_neuron_backward_input_weight(grad_output, pos, grad_input, grad_weight, ctx.group, ctx.q,
+                                                 ctx.truncate)
+        elif want_x:
+            _C.sort_neuron_backward_input(grad_output, pos, grad_input, ctx.group, ctx.q, ctx.truncate)
+        return (grad_input if want_x else None), grad_weight, None, None, None, None, None
+
+
+class BoundInfDistF(torch.autograd.Function):
+    """Interval bounds through the l-inf layer, forward and backward.  Mirrors core/norm_dist.py:136-173."""
+
+    @staticmethod
+    def forward(ctx, x_lower, x_upper, weight, group, need_grad, tag):
+        assert x_lower.size() == x_upper.size()
+        assert weight.size(1) * group == x_lower.size(1)
+        y_lower = _new_out(x_lower, weight.size(0))
+        y_upper = torch.empty_like(y_lower)
+        ctx.group, ctx.tag = group, tag
+        if need_grad:
+            pos_lower = torch.empty_like(y_lower, dtype=torch.int)
+            pos_upper = torch.empty_like(pos_lower)
+            _C.bound_inf_dist_forward(x_lower, x_upper, weight, y_lower, y_upper, pos_lower, pos_upper, group)
+            ctx.save_for_backward(x_lower, x_upper, weight, pos_lower, pos_upper)
+        else:
+            _C.bound_inf_dist_forward_nograd(x_lower, x_upper, weight, y_lower, y_upper, group)
+        return y_lower, y_upper
+
+    @staticmethod
+    def backward(ctx, grad_y_lower, grad_y_upper):
+        grad_y_lower = grad_y_lower.contiguous()
+        grad_y_upper = grad_y_upper.contiguous()
+        x_lower, x_upper, weight, pos_lower, pos_upper = ctx.saved_tensors
+        want_l, want_u, want_w = ctx.needs_input_grad[:3]
+        grad_x_lower = torch.zeros_like(x_lower)
+        grad_x_upper = torch.zeros_like(x_upper)
+        grad_weight = None
+        if want_w:
+            grad_weight = torch.zeros_like(weight)
+            _C.bound_inf_dist_backward_input_weight(grad_y_lower, grad_y_upper, pos_lower, pos_upper,
+                                                    grad_x_lower, grad_x_upper, grad_weight, ctx.group)
+        elif want_l and want_u:
+            _C.bound_inf_dist_backward_input(grad_y_lower, grad_y_upper, pos_lower, pos_upper,
+                                             grad_x_lower, grad_x_upper, ctx.group)
+        return (grad_x_lower if want_l else None), (grad_x_upper if want_u else None), grad_weight, None, None, None
+
+
+class MaskedInfDistF(torch.autograd.Function):
+    """SortNet's training neuron as one fused op: max over a Bernoulli(q)-kept subset of |x - w|,
+    the keep decisions drawn on the GPU from a stateless counter RNG of (seed, b, m, n).
+    The reference builds the same kind of subset on the host (core/models/norm_dist.py:14-17) and
+    feeds index lists to NormDistDropoutF; the backward here is the l-inf scatter through the
+    saved arg-max index, identical to NormDistF's (core/norm_dist.py:29-39)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, group, q, seed, mode, need_grad, tag):
+        assert weight.size(1) * group == x.size(1)
+        y = _new_out(x, weight.size(0))
+        ctx.group, ctx.tag = group, tag
+        if need_grad:
+            pos = torch.empty_like(y, dtype=torch.int)
+            _C.masked_inf_dist_forward(x, weight, y, pos, group, q, seed, mode)
+            ctx.save_for_backward(x, weight, pos)
+        else:
+            _C.masked_inf_dist_forward(x, weight, y, None, group, q, seed, mode)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, weight, pos = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        want_x, want_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        grad_input = torch.empty_like(x)
+        grad_weight = None
+        if want_w:
+            grad_weight = torch.empty_like(weight)
+            _C.inf_dist_backward_input_weight(grad_output, pos, grad_input, grad_weight, ctx.group)
+        elif want_x:
+            _C.inf_dist_backward_input(grad_output, pos, grad_input, ctx.group)
+        return (grad_input if want_x else None), grad_weight, None, None, None, None, None, None
+
+
+def norm_dist(input, weight, p, groups=1, use_custom_cuda_func=True, tag=None):
+    """core/norm_dist.py:176-186."""
+    _no_fallback(use_custom_cuda_func, "norm_dist")
+    return NormDistF.apply(input, weight, groups, p, _want_grad(input, weight), tag)
+
+
+def norm_dist_dropout(input, weight, w_index_ci, w_index_co, p, groups=1, use_custom_cuda_func=True, tag=None):
+    """core/norm_dist.py:191-214.  `input` is already compacted to the kept channels; `weight` is the
+    full tensor; the same index list serves the 32 samples of a sub-batch."""
+    _no_fallback(use_custom_cuda_func, "norm_dist_dropout")
+    return NormDistDropoutF.apply(input, weight, w_index_ci, w_index_co, groups, p, tag)
+
+
+def sort_neuron(input, weight, groups=1, q=0.5, truncate=10, use_custom_cuda_func=True, tag=None):
+    """core/norm_dist.py:217-231."""
+    truncate = min(weight.size(-1), truncate)
+    if q is None or q == 1.0 or truncate == 1:
+        return norm_dist(input, weight, float("inf"), groups, tag=tag)
+    _no_fallback(use_custom_cuda_func, "sort_neuron")
+    return SortNeuronF.apply(input, weight, groups, q, truncate, _want_grad(input, weight), tag)
+
+
+def bound_sort_neuron(x_lower, x_upper, weight, groups=1, q=0.5, truncate=10, tag=None):
+    """core/norm_dist.py:234-243.  Forward only, as in the reference."""
+    truncate = min(weight.size(-1), truncate)
+    if q is None or q == 1.0 or truncate == 1:
+        return bound_inf_dist(x_lower, x_upper, weight, groups, tag=tag)
+    assert not _want_grad(x_lower, x_upper, weight)
+    y_lower = _new_out(x_lower, weight.size(0))
+    y_upper = torch.empty_like(y_lower)
+    _C.bound_sort_neuron_forward(x_lower, x_upper, weight, y_lower, y_upper, groups, q, truncate)
+    return y_lower, y_upper
+
+
+def bound_inf_dist(x_lower, x_upper, weight, groups=1, use_custom_cuda_func=True, tag=None):
+    """core/norm_dist.py:246-260."""
+    _no_fallback(use_custom_cuda_func, "bound_inf_dist")
+    return BoundInfDistF.apply(x_lower, x_upper, weight, groups, _want_grad(x_lower, x_upper, weight), tag)
+
+
+def masked_inf_dist(input, weight, q, seed, groups=1, mode=_C.MASK_TERM, tag=None):
+    """Masked order-statistic neuron (see MaskedInfDistF).  `mode` is ext.MASK_TERM (independent
+    draw per term) or ext.MASK_FACTORED (keep = keep_x(b, n) & keep_w(m, n))."""
+    if q is None or q == 1.0:
+        return norm_dist(input, weight, float("inf"), groups, tag=tag)
+    return MaskedInfDistF.apply(input, weight, groups, q, seed, mode, _want_grad(input, weight), tag)
