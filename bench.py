@@ -1,0 +1,197 @@
+#!/usr/bin/env python3
+"""Benchmark of the distance-neuron hot path on one MI355X.
+
+A step is one training pass of the 5x5120 SortNet-MLP on a batch of 512 synthetic CIFAR-shaped
+inputs (3072 features in [0,1], 10 classes): forward through the distance layers (l-inf on the
+first layer, masked order-statistic neuron with q = 0.3 on the others) with mean shift, hinge
+loss on the 1-Lipschitz margin, backward through every layer (grad_input and grad_weight),
+AdamW update, and the interval-bound (certification) pass with eps = 8/255 through all layers.
+Prints one JSON line; see --help for the knobs.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+FP32_VECTOR_PEAK_TFLOPS = 157.3     # MI355X published fp32 vector peak (packed FMA)
+VALU_LANE_RATE = 39.32e12           # 256 CUs x 4 SIMD x 16 lanes x 2.4 GHz lane-instructions/s
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=512)
+    ap.add_argument("--width", type=int, default=5120)
+    ap.add_argument("--depth", type=int, default=6, help="distance layers incl. the class layer (reference: depth=6)")
+    ap.add_argument("--in-features", type=int, default=3072)
+    ap.add_argument("--classes", type=int, default=10)
+    ap.add_argument("--q", type=float, default=0.3)
+    ap.add_argument("--eps", type=float, default=8.0 / 255)
+    ap.add_argument("--mask", choices=["term", "factored"], default="term")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-batch", type=int, default=0, help="samples of the CPU baseline (0 = pick for ~15 s)")
+    return ap.parse_args()
+
+
+def cpu_baseline(args, model_dims):
+    """The CPU oracle timed on this host's cores on a bounded sample of the same step:
+    `nb` samples through forward (+positions), scatter backward and interval bounds of every layer."""
+    import numpy as np
+    import oracle
+    oracle.build()
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    oracle.set_num_threads(cores)
+    rng = np.random.default_rng(0)
+    ws = [(rng.standard_normal((o, i)) * i ** -0.5).astype(np.float32) for i, o in zip(model_dims[:-1], model_dims[1:])]
+
+    def run(nb):
+        x = rng.random((nb, model_dims[0], 1), dtype=np.float32)
+        lo, up = np.maximum(x - np.float32(args.eps), 0), np.minimum(x + np.float32(args.eps), 1)
+        t0 = time.perf_counter()
+        h, saved = x, []
+        for li, w in enumerate(ws):
+            if li == 0 or args.q >= 1.0:
+                y, pos = oracle.inf_dist_forward(h, w)
+            else:
+                y, pos = oracle.masked_inf_dist_forward(h, w, args.q, li, oracle.MASK_TERM if args.mask == "term" else oracle.MASK_FACTORED)
+            saved.append((h.shape, pos))
+            h = y - y.mean(axis=(0, 2), keepdims=True) if li < len(ws) - 1 else y
+        g = np.ones_like(h)
+        for li in reversed(range(len(ws))):
+            g, _ = oracle.inf_dist_backward(g, saved[li][1], saved[li][0], ws[li].shape)
+        for li, w in enumerate(ws):
+            lo, up = oracle.bound_inf_dist_forward(lo, up, w, need_pos=False)
+        return time.perf_counter() - t0
+
+    nb = args.cpu_batch
+    if nb <= 0:
+        t = run(2)
+        nb = int(max(2, min(args.batch, 15.0 / max(t / 2, 1e-6))))
+    t = run(nb)
+    return {"value": nb / t, "unit": "samples/s", "cores": cores, "kind": "port",
+            "sample": "%d samples through the same step (oracle forward+positions, scatter backward, interval "
+                      "bounds of all %d layers; no optimizer), %.1f s" % (nb, len(ws), t)}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (no collective path exists); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from sortnet_amd import ext
+    from sortnet_amd.model import DistanceMLP, margins, hinge_loss
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    mode = ext.MASK_TERM if args.mask == "term" else ext.MASK_FACTORED
+    model = DistanceMLP(args.in_features, args.width, args.depth, args.classes, q=args.q, device=dev, seed=0,
+                        mask_mode=mode)
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-4, fused=True)
+    g = torch.Generator().manual_seed(0)
+    x = torch.rand(args.batch, args.in_features, generator=g).to(dev)
+    targets = torch.randint(0, args.classes, (args.batch,), generator=g).to(dev)
+    lower, upper = (x - args.eps).clamp(min=0), (x + args.eps).clamp(max=1)
+
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    phase_ms = {"forward": 0.0, "backward": 0.0, "optimizer": 0.0, "bounds": 0.0}
+    ibp_events = []
+
+    def step(i, timed):
+        marks = [ev() for _ in range(5)]
+        marks[0].record()
+        dist = model.forward(x, step_seed=i)
+        logits, worst = margins(dist, targets, args.eps)
+        loss = hinge_loss(worst)
+        marks[1].record()
+        opt.zero_grad(set_to_none=True)
+        loss.backward()
+        marks[2].record()
+        opt.step()
+        marks[3].record()
+        if timed:
+            # per-launch timing of the dominant kernel: the interval-bound forward of a width x width layer
+            lo, up = lower.unsqueeze(-1).contiguous(), upper.unsqueeze(-1).contiguous()
+            with torch.no_grad():
+                for li, w in enumerate(model.weights):
+                    ylo = torch.empty(lo.size(0), w.size(0), 1, device=dev)
+                    yup = torch.empty_like(ylo)
+                    e0, e1 = ev(), ev()
+                    e0.record()
+                    ext.bound_inf_dist_forward_nograd(lo, up, w, ylo, yup, 1)
+                    e1.record()
+                    if w.size(0) == args.width and w.size(1) == args.width:
+                        ibp_events.append((e0, e1))
+                    shift = (model.running_mean[li].view(1, -1, 1) if li < model.num_layers - 1
+                             else -model.bias.view(1, -1, 1))
+                    lo, up = ylo - shift, yup - shift
+                cert = margins(dist.detach(), targets, args.eps, lo.squeeze(-1), up.squeeze(-1))[1]
+        else:
+            lo, up = model.bounds(lower, upper)
+            cert = margins(dist.detach(), targets, args.eps, lo, up)[1]
+        marks[4].record()
+        return marks, loss, cert
+
+    for i in range(args.warmup):
+        step(i, False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    all_marks = []
+    for i in range(args.steps):
+        marks, loss, cert = step(args.warmup + i, True)
+        all_marks.append(marks)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    for marks in all_marks:
+        for k, (a, b) in zip(phase_ms, zip(marks[:-1], marks[1:])):
+            phase_ms[k] += a.elapsed_time(b) / args.steps
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = args.batch / (elapsed / args.steps)
+
+    terms = model.terms_per_sample() * args.batch
+    step_flops = terms * (2 + 6)                      # forward 2 flops/term, interval bounds 6 flops/term
+    layer_terms = args.batch * args.width * args.width
+    ibp_ms = sum(a.elapsed_time(b) for a, b in ibp_events) / max(len(ibp_events), 1)
+    achieved = 6.0 * layer_terms / (ibp_ms * 1e-3) / 1e12 if ibp_events else None
+    roofline = {
+        "bound": "valu", "kernel": "fwd_kernel<BoundNograd,4,8> (interval bounds, %dx%dx%d)" % (args.batch, args.width, args.width),
+        "achieved": achieved, "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": achieved / FP32_VECTOR_PEAK_TFLOPS if achieved else None, "traffic": None,
+        "avg_launch_ms": ibp_ms, "launches_timed": len(ibp_events),
+        "valu_issue_frac": 4.0 * layer_terms / (ibp_ms * 1e-3) / VALU_LANE_RATE if ibp_events else None,
+        "note": "tropical (sub/min/max) contraction on the fp32 vector ALUs, not MFMA; peak is the packed-FMA "
+                "fp32 vector figure, of which this instruction mix can reach at most 37.5% (6 flops in 4 issue slots)",
+    }
+    out = {
+        "metric": "train samples/s (fwd+bwd+IBP) 5x5120 SortNet-MLP, B=512; % FP32 VALU peak",
+        "value": value, "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "SortNet-MLP training step: %d->%s->%d distance layers, B=%d, q=%.2f (%s mask), "
+                               "forward+hinge loss+backward+AdamW+interval bounds eps=%.4f"
+                               % (args.in_features, "x".join([str(args.width)] * (args.depth - 1)), args.classes,
+                                  args.batch, args.q, args.mask, args.eps),
+                   "batch": args.batch, "width": args.width, "distance_layers": args.depth, "mask": args.mask},
+        "step_fp32_vector_frac": step_flops / (elapsed / args.steps) / (FP32_VECTOR_PEAK_TFLOPS * 1e12),
+        "phase_ms": phase_ms,
+        "roofline": roofline,
+        "loss": float(loss), "certified_frac": float((cert.max(dim=1)[0] < 0).float().mean()),
+    }
+    dims = [args.in_features] + [args.width] * (args.depth - 1) + [args.classes]
+    out["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args, dims)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

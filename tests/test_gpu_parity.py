@@ -368,7 +368,7 @@ def test_argument_errors():
     with pytest.raises(RuntimeError, match="CUDA tensor"):
         ext.inf_dist_forward_nograd(x.cpu(), w, y, 1)
     with pytest.raises(RuntimeError, match="contiguous"):
-        ext.inf_dist_forward_nograd(x.expand(4, 8, 2)[:, :, :1], w, y, 1)
+        ext.inf_dist_forward_nograd(torch.rand(8, 4, 1, device=dev).transpose(0, 1), w, y, 1)
     with pytest.raises(RuntimeError, match="K="):
         ext.sort_neuron_forward_nograd(x, w, y, 1, 0.5, 40)
     with pytest.raises(RuntimeError, match="multiples of G"):
