@@ -39,6 +39,7 @@ struct FwdArgs {
     float* y1;            // upper output
     int* p0;              // pos / posL / sort pos (K, B, CO, HW)
     int* p1;              // posU
+    unsigned long long* packed0;  // (value bits << 32 | ~chunk) merge buffer of split-N position kernels
     const int* ci_idx;    // (S, G, CIg) or null
     const int* co_idx;    // (S, G, COg) or null
     int B, R, HW, G;      // R = B * HW rows of the batch tile
@@ -62,6 +63,10 @@ int check_launch(const char* what);
 
 // number of compute units of the current device (cached)
 int num_cus();
+
+// grow-only per-device scratch buffer owned by the library (split-N merge of position kernels).
+// Calls that use it must be ordered on one stream per device.
+void* workspace(size_t bytes);
 
 // zero-fill n floats on `stream` with a kernel (graph-capture friendly, no memset node)
 int fill_zero(void* ptr, size_t n_words, hipStream_t stream);

@@ -182,7 +182,7 @@ __global__ void __launch_bounds__(256) fwd_kernel(FwdArgs a) {
             #pragma unroll
             for (int i = 0; i < TB; i++) {
                 #pragma unroll
-                for (int j = 0; j < TM; j++) P::chunk_end(acc[i][j], a, pass);
+                for (int j = 0; j < TM; j++) P::chunk_end(acc[i][j], a, pass, k0);
             }
         }
         __syncthreads();
@@ -216,7 +216,7 @@ int launch_fwd(const FwdArgs& a, hipStream_t stream) {
 struct PolicyBase {
     static constexpr int NX = 1;
     static constexpr int PASSES = 1;
-    template <class A> static __device__ __forceinline__ void chunk_end(A&, const FwdArgs&, int) {}
+    template <class A> static __device__ __forceinline__ void chunk_end(A&, const FwdArgs&, int, int) {}
 };
 
 // l-inf forward without indices (core/cuda/inf_dist_cuda.cu:17-107)
@@ -255,6 +255,64 @@ struct LinfPos : PolicyBase {
         a.y0[o] = fabsf(A.bd);
         a.p0[o] = A.bn | (A.bd < 0.f ? (int)kSign : 0);
     }
+};
+
+// Same result as LinfPos at a fraction of the cost: inside a chunk of KT inputs only the maximum
+// is kept (one subtract per term, one 3-input max per two terms); at the end of the chunk the
+// running (best, chunk index) pair is replaced only on a strictly larger maximum, so the lowest
+// chunk attaining the final value survives.  The (best, chunk) pairs of the split-N slices are
+// merged with a 64-bit atomic max on (value bits << 32 | ~chunk) and resolve_pos_kernel then
+// rescans the one winning chunk of every output for the first input attaining the value.
+__device__ __forceinline__ void store_chunk_winner(const FwdArgs& a, size_t o, float best, int cid) {
+    if (a.nsplit > 1) {
+        if (cid >= 0) {
+            unsigned long long key = ((unsigned long long)__float_as_uint(best) << 32) |
+                                     (unsigned long long)(0xffffffffu - (uint32_t)cid);
+            atomicMax(a.packed0 + o, key);
+        }
+    } else { a.y0[o] = best; a.p0[o] = cid; }
+}
+
+struct LinfChunk : PolicyBase {
+    struct Acc { float best, cm; int cid; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.best = kEps; A.cm = 0.f; A.cid = -1; }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
+                                                 const float4& w, int, int) {
+        float v = A.cm;
+        v = fmaxf(fmaxf(v, fabsf(x.x - w.x)), fabsf(x.y - w.y));
+        v = fmaxf(fmaxf(v, fabsf(x.z - w.z)), fabsf(x.w - w.w));
+        A.cm = v;
+    }
+    static __device__ __forceinline__ void chunk_end(Acc& A, const FwdArgs&, int, int k0) {
+        if (A.cm > A.best) { A.best = A.cm; A.cid = k0 / KT; }
+        A.cm = 0.f;
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) { store_chunk_winner(a, o, A.best, A.cid); }
+};
+
+// the per-term masked neuron with the same chunk tracking
+struct MaskedTermChunk : PolicyBase {
+    struct Acc { float best, cm; int cid; uint32_t key; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool) {
+        A.best = kEps; A.cm = 0.f; A.cid = -1; A.key = rng_row_key(a.seed, 0u, (uint32_t)o);
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
+                                                 const float4& w, int n, int) {
+        uint32_t word = rng_word(A.key, (uint32_t)n >> 2);
+        float d0 = (word & 0xffu) < a.t8 ? x.x - w.x : 0.f;
+        float d1 = ((word >> 8) & 0xffu) < a.t8 ? x.y - w.y : 0.f;
+        float d2 = ((word >> 16) & 0xffu) < a.t8 ? x.z - w.z : 0.f;
+        float d3 = (word >> 24) < a.t8 ? x.w - w.w : 0.f;
+        float v = A.cm;
+        v = fmaxf(fmaxf(v, fabsf(d0)), fabsf(d1));
+        v = fmaxf(fmaxf(v, fabsf(d2)), fabsf(d3));
+        A.cm = v;
+    }
+    static __device__ __forceinline__ void chunk_end(Acc& A, const FwdArgs&, int, int k0) {
+        if (A.cm > A.best) { A.best = A.cm; A.cid = k0 / KT; }
+        A.cm = 0.f;
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) { store_chunk_winner(a, o, A.best, A.cid); }
 };
 
 // masked neuron, independent draw per term: byte (n & 3) of word(key(output), n >> 2) < t8 keeps
@@ -488,7 +546,7 @@ struct LpOnline : PolicyBase {
             A.s += pow_pos<IP>(fabsf(x.w - w.w) * A.rinv, a.p);
         }
     }
-    static __device__ __forceinline__ void chunk_end(Acc& A, const FwdArgs& a, int pass) {
+    static __device__ __forceinline__ void chunk_end(Acc& A, const FwdArgs& a, int pass, int) {
         if (pass == 0) {
             if (A.cm > A.M) {
                 A.s *= __builtin_amdgcn_exp2f(a.p * __builtin_amdgcn_logf(A.M / A.cm));
@@ -522,5 +580,62 @@ struct LpWithMax : PolicyBase {
         a.y0[o] = powf(A.s, a.inv_p) / A.rinv;
     }
 };
+
+
+// -------------------------------------------------------------------------------------------
+// resolve_pos_kernel: one work-item per output.  Reads the winning (value, chunk) pair left by a
+// chunk-tracking policy (from y/pos when the reduction was not split, else from the packed
+// workspace), rescans that chunk in ascending input order for the first kept term whose
+// magnitude equals the value bit for bit, and writes the final value and position.
+// -------------------------------------------------------------------------------------------
+template <bool PACKED>
+__global__ void __launch_bounds__(256) resolve_pos_kernel(FwdArgs a) {
+    long long total = (long long)a.R * a.G * a.COg;
+    long long o = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (o >= total) return;
+    int hw = (int)(o % a.HW);
+    long long t = o / a.HW;
+    int c = (int)(t % (a.G * a.COg));
+    int b = (int)(t / (a.G * a.COg));
+    int g = c / a.COg, m = c - g * a.COg;
+    float best; int cid;
+    if (PACKED) {
+        unsigned long long v = a.packed0[o];
+        uint32_t low = (uint32_t)v;
+        best = low ? __uint_as_float((uint32_t)(v >> 32)) : kEps;
+        cid = low ? (int)(0xffffffffu - low) : -1;
+    } else { best = a.y0[o]; cid = a.p0[o]; }
+    int pos = 0;
+    if (cid >= 0) {
+        const int s = b / kSubBatch;
+        const int wrow = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + m] : m;
+        const float* wr = a.w + (size_t)(g * a.W_COg + wrow) * a.W_CIg;
+        const float* xr = a.x0 + ((size_t)(b * a.G + g) * a.CIg) * a.HW + hw;
+        const int* cidx = a.ci_idx ? a.ci_idx + (size_t)(s * a.G + g) * a.CIg : nullptr;
+        const uint32_t key_t = rng_row_key(a.seed, 0u, (uint32_t)o);
+        const uint32_t key_x = rng_row_key(a.seed, 1u, (uint32_t)((b * a.G + g) * a.HW + hw));
+        const uint32_t key_w = rng_row_key(a.seed, 2u, (uint32_t)c);
+        int n0 = cid * KT, n1 = n0 + KT < a.CIg ? n0 + KT : a.CIg;
+        for (int n = n0; n < n1; n++) {
+            bool keep = true;
+            if (a.mask_mode == SD_MASK_TERM)
+                keep = ((rng_word(key_t, (uint32_t)n >> 2) >> (8 * (n & 3))) & 0xffu) < a.t8;
+            else if (a.mask_mode == SD_MASK_FACTORED)
+                keep = (rng_word(key_x, (uint32_t)n) >> 16) < a.t16 && (rng_word(key_w, (uint32_t)n) >> 16) < a.t16;
+            float d = xr[(size_t)n * a.HW] - wr[cidx ? cidx[n] : n];
+            if (keep && fabsf(d) == best) { pos = n | (d < 0.f ? (int)kSign : 0); break; }
+        }
+    }
+    a.y0[o] = best;
+    a.p0[o] = pos;
+}
+
+inline int launch_resolve(const FwdArgs& a, hipStream_t stream) {
+    long long total = (long long)a.R * a.G * a.COg;
+    dim3 grid((unsigned)((total + 255) / 256));
+    if (a.nsplit > 1) hipLaunchKernelGGL((resolve_pos_kernel<true>), grid, dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL((resolve_pos_kernel<false>), grid, dim3(256), 0, stream, a);
+    return check_launch("resolve_pos_kernel");
+}
 
 }  // namespace sd

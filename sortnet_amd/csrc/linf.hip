@@ -4,6 +4,25 @@
 
 using namespace sd;
 
+// forward with positions: chunk-tracking kernel (split-N through the packed workspace when the
+// grid would otherwise be too small) followed by the position resolve pass
+template <class P>
+static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st) {
+    // with index lists a batch tile must stay inside one 32-sample sub-batch
+    const int TB = (index_lists || a.R <= 32) ? 2 : 4;
+    a.nsplit = pick_nsplit(a, 16 * TB, 128);
+    int rc;
+    if (a.nsplit > 1) {
+        size_t n = (size_t)a.R * a.G * a.COg;
+        a.packed0 = static_cast<unsigned long long*>(workspace(n * 8));
+        if (!a.packed0) return SD_ERR_HIP;
+        if ((rc = fill_zero(a.packed0, n * 2, st))) return rc;
+    }
+    rc = TB == 2 ? launch_fwd<P, 2, 8>(a, st) : launch_fwd<P, 4, 8>(a, st);
+    if (rc) return rc;
+    return launch_resolve(a, st);
+}
+
 extern "C" int sd_inf_dist_forward_nograd(const float* input, const float* weight,
                                           int B, int CO, int CI, int G, int HW, float* output, sd_stream_t stream) {
     FwdArgs a;
@@ -31,9 +50,7 @@ extern "C" int sd_inf_dist_forward(const float* input, const float* weight,
     SD_REQUIRE(output && pos, "inf_dist_forward: null output or pos");
     a.y0 = output; a.p0 = pos;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // with index lists a batch tile must stay inside one 32-sample sub-batch
-    if (w_index_ci || w_index_co || a.R <= 32) return launch_fwd<LinfPos, 2, 8>(a, st);
-    return launch_fwd<LinfPos, 4, 8>(a, st);
+    return run_chunk_pos<LinfChunk>(a, w_index_ci || w_index_co, st);
 }
 
 extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weight,
@@ -51,12 +68,12 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = a.R <= 32;
     if (mode == SD_MASK_TERM) {
-        if (pos) return small ? launch_fwd<MaskedTerm<true>, 2, 8>(a, st) : launch_fwd<MaskedTerm<true>, 4, 8>(a, st);
+        if (pos) return run_chunk_pos<MaskedTermChunk>(a, false, st);
         return small ? launch_fwd<MaskedTerm<false>, 2, 8>(a, st) : launch_fwd<MaskedTerm<false>, 4, 8>(a, st);
     }
     // factored mask: dropped inputs / weights are replaced by NaN while staging the tiles and
     // NaN terms never win the maximum, so the plain l-inf policies apply unchanged
-    if (pos) return small ? launch_fwd<LinfPos, 2, 8>(a, st) : launch_fwd<LinfPos, 4, 8>(a, st);
+    if (pos) return run_chunk_pos<LinfChunk>(a, false, st);
     const int TB = a.R <= 32 ? 2 : a.R <= 64 ? 4 : 8;
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;

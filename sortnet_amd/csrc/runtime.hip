@@ -34,6 +34,22 @@ int num_cus() {
     return cached[dev];
 }
 
+void* workspace(size_t bytes) {
+    static void* buf[64] = {nullptr};
+    static size_t cap[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { set_error("workspace: no current device"); return nullptr; }
+    if (cap[dev] < bytes) {
+        // the old buffer may still be in use by queued kernels: release it only after the device is idle
+        if (buf[dev]) { (void)hipDeviceSynchronize(); (void)hipFree(buf[dev]); buf[dev] = nullptr; cap[dev] = 0; }
+        size_t want = bytes + bytes / 4;
+        void* p = nullptr;
+        if (hipMalloc(&p, want) != hipSuccess) { (void)hipGetLastError(); set_error("workspace: hipMalloc of %zu bytes failed", want); return nullptr; }
+        buf[dev] = p; cap[dev] = want;
+    }
+    return buf[dev];
+}
+
 __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t* __restrict__ p, size_t n) {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     size_t stride = (size_t)gridDim.x * 256;
