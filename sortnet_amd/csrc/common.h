@@ -40,6 +40,8 @@ struct FwdArgs {
     int* p0;              // pos / posL / sort pos (K, B, CO, HW)
     int* p1;              // posU
     unsigned long long* packed0;  // (value bits << 32 | ~chunk) merge buffer of split-N position kernels
+    const uint32_t* xmask;  // factored mask: keep bits of x rows, one word per (row, chunk), or null
+    const uint32_t* wmask;  // same for w rows
     const int* ci_idx;    // (S, G, CIg) or null
     const int* co_idx;    // (S, G, COg) or null
     int B, R, HW, G;      // R = B * HW rows of the batch tile

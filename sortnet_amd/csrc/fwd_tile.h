@@ -12,7 +12,18 @@
 // still fill 256 compute units.
 #pragma once
 #include <float.h>
+#include <stdlib.h>
 #include "common.h"
+
+#ifndef SD_MINW
+#define SD_MINW 3
+#endif
+#ifndef SD_UNR
+#define SD_UNR 1
+#endif
+#ifndef SD_PIPEW
+#define SD_PIPEW 3
+#endif
 
 namespace sd {
 
@@ -133,7 +144,7 @@ __device__ __forceinline__ void load_w_tile(float (*ws)[LDP], const FwdArgs& a,
 // the kernel
 // -------------------------------------------------------------------------------------------
 template <class P, int TB, int TM>
-__global__ void __launch_bounds__(256) fwd_kernel(FwdArgs a) {
+__global__ void __launch_bounds__(256, P::MIN_WAVES) fwd_kernel(FwdArgs a) {
     constexpr int BB = 16 * TB, BM = 16 * TM, NX = P::NX;
     __shared__ __attribute__((aligned(16))) float xs[NX][BB][LDP];
     __shared__ __attribute__((aligned(16))) float ws[BM][LDP];
@@ -166,15 +177,20 @@ __global__ void __launch_bounds__(256) fwd_kernel(FwdArgs a) {
         __syncthreads();
         #pragma unroll
         for (int pass = 0; pass < P::PASSES; pass++) {
-            #pragma unroll 2
+            #pragma unroll P::UNROLL4
             for (int n4 = 0; n4 < KT; n4 += 4) {
                 float4 wv[TM];
+#ifdef SD_EXP_NOLDS
+                const int n4l = 0;
+#else
+                const int n4l = n4;
+#endif
                 #pragma unroll
-                for (int j = 0; j < TM; j++) wv[j] = *reinterpret_cast<const float4*>(&ws[tm + 16 * j][n4]);
+                for (int j = 0; j < TM; j++) wv[j] = *reinterpret_cast<const float4*>(&ws[tm + 16 * j][n4l]);
                 #pragma unroll
                 for (int i = 0; i < TB; i++) {
-                    float4 xl = *reinterpret_cast<const float4*>(&xs[0][tb + 16 * i][n4]);
-                    float4 xu = (NX == 2) ? *reinterpret_cast<const float4*>(&xs[NX - 1][tb + 16 * i][n4]) : xl;
+                    float4 xl = *reinterpret_cast<const float4*>(&xs[0][tb + 16 * i][n4l]);
+                    float4 xu = (NX == 2) ? *reinterpret_cast<const float4*>(&xs[NX - 1][tb + 16 * i][n4l]) : xl;
                     #pragma unroll
                     for (int j = 0; j < TM; j++) P::step4(acc[i][j], a, xl, xu, wv[j], k0 + n4, pass);
                 }
@@ -202,11 +218,191 @@ __global__ void __launch_bounds__(256) fwd_kernel(FwdArgs a) {
     }
 }
 
+// -------------------------------------------------------------------------------------------
+// Pipelined variant for the vector-load case (HW == 1, reduction length a multiple of 4, no input
+// index list).  The global loads of chunk k+1 are issued into registers, branch-free, right after
+// chunk k has been published in LDS, and are written to LDS once chunk k has been consumed, so
+// HBM/L2 latency hides behind the VALU work of the same workgroup.  One LDS buffer keeps four
+// workgroups resident per compute unit: the fp32 vector ALUs only reach their full rate when at
+// least two wavefronts per SIMD have VALU work ready.
+// In the factored mask mode the keep bits come from bit-mask words built by build_masks_kernel
+// (one 32-bit word per row and chunk).
+// -------------------------------------------------------------------------------------------
+template <class P, int TB, int TM>
+__global__ void __launch_bounds__(256, P::PIPE_WAVES) fwd_kernel_pipe(FwdArgs a) {
+    constexpr int BB = 16 * TB, BM = 16 * TM, NX = P::NX;
+    constexpr int NXV = (BB * 8 + 255) / 256, NWV = (BM * 8 + 255) / 256;
+    __shared__ __attribute__((aligned(16))) float xs[NX][BB][LDP];
+    __shared__ __attribute__((aligned(16))) float ws[BM][LDP];
+
+    const int tid = threadIdx.x, tm = tid & 15, tb = tid >> 4;
+    const int g = blockIdx.z % a.G, split = blockIdx.z / a.G;
+    const int r0 = blockIdx.y * BB, m0 = blockIdx.x * BM;
+    const int s = r0 / kSubBatch;
+    const bool masked = (NX == 1) && a.mask_mode == SD_MASK_FACTORED;
+
+    const int nchunks = (a.CIg + KT - 1) / KT;
+    const int n_begin = (int)((long long)split * nchunks / a.nsplit) * KT;
+    int n_end = (int)((long long)(split + 1) * nchunks / a.nsplit) * KT;
+    if (n_end > a.CIg) n_end = a.CIg;
+
+    // staging slot v of a work-item: float4 number v * 256 + tid of a tile = row (tid >> 3) + 32 v,
+    // columns (tid & 7) * 4 .. +3.  Rows outside the tensor read row 0 of the tile's first valid
+    // row instead (always a legal address) and are zeroed afterwards.
+    const int lrow = tid >> 3, lc4 = (tid & 7) * 4;
+    // 32-bit element offsets of the rows this work-item stages (pointers would cost twice the registers)
+    int xoff[NXV], woff[NWV], xmoff[NXV], wmoff[NWV];
+    uint32_t okbits = 0;   // bit v: x row v valid, bit 8 + v: w row v valid
+    #pragma unroll
+    for (int v = 0; v < NXV; v++) {
+        int row = lrow + 32 * v, r = r0 + row;
+        bool ok = row < BB && r < a.R;
+        int rr = ok ? r : r0;
+        okbits |= ok ? 1u << v : 0u;
+        xoff[v] = (rr * a.G + g) * a.CIg;
+        xmoff[v] = masked ? (rr * a.G + g) * nchunks : 0;
+    }
+    #pragma unroll
+    for (int v = 0; v < NWV; v++) {
+        int row = lrow + 32 * v, m = m0 + row;
+        bool ok = row < BM && m < a.COg;
+        int mm = ok ? m : m0;
+        okbits |= ok ? 1u << (8 + v) : 0u;
+        int wrow = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + mm] : mm;
+        woff[v] = (g * a.W_COg + wrow) * a.W_CIg;
+        wmoff[v] = masked ? (g * a.COg + mm) * nchunks : 0;
+    }
+    // unmasked: the mask pointers alias x and word 0 is read and ignored
+    const uint32_t* xmbase = masked ? a.xmask : reinterpret_cast<const uint32_t*>(a.x0);
+    const uint32_t* wmbase = masked ? a.wmask : reinterpret_cast<const uint32_t*>(a.x0);
+    const int mstep = masked ? 1 : 0;
+
+    float4 px0[NXV], px1[NXV], pw[NWV];
+    uint32_t mx[NXV], mw[NWV];
+
+    auto gload = [&](int k0) {
+        int n = k0 + lc4;
+        if (n > a.CIg - 4) n = a.CIg - 4;     // keeps the address inside the row; zeroed in sstore()
+        #pragma unroll
+        for (int v = 0; v < NXV; v++) {
+            px0[v] = *reinterpret_cast<const float4*>(a.x0 + xoff[v] + n);
+            if (NX == 2) px1[v] = *reinterpret_cast<const float4*>(a.x1 + xoff[v] + n);
+            if (NX == 1) mx[v] = xmbase[xmoff[v] + (k0 / KT) * mstep];
+        }
+        #pragma unroll
+        for (int v = 0; v < NWV; v++) {
+            pw[v] = *reinterpret_cast<const float4*>(a.w + woff[v] + n);
+            if (NX == 1) mw[v] = wmbase[wmoff[v] + (k0 / KT) * mstep];
+        }
+    };
+    auto fix = [&](float4& v, bool ok, uint32_t bits) {
+        const float qnan = __builtin_nanf("");
+        if (NX == 1) {
+            bits = masked ? bits >> lc4 : 0xfu;
+            v.x = (bits & 1u) ? v.x : qnan; v.y = (bits & 2u) ? v.y : qnan;
+            v.z = (bits & 4u) ? v.z : qnan; v.w = (bits & 8u) ? v.w : qnan;
+        }
+        v.x = ok ? v.x : 0.f; v.y = ok ? v.y : 0.f; v.z = ok ? v.z : 0.f; v.w = ok ? v.w : 0.f;
+    };
+    // writes the staged chunk k0 to LDS (zeroing what lies outside the tensor / the slice)
+    auto sstore = [&](int k0) {
+        const bool in = k0 + lc4 < n_end;
+        #pragma unroll
+        for (int v = 0; v < NXV; v++) {
+            int row = lrow + 32 * v;
+            float4 l = px0[v], u = px1[v];
+            if (NX == 2) {
+                if (l.x > u.x) l.x = u.x = (l.x + u.x) * 0.5f;
+                if (l.y > u.y) l.y = u.y = (l.y + u.y) * 0.5f;
+                if (l.z > u.z) l.z = u.z = (l.z + u.z) * 0.5f;
+                if (l.w > u.w) l.w = u.w = (l.w + u.w) * 0.5f;
+                fix(u, ((okbits >> v) & 1u) && in, 0u);
+            }
+            fix(l, ((okbits >> v) & 1u) && in, NX == 1 ? mx[v] : 0u);
+            if (NXV * 32 == BB || row < BB) {
+                *reinterpret_cast<float4*>(&xs[0][row][lc4]) = l;
+                if (NX == 2) *reinterpret_cast<float4*>(&xs[NX - 1][row][lc4]) = u;
+            }
+        }
+        #pragma unroll
+        for (int v = 0; v < NWV; v++) {
+            int row = lrow + 32 * v;
+            float4 t = pw[v];
+            fix(t, ((okbits >> (8 + v)) & 1u) && in, NX == 1 ? mw[v] : 0u);
+            if (NWV * 32 == BM || row < BM) *reinterpret_cast<float4*>(&ws[row][lc4]) = t;
+        }
+    };
+
+    typename P::Acc acc[TB][TM];
+    #pragma unroll
+    for (int i = 0; i < TB; i++) {
+        #pragma unroll
+        for (int j = 0; j < TM; j++) {
+            int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
+            size_t o = (size_t)(r * a.G + g) * a.COg + m;
+            P::init(acc[i][j], a, o, r < a.R && m < a.COg);
+        }
+    }
+
+    if (n_begin < n_end) gload(n_begin);
+#if defined(SD_EXP1) || defined(SD_EXP2)
+    sstore(n_begin);
+    __syncthreads();
+#endif
+    for (int k0 = n_begin; k0 < n_end; k0 += KT) {
+#if defined(SD_EXP1)
+        __syncthreads();
+#elif defined(SD_EXP2)
+#else
+        sstore(k0);
+        __syncthreads();
+        if (k0 + KT < n_end) gload(k0 + KT);
+#endif
+        #pragma unroll
+        for (int pass = 0; pass < P::PASSES; pass++) {
+            #pragma unroll P::UNROLL4
+            for (int n4 = 0; n4 < KT; n4 += 4) {
+                float4 wv[TM];
+                #pragma unroll
+                for (int j = 0; j < TM; j++) wv[j] = *reinterpret_cast<const float4*>(&ws[tm + 16 * j][n4]);
+                #pragma unroll
+                for (int i = 0; i < TB; i++) {
+                    float4 xl = *reinterpret_cast<const float4*>(&xs[0][tb + 16 * i][n4]);
+                    float4 xu = (NX == 2) ? *reinterpret_cast<const float4*>(&xs[NX - 1][tb + 16 * i][n4]) : xl;
+                    #pragma unroll
+                    for (int j = 0; j < TM; j++) P::step4(acc[i][j], a, xl, xu, wv[j], k0 + n4, pass);
+                }
+            }
+            #pragma unroll
+            for (int i = 0; i < TB; i++) {
+                #pragma unroll
+                for (int j = 0; j < TM; j++) P::chunk_end(acc[i][j], a, pass, k0);
+            }
+        }
+#if !defined(SD_EXP2)
+        __syncthreads();
+#endif
+    }
+
+    #pragma unroll
+    for (int i = 0; i < TB; i++) {
+        #pragma unroll
+        for (int j = 0; j < TM; j++) {
+            int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
+            if (r < a.R && m < a.COg) P::store(acc[i][j], a, (size_t)(r * a.G + g) * a.COg + m);
+        }
+    }
+}
+
 // host-side launcher; the caller has validated shapes
 template <class P, int TB, int TM>
 int launch_fwd(const FwdArgs& a, hipStream_t stream) {
     dim3 grid((a.COg + 16 * TM - 1) / (16 * TM), (a.R + 16 * TB - 1) / (16 * TB), a.G * a.nsplit);
-    hipLaunchKernelGGL((fwd_kernel<P, TB, TM>), grid, dim3(256), 0, stream, a);
+    static const bool use_pipe = !getenv("SD_FWD_PIPE") || atoi(getenv("SD_FWD_PIPE")) != 0;
+    if (use_pipe && a.fast_x && a.fast_w && (a.mask_mode != SD_MASK_FACTORED || a.xmask))
+        hipLaunchKernelGGL((fwd_kernel_pipe<P, TB, TM>), grid, dim3(256), 0, stream, a);
+    else
+        hipLaunchKernelGGL((fwd_kernel<P, TB, TM>), grid, dim3(256), 0, stream, a);
     return check_launch("fwd_kernel");
 }
 
@@ -216,11 +412,17 @@ int launch_fwd(const FwdArgs& a, hipStream_t stream) {
 struct PolicyBase {
     static constexpr int NX = 1;
     static constexpr int PASSES = 1;
+    static constexpr int MIN_WAVES = 1;   // waves per SIMD the register budget must allow
+    static constexpr int PIPE_WAVES = 2;  // same for the pipelined kernel
+    static constexpr int UNROLL4 = 2;     // unroll factor of the loop over groups of four inputs
     template <class A> static __device__ __forceinline__ void chunk_end(A&, const FwdArgs&, int, int) {}
 };
 
 // l-inf forward without indices (core/cuda/inf_dist_cuda.cu:17-107)
 struct LinfNograd : PolicyBase {
+    static constexpr int PIPE_WAVES = SD_PIPEW;
+    static constexpr int MIN_WAVES = SD_MINW;
+    static constexpr int UNROLL4 = SD_UNR;
     struct Acc { float v; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.v = kEps; }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
@@ -274,6 +476,9 @@ __device__ __forceinline__ void store_chunk_winner(const FwdArgs& a, size_t o, f
 }
 
 struct LinfChunk : PolicyBase {
+    static constexpr int PIPE_WAVES = 2;   // three accumulator registers per output: no room for more waves
+    static constexpr int MIN_WAVES = 2;
+    static constexpr int UNROLL4 = 2;
     struct Acc { float best, cm; int cid; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.best = kEps; A.cm = 0.f; A.cid = -1; }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
@@ -292,6 +497,8 @@ struct LinfChunk : PolicyBase {
 
 // the per-term masked neuron with the same chunk tracking
 struct MaskedTermChunk : PolicyBase {
+    static constexpr int PIPE_WAVES = 2;
+    static constexpr int MIN_WAVES = 2;
     struct Acc { float best, cm; int cid; uint32_t key; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool) {
         A.best = kEps; A.cm = 0.f; A.cid = -1; A.key = rng_row_key(a.seed, 0u, (uint32_t)o);
@@ -343,7 +550,10 @@ struct MaskedTerm : PolicyBase {
 
 // interval bounds, values only (core/cuda/bound_inf_dist_cuda.cu:15-118)
 struct BoundNograd : PolicyBase {
+    static constexpr int PIPE_WAVES = SD_PIPEW;
     static constexpr int NX = 2;
+    static constexpr int MIN_WAVES = SD_MINW;
+    static constexpr int UNROLL4 = SD_UNR;
     struct Acc { float lo, hi; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.lo = -kEps; A.hi = kEps; }
     static __device__ __forceinline__ void term(Acc& A, float l, float u, float w) {
@@ -612,18 +822,60 @@ __global__ void __launch_bounds__(256) resolve_pos_kernel(FwdArgs a) {
         const float* wr = a.w + (size_t)(g * a.W_COg + wrow) * a.W_CIg;
         const float* xr = a.x0 + ((size_t)(b * a.G + g) * a.CIg) * a.HW + hw;
         const int* cidx = a.ci_idx ? a.ci_idx + (size_t)(s * a.G + g) * a.CIg : nullptr;
-        const uint32_t key_t = rng_row_key(a.seed, 0u, (uint32_t)o);
-        const uint32_t key_x = rng_row_key(a.seed, 1u, (uint32_t)((b * a.G + g) * a.HW + hw));
-        const uint32_t key_w = rng_row_key(a.seed, 2u, (uint32_t)c);
-        int n0 = cid * KT, n1 = n0 + KT < a.CIg ? n0 + KT : a.CIg;
-        for (int n = n0; n < n1; n++) {
-            bool keep = true;
-            if (a.mask_mode == SD_MASK_TERM)
-                keep = ((rng_word(key_t, (uint32_t)n >> 2) >> (8 * (n & 3))) & 0xffu) < a.t8;
-            else if (a.mask_mode == SD_MASK_FACTORED)
-                keep = (rng_word(key_x, (uint32_t)n) >> 16) < a.t16 && (rng_word(key_w, (uint32_t)n) >> 16) < a.t16;
-            float d = xr[(size_t)n * a.HW] - wr[cidx ? cidx[n] : n];
-            if (keep && fabsf(d) == best) { pos = n | (d < 0.f ? (int)kSign : 0); break; }
+        const int n0 = cid * KT;
+        // keep bits of the 32 inputs of the chunk
+        uint32_t keep = 0xffffffffu;
+        if (a.mask_mode == SD_MASK_TERM) {
+            const uint32_t key_t = rng_row_key(a.seed, 0u, (uint32_t)o);
+            keep = 0u;
+            #pragma unroll
+            for (int q4 = 0; q4 < KT / 4; q4++) {
+                uint32_t word = rng_word(key_t, (uint32_t)(n0 >> 2) + q4);
+                #pragma unroll
+                for (int c4 = 0; c4 < 4; c4++)
+                    if (((word >> (8 * c4)) & 0xffu) < a.t8) keep |= 1u << (q4 * 4 + c4);
+            }
+        } else if (a.mask_mode == SD_MASK_FACTORED) {
+            if (a.xmask) {
+                const int nchunks = (a.CIg + KT - 1) / KT;
+                keep = a.xmask[(size_t)((b * a.G + g) * a.HW + hw) * nchunks + cid] & a.wmask[(size_t)c * nchunks + cid];
+            } else {
+                const uint32_t key_x = rng_row_key(a.seed, 1u, (uint32_t)((b * a.G + g) * a.HW + hw));
+                const uint32_t key_w = rng_row_key(a.seed, 2u, (uint32_t)c);
+                keep = 0u;
+                for (int k = 0; k < KT; k++)
+                    if ((rng_word(key_x, (uint32_t)(n0 + k)) >> 16) < a.t16 && (rng_word(key_w, (uint32_t)(n0 + k)) >> 16) < a.t16)
+                        keep |= 1u << k;
+            }
+        }
+        if (a.fast_x && a.fast_w) {
+            // 128-bit loads of the whole chunk, then a branch-free scan from the top so that the
+            // lowest matching input is the one that remains
+            float4 xv[KT / 4], wv[KT / 4];
+            #pragma unroll
+            for (int q4 = 0; q4 < KT / 4; q4++) {
+                int n = n0 + 4 * q4;
+                if (n > a.CIg - 4) n = a.CIg - 4;
+                xv[q4] = *reinterpret_cast<const float4*>(xr + n);
+                wv[q4] = *reinterpret_cast<const float4*>(wr + n);
+            }
+            #pragma unroll
+            for (int q4 = KT / 4 - 1; q4 >= 0; q4--) {
+                const int n = n0 + 4 * q4;
+                const bool in = n < a.CIg;
+                float d3 = xv[q4].w - wv[q4].w, d2 = xv[q4].z - wv[q4].z, d1 = xv[q4].y - wv[q4].y, d0 = xv[q4].x - wv[q4].x;
+                uint32_t kb = keep >> (4 * q4);
+                if (in && (kb & 8u) && fabsf(d3) == best) pos = (n + 3) | (d3 < 0.f ? (int)kSign : 0);
+                if (in && (kb & 4u) && fabsf(d2) == best) pos = (n + 2) | (d2 < 0.f ? (int)kSign : 0);
+                if (in && (kb & 2u) && fabsf(d1) == best) pos = (n + 1) | (d1 < 0.f ? (int)kSign : 0);
+                if (in && (kb & 1u) && fabsf(d0) == best) pos = n | (d0 < 0.f ? (int)kSign : 0);
+            }
+        } else {
+            const int n1 = n0 + KT < a.CIg ? n0 + KT : a.CIg;
+            for (int n = n0; n < n1; n++) {
+                float d = xr[(size_t)n * a.HW] - wr[cidx ? cidx[n] : n];
+                if (((keep >> (n - n0)) & 1u) && fabsf(d) == best) { pos = n | (d < 0.f ? (int)kSign : 0); break; }
+            }
         }
     }
     a.y0[o] = best;

@@ -4,6 +4,31 @@
 
 using namespace sd;
 
+#ifndef SD_NG_TB
+#define SD_NG_TB 8
+#endif
+#ifndef SD_BD_TM
+#define SD_BD_TM 8
+#endif
+
+// One work-item per (row, chunk): the 32 keep bits of the factored mask for inputs
+// chunk*32 .. chunk*32+31 of an x row (stream 1) or a w row (stream 2).
+static __global__ void __launch_bounds__(256) build_masks_kernel(uint32_t* __restrict__ out, long long rows, int nchunks,
+                                                          int CIg, uint32_t seed, uint32_t stream, uint32_t t16) {
+    long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * nchunks) return;
+    uint32_t row = (uint32_t)(i / nchunks);
+    int chunk = (int)(i - (long long)row * nchunks);
+    uint32_t key = rng_row_key(seed, stream, row);
+    uint32_t bits = 0;
+    #pragma unroll 8
+    for (int k = 0; k < KT; k++) {
+        int n = chunk * KT + k;
+        if (n < CIg && (rng_word(key, (uint32_t)n) >> 16) < t16) bits |= 1u << k;
+    }
+    out[i] = bits;
+}
+
 // forward with positions: chunk-tracking kernel (split-N through the packed workspace when the
 // grid would otherwise be too small) followed by the position resolve pass
 template <class P>
@@ -13,8 +38,10 @@ static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st) {
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     int rc;
     if (a.nsplit > 1) {
+        // the merge buffer sits at the start of the workspace; a factored-mask call has already sized
+        // the workspace for it and placed its bit masks behind it
         size_t n = (size_t)a.R * a.G * a.COg;
-        a.packed0 = static_cast<unsigned long long*>(workspace(n * 8));
+        a.packed0 = static_cast<unsigned long long*>(a.xmask ? workspace(0) : workspace(n * 8));
         if (!a.packed0) return SD_ERR_HIP;
         if ((rc = fill_zero(a.packed0, n * 2, st))) return rc;
     }
@@ -31,7 +58,7 @@ extern "C" int sd_inf_dist_forward_nograd(const float* input, const float* weigh
     SD_REQUIRE(output, "inf_dist_forward_nograd: null output");
     a.y0 = output;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int TB = a.R <= 32 ? 2 : a.R <= 64 ? 4 : 8;
+    const int TB = a.R <= 32 ? 2 : a.R <= 64 ? 4 : SD_NG_TB;
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;
     if (TB == 2) return launch_fwd<LinfNograd, 2, 8>(a, st);
@@ -65,14 +92,31 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
     a.y0 = output; a.p0 = pos;
     a.q = q; a.seed = seed; a.mask_mode = mode;
     a.t8 = sd_mask_threshold8(q); a.t16 = sd_mask_threshold16(q);
-    hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = a.R <= 32;
+    hipStream_t st = static_cast<hipStream_t>(stream);
     if (mode == SD_MASK_TERM) {
         if (pos) return run_chunk_pos<MaskedTermChunk>(a, false, st);
         return small ? launch_fwd<MaskedTerm<false>, 2, 8>(a, st) : launch_fwd<MaskedTerm<false>, 4, 8>(a, st);
     }
     // factored mask: dropped inputs / weights are replaced by NaN while staging the tiles and
-    // NaN terms never win the maximum, so the plain l-inf policies apply unchanged
+    // NaN terms never win the maximum, so the plain l-inf policies apply unchanged.  On the
+    // vector-load path the keep bits are built once per call into the library workspace.
+    size_t packed_bytes = 0;
+    if (a.fast_x && a.fast_w) {
+        const int nchunks = (a.CIg + KT - 1) / KT;
+        const long long xrows = (long long)a.R * G, wrows = (long long)CO;
+        packed_bytes = pos ? (((size_t)a.R * CO * 8 + 255) / 256) * 256 : 0;
+        char* base = static_cast<char*>(workspace(packed_bytes + (size_t)(xrows + wrows) * nchunks * 4));
+        if (!base) return SD_ERR_HIP;
+        uint32_t* xm = reinterpret_cast<uint32_t*>(base + packed_bytes);
+        uint32_t* wm = xm + xrows * nchunks;
+        hipLaunchKernelGGL(build_masks_kernel, dim3((unsigned)((xrows * nchunks + 255) / 256)), dim3(256), 0, st,
+                           xm, xrows, nchunks, a.CIg, seed, 1u, a.t16);
+        hipLaunchKernelGGL(build_masks_kernel, dim3((unsigned)((wrows * nchunks + 255) / 256)), dim3(256), 0, st,
+                           wm, wrows, nchunks, a.CIg, seed, 2u, a.t16);
+        if ((rc = check_launch("build_masks_kernel"))) return rc;
+        a.xmask = xm; a.wmask = wm;
+    }
     if (pos) return run_chunk_pos<LinfChunk>(a, false, st);
     const int TB = a.R <= 32 ? 2 : a.R <= 64 ? 4 : 8;
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
@@ -94,13 +138,13 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
     a.y0 = outputL; a.y1 = outputU;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int TB = a.R <= 32 ? 2 : 4;
-    a.nsplit = pick_nsplit(a, 16 * TB, 128);
+    a.nsplit = pick_nsplit(a, 16 * TB, 16 * SD_BD_TM);
     if (a.nsplit > 1) {
         if ((rc = fill_zero(outputL, (size_t)B * CO * HW, st))) return rc;
         if ((rc = fill_zero(outputU, (size_t)B * CO * HW, st))) return rc;
     }
     if (TB == 2) return launch_fwd<BoundNograd, 2, 8>(a, st);
-    return launch_fwd<BoundNograd, 4, 8>(a, st);
+    return launch_fwd<BoundNograd, 4, SD_BD_TM>(a, st);
 }
 
 extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* inputU, const float* weight,

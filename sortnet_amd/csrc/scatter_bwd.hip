@@ -74,6 +74,81 @@ __global__ void __launch_bounds__(256) bound_bwd_kernel(BwdArgs a) {
     if (HAS_W) unsafeAtomicAdd(a.gw + wrow + nu, -vu);
 }
 
+// Row-histogram variants: one workgroup owns one (sample, group, position) row of grad_input,
+// accumulates it in LDS (colliding adds stay on chip) and writes it out once, so grad_input needs
+// neither a zero-fill pass nor global atomics.  grad_weight is still scattered with atomics.
+constexpr int kMaxRowLds = 12288;   // floats of LDS one row histogram may take
+
+template <bool SORT, bool HAS_W>
+__global__ void __launch_bounds__(256) scatter_bwd_rows_kernel(BwdArgs a) {
+    extern __shared__ float hist[];
+    const int row = blockIdx.x;                 // ((b * G) + g) * HW + hw
+    const int hw = row % a.HW;
+    const int bg = row / a.HW;
+    const int g = bg % a.G, b = bg / a.G;
+    const int s = b / kSubBatch;
+    for (int n = threadIdx.x; n < a.CIg; n += 256) hist[n] = 0.f;
+    __syncthreads();
+    const size_t obase = ((size_t)(b * a.G + g) * a.COg) * a.HW + hw;
+    const int K = SORT ? a.K : 1;
+    for (int m = threadIdx.x; m < a.COg; m += 256) {
+        size_t o = obase + (size_t)m * a.HW;
+        float grad = a.g0[o];
+        float coef = a.coef0;
+        size_t wrow = 0;
+        if (HAS_W) {
+            int mm = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + m] : m;
+            wrow = (size_t)(g * a.W_COg + mm) * a.W_CIg;
+        }
+        for (int k = 0; k < K; k++) {
+            int pr = a.p0[(size_t)k * a.total + o];
+            int n = pr & 0x7fffffff;
+            float v = pr >= 0 ? grad : -grad;
+            if (SORT) { v = v * coef * a.q; coef *= 1.f - a.q; }
+            atomicAdd(&hist[n], v);
+            if (HAS_W) {
+                int nn = a.ci_idx ? a.ci_idx[(s * a.G + g) * a.CIg + n] : n;
+                unsafeAtomicAdd(a.gw + wrow + nn, -v);
+            }
+        }
+    }
+    __syncthreads();
+    const size_t xbase = ((size_t)(b * a.G + g) * a.CIg) * a.HW + hw;
+    for (int n = threadIdx.x; n < a.CIg; n += 256) a.gx0[xbase + (size_t)n * a.HW] = hist[n];
+}
+
+template <bool HAS_W>
+__global__ void __launch_bounds__(256) bound_bwd_rows_kernel(BwdArgs a) {
+    extern __shared__ float hist[];             // [0, CIg) lower, [CIg, 2 CIg) upper
+    const int row = blockIdx.x;
+    const int hw = row % a.HW;
+    const int bg = row / a.HW;
+    const int g = bg % a.G, b = bg / a.G;
+    for (int n = threadIdx.x; n < 2 * a.CIg; n += 256) hist[n] = 0.f;
+    __syncthreads();
+    const size_t obase = ((size_t)(b * a.G + g) * a.COg) * a.HW + hw;
+    for (int m = threadIdx.x; m < a.COg; m += 256) {
+        size_t o = obase + (size_t)m * a.HW;
+        size_t wrow = (size_t)(g * a.COg + m) * a.CIg;
+        int pl = a.p0[o], pu = a.p1[o];
+        float gl = a.g0[o], gu = a.g1[o];
+        int nl = pl & 0x7fffffff, nu = pu & 0x7fffffff;
+        float vl = pl >= 0 ? gl : -gl, vu = pu >= 0 ? gu : -gu;
+        if ((uint32_t)pl != kNanId) {
+            atomicAdd(&hist[(pl >= 0 ? 0 : a.CIg) + nl], vl);
+            if (HAS_W) unsafeAtomicAdd(a.gw + wrow + nl, -vl);
+        }
+        atomicAdd(&hist[(pu >= 0 ? a.CIg : 0) + nu], vu);
+        if (HAS_W) unsafeAtomicAdd(a.gw + wrow + nu, -vu);
+    }
+    __syncthreads();
+    const size_t xbase = ((size_t)(b * a.G + g) * a.CIg) * a.HW + hw;
+    for (int n = threadIdx.x; n < a.CIg; n += 256) {
+        a.gx0[xbase + (size_t)n * a.HW] = hist[n];
+        a.gx1[xbase + (size_t)n * a.HW] = hist[a.CIg + n];
+    }
+}
+
 static int make_bwd_args(BwdArgs& a, const char* who, int B, int CO, int CI, int G, int HW,
                          const int* ci_idx, const int* co_idx, int W_CO, int W_CI) {
     SD_REQUIRE(B > 0 && CO > 0 && CI > 0 && G > 0 && HW > 0, "%s: sizes must be positive", who);
@@ -95,8 +170,15 @@ static int make_bwd_args(BwdArgs& a, const char* who, int B, int CO, int CI, int
 template <bool SORT>
 static int run_scatter(BwdArgs& a, hipStream_t st) {
     int rc;
-    if ((rc = fill_zero(a.gx0, (size_t)a.B * a.G * a.CIg * a.HW, st))) return rc;
     if (a.gw && (rc = fill_zero(a.gw, (size_t)a.G * a.W_COg * a.W_CIg, st))) return rc;
+    if (a.CIg <= kMaxRowLds) {
+        dim3 rows((unsigned)(a.B * a.G * a.HW));
+        size_t lds = (size_t)a.CIg * sizeof(float);
+        if (a.gw) hipLaunchKernelGGL((scatter_bwd_rows_kernel<SORT, true>), rows, dim3(256), lds, st, a);
+        else hipLaunchKernelGGL((scatter_bwd_rows_kernel<SORT, false>), rows, dim3(256), lds, st, a);
+        return check_launch("scatter_bwd_rows_kernel");
+    }
+    if ((rc = fill_zero(a.gx0, (size_t)a.B * a.G * a.CIg * a.HW, st))) return rc;
     dim3 grid((unsigned)((a.total + 255) / 256));
     if (a.gw) hipLaunchKernelGGL((scatter_bwd_kernel<SORT, true>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((scatter_bwd_kernel<SORT, false>), grid, dim3(256), 0, st, a);
@@ -167,9 +249,16 @@ static int bound_bwd(const char* who, const float* gL, const float* gU, const in
     a.g0 = gL; a.g1 = gU; a.p0 = posL; a.p1 = posU; a.gx0 = gxL; a.gx1 = gxU; a.gw = gw;
     hipStream_t st = static_cast<hipStream_t>(stream);
     size_t nx = (size_t)B * CI * HW;
+    if (gw && (rc = fill_zero(gw, (size_t)CO * a.CIg, st))) return rc;
+    if (2 * a.CIg <= kMaxRowLds) {
+        dim3 rows((unsigned)(B * G * HW));
+        size_t lds = (size_t)2 * a.CIg * sizeof(float);
+        if (gw) hipLaunchKernelGGL((bound_bwd_rows_kernel<true>), rows, dim3(256), lds, st, a);
+        else hipLaunchKernelGGL((bound_bwd_rows_kernel<false>), rows, dim3(256), lds, st, a);
+        return check_launch("bound_bwd_rows_kernel");
+    }
     if ((rc = fill_zero(gxL, nx, st))) return rc;
     if ((rc = fill_zero(gxU, nx, st))) return rc;
-    if (gw && (rc = fill_zero(gw, (size_t)CO * a.CIg, st))) return rc;
     dim3 grid((unsigned)((a.total + 255) / 256));
     if (gw) hipLaunchKernelGGL((bound_bwd_kernel<true>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((bound_bwd_kernel<false>), grid, dim3(256), 0, st, a);

@@ -76,6 +76,33 @@ def test_inf_dist_forward_and_backward(oracle, B, CI, CO, G, HW):
     _close(gx2, rgx)
 
 
+def test_backward_long_rows_use_global_atomics(oracle):
+    """Reduction length above the LDS row-histogram limit: the atomic fallback kernels."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, CI, CO = 3, 12300, 5
+    x, w, gy = _gen((B, CI, 1), 61, "rand"), _gen((CO, CI), 62, scale=0.3), _gen((B, CO, 1), 63)
+    ry, rpos = oracle.inf_dist_forward(x.numpy(), w.numpy())
+    y = torch.empty(B, CO, 1, device=dev)
+    pos = torch.empty(B, CO, 1, device=dev, dtype=torch.int32)
+    ext.inf_dist_forward(x.to(dev), w.to(dev), y, pos, 1)
+    assert np.array_equal(y.cpu().numpy(), ry) and np.array_equal(pos.cpu().numpy(), rpos)
+    rgx, rgw = oracle.inf_dist_backward(gy.numpy(), rpos, x.shape, w.shape)
+    gx, gw = torch.empty(B, CI, 1, device=dev), torch.empty(CO, CI, device=dev)
+    ext.inf_dist_backward_input_weight(gy.to(dev), pos, gx, gw, 1)
+    _close(gx, rgx)
+    _close(gw, rgw)
+    xl, xu = (x - 0.01).contiguous(), (x + 0.01).contiguous()
+    rl, ru, rpl, rpu = oracle.bound_inf_dist_forward(xl.numpy(), xu.numpy(), w.numpy())
+    rgl, rgu, rgw2 = oracle.bound_inf_dist_backward(gy.numpy(), gy.numpy(), rpl, rpu, x.shape, w.shape)
+    gl, gu, gw2 = torch.empty(B, CI, 1, device=dev), torch.empty(B, CI, 1, device=dev), torch.empty(CO, CI, device=dev)
+    ext.bound_inf_dist_backward_input_weight(gy.to(dev), gy.to(dev), torch.from_numpy(rpl).to(dev),
+                                             torch.from_numpy(rpu).to(dev), gl, gu, gw2, 1)
+    _close(gl, rgl)
+    _close(gu, rgu)
+    _close(gw2, rgw2)
+
+
 def test_inf_dist_ties_and_floor(oracle):
     from sortnet_amd import ext
     dev = _dev()
