@@ -156,6 +156,20 @@ int sd_masked_inf_dist_forward(const float* input, const float* weight,
                                int B, int CO, int CI, int G, int HW, float* output, int* pos,
                                float q, uint32_t seed, int mode, sd_stream_t stream);
 
+/* ---- mean shift, the step after every distance layer (MeanShiftDropout without index list,
+ * core/models/bound_basic_module.py:123-157; done with torch ops in the reference) ---- */
+
+/* Training form: mean[c] = mean over (b, hw) of input; running_mean (may be NULL) is updated in place as
+ * (1 - momentum) running_mean + momentum mean; output = input - mean[c].  Applied to an upstream
+ * gradient with running_mean = NULL it is also the backward of itself. */
+int sd_mean_shift_forward(const float* input, int B, int C, int HW, float* mean, float* running_mean,
+                          float momentum, float* output, sd_stream_t stream);
+
+/* output = input + sign * shift[c]: evaluation-mode mean shift (sign = -1) and bias add (sign = +1),
+ * core/models/bound_basic_module.py:155 and core/models/norm_dist.py:102-103. */
+int sd_channel_shift(const float* input, const float* shift, int B, int C, int HW, float sign,
+                     float* output, sd_stream_t stream);
+
 /* The counter RNG and the thresholds it is compared with, exposed for verification. */
 uint32_t sd_rng_word(uint32_t seed, uint32_t stream_id, uint32_t row, uint32_t col);
 uint32_t sd_mask_threshold8(float q);

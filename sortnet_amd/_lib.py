@@ -37,6 +37,8 @@ SIGNATURES = {
     "sd_norm_dist_backward_input": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _f, _I, _I, _i, _i, _S],
     "sd_norm_dist_backward_input_weight": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _F, _f, _I, _I, _i, _i, _S],
     "sd_masked_inf_dist_forward": [_F, _F, _i, _i, _i, _i, _i, _F, _I, _f, _u, _i, _S],
+    "sd_mean_shift_forward": [_F, _i, _i, _i, _F, _F, _f, _F, _S],
+    "sd_channel_shift": [_F, _F, _i, _i, _i, _f, _F, _S],
 }
 _OTHER = {
     "sd_version": ([], _i),

@@ -1,0 +1,108 @@
+// Mean shift over batch and spatial positions, the step that follows every distance layer
+// (core/models/bound_basic_module.py:106-157, training form without index list):
+//   mean[c] = mean_{b,hw} x[b,c,hw];  running = (1 - momentum) running + momentum mean;  y = x - mean[c]
+// and the plain per-channel shift y = x - shift[c] used in evaluation mode and for a bias.
+#include "common.h"
+
+namespace sd {
+
+// One workgroup owns 64 channels (HW == 1) or one channel (HW > 1); 16 groups of 64 work-items walk
+// the batch in parallel, partial sums meet in LDS, the sum order is fixed (deterministic result).
+__global__ void __launch_bounds__(1024) channel_mean_kernel(const float* __restrict__ x, int B, int C, int HW,
+                                                            float* __restrict__ mean, float* __restrict__ running,
+                                                            float momentum) {
+    __shared__ float part[16][64];
+    const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    float s = 0.f;
+    if (HW == 1) {
+        const int c = blockIdx.x * 64 + lane;
+        if (c < C)
+            for (int b = grp; b < B; b += 16) s += x[(size_t)b * C + c];
+        part[grp][lane] = s;
+        __syncthreads();
+        if (grp == 0 && c < C) {
+            float t = 0.f;
+            #pragma unroll
+            for (int k = 0; k < 16; k++) t += part[k][lane];
+            float m = t / (float)B;
+            mean[c] = m;
+            if (running) running[c] = (1.f - momentum) * running[c] + momentum * m;
+        }
+    } else {
+        const int c = blockIdx.x;
+        const long long n = (long long)B * HW;
+        for (long long i = threadIdx.x; i < n; i += 1024) {
+            long long b = i / HW, hw = i - b * HW;
+            s += x[((size_t)b * C + c) * HW + hw];
+        }
+        part[grp][lane] = s;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float t = 0.f;
+            for (int k = 0; k < 16; k++)
+                for (int l = 0; l < 64; l++) t += part[k][l];
+            float m = t / (float)n;
+            mean[c] = m;
+            if (running) running[c] = (1.f - momentum) * running[c] + momentum * m;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) channel_shift_kernel(const float* __restrict__ x, const float* __restrict__ shift,
+                                                            long long total, int C, int HW, float sign,
+                                                            float* __restrict__ y) {
+    long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= total) return;
+    if (HW == 1 && C % 4 == 0 && i + 3 < total) {
+        float4 v = *reinterpret_cast<const float4*>(x + i);
+        float4 sh = *reinterpret_cast<const float4*>(shift + (i % C));
+        v.x += sign * sh.x; v.y += sign * sh.y; v.z += sign * sh.z; v.w += sign * sh.w;
+        *reinterpret_cast<float4*>(y + i) = v;
+    } else {
+        for (int k = 0; k < 4 && i + k < total; k++) {
+            long long j = i + k;
+            int c = (int)((j / HW) % C);
+            y[j] = x[j] + sign * shift[c];
+        }
+    }
+}
+
+static int check_dims(const char* who, int B, int C, int HW) {
+    SD_REQUIRE(B > 0 && C > 0 && HW > 0, "%s: sizes must be positive", who);
+    SD_REQUIRE((long long)B * C * HW < (1ll << 31), "%s: tensor too large for 32-bit indexing", who);
+    return SD_OK;
+}
+
+}  // namespace sd
+
+using namespace sd;
+
+extern "C" int sd_mean_shift_forward(const float* input, int B, int C, int HW, float* mean, float* running_mean,
+                                     float momentum, float* output, sd_stream_t stream) {
+    int rc = check_dims("mean_shift_forward", B, C, HW);
+    if (rc) return rc;
+    SD_REQUIRE(input && mean && output, "mean_shift_forward: null pointer");
+    SD_REQUIRE(reinterpret_cast<uintptr_t>(input) % 16 == 0 && reinterpret_cast<uintptr_t>(output) % 16 == 0 &&
+               reinterpret_cast<uintptr_t>(mean) % 16 == 0, "mean_shift_forward: buffers must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    dim3 grid(HW == 1 ? (C + 63) / 64 : C);
+    hipLaunchKernelGGL(channel_mean_kernel, grid, dim3(1024), 0, st, input, B, C, HW, mean, running_mean, momentum);
+    if ((rc = check_launch("channel_mean_kernel"))) return rc;
+    long long total = (long long)B * C * HW;
+    hipLaunchKernelGGL(channel_shift_kernel, dim3((unsigned)((total / 4 + 255) / 256 + 1)), dim3(256), 0, st,
+                       input, mean, total, C, HW, -1.f, output);
+    return check_launch("channel_shift_kernel");
+}
+
+extern "C" int sd_channel_shift(const float* input, const float* shift, int B, int C, int HW, float sign,
+                                float* output, sd_stream_t stream) {
+    int rc = check_dims("channel_shift", B, C, HW);
+    if (rc) return rc;
+    SD_REQUIRE(input && shift && output, "channel_shift: null pointer");
+    SD_REQUIRE(reinterpret_cast<uintptr_t>(input) % 16 == 0 && reinterpret_cast<uintptr_t>(output) % 16 == 0 &&
+               reinterpret_cast<uintptr_t>(shift) % 16 == 0, "channel_shift: buffers must be 16-byte aligned");
+    long long total = (long long)B * C * HW;
+    hipLaunchKernelGGL(channel_shift_kernel, dim3((unsigned)((total / 4 + 255) / 256 + 1)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), input, shift, total, C, HW, sign, output);
+    return check_launch("channel_shift_kernel");
+}

@@ -162,3 +162,17 @@ def masked_inf_dist_forward(input, weight, output, pos, G, q, seed, mode=MASK_TE
     B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
     _run("sd_masked_inf_dist_forward", input, _chk(input, "input"), _chk(weight, "weight"), B, CO, CI, G, HW,
          _chk(output, "output"), None if pos is None else _chk(pos, "pos", torch.int32), q, seed & 0xFFFFFFFF, mode)
+
+
+def mean_shift_forward(input, mean, running_mean, momentum, output):
+    """Not in the reference extension (done there with torch ops): mean over batch and positions,
+    optional in-place running-mean update, output = input - mean."""
+    B, C, HW = input.size(0), input.size(1), input.size(2)
+    _run("sd_mean_shift_forward", input, _chk(input, "input"), B, C, HW, _chk(mean, "mean"),
+         None if running_mean is None else _chk(running_mean, "running_mean"), momentum, _chk(output, "output"))
+
+
+def channel_shift(input, shift, sign, output):
+    """output = input + sign * shift[c] (evaluation-mode mean shift, bias add)."""
+    B, C, HW = input.size(0), input.size(1), input.size(2)
+    _run("sd_channel_shift", input, _chk(input, "input"), _chk(shift, "shift"), B, C, HW, sign, _chk(output, "output"))

@@ -17,6 +17,7 @@ from . import ext as _C
 __all__ = [
     "NormDistF", "NormDistDropoutF", "SortNeuronF", "BoundInfDistF", "MaskedInfDistF",
     "norm_dist", "norm_dist_dropout", "sort_neuron", "bound_sort_neuron", "bound_inf_dist", "masked_inf_dist",
+    "MeanShiftF", "mean_shift",
 ]
 
 
@@ -233,6 +234,35 @@ class MaskedInfDistF(torch.autograd.Function):
         elif want_x:
             _C.inf_dist_backward_input(grad_output, pos, grad_input, ctx.group)
         return (grad_input if want_x else None), grad_weight, None, None, None, None, None, None
+
+
+class MeanShiftF(torch.autograd.Function):
+    """y = x - mean_{b,hw}(x) with the mean inside the graph, plus the running-mean update the
+    reference's MeanShiftDropout does under no_grad (core/models/bound_basic_module.py:123-157, the
+    form without an index list).  The backward of the centring is the centring of the gradient."""
+
+    @staticmethod
+    def forward(ctx, x, running_mean, momentum):
+        x = x.contiguous()
+        y = torch.empty_like(x)
+        mean = torch.empty(x.size(1), device=x.device, dtype=torch.float32)
+        _C.mean_shift_forward(x, mean, running_mean, momentum, y)
+        ctx.mark_non_differentiable(mean)
+        return y, mean
+
+    @staticmethod
+    def backward(ctx, grad_y, _grad_mean):
+        grad_y = grad_y.contiguous()
+        grad_x = torch.empty_like(grad_y)
+        scratch = torch.empty(grad_y.size(1), device=grad_y.device, dtype=torch.float32)
+        _C.mean_shift_forward(grad_y, scratch, None, 0.0, grad_x)
+        return grad_x, None, None
+
+
+def mean_shift(x, running_mean=None, momentum=0.1):
+    """Training-mode mean shift of a (B, C, HW) tensor; returns (x - mean, mean) and updates
+    `running_mean` in place when given."""
+    return MeanShiftF.apply(x, running_mean, momentum)
 
 
 def norm_dist(input, weight, p, groups=1, use_custom_cuda_func=True, tag=None):

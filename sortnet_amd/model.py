@@ -43,10 +43,7 @@ class DistanceMLP:
             else:
                 h = F.masked_inf_dist(h, w, self.q, seed=step_seed * 64 + i, mode=self.mask_mode)
             if i < self.num_layers - 1:
-                mean = h.mean(dim=(0, 2))
-                with torch.no_grad():
-                    self.running_mean[i].mul_(1 - self.momentum).add_(mean, alpha=self.momentum)
-                h = h - mean.view(1, -1, 1)
+                h, _ = F.mean_shift(h, self.running_mean[i], self.momentum)
             else:
                 h = h + self.bias.view(1, -1, 1)
         return h.squeeze(-1)

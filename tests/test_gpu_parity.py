@@ -386,6 +386,32 @@ def test_full_size_properties():
     assert torch.equal(ym, y)
 
 
+@pytest.mark.parametrize("B,C,HW", [(70, 200, 1), (33, 37, 1), (6, 24, 3), (512, 5120, 1)])
+def test_mean_shift(oracle, B, C, HW):
+    from sortnet_amd import ext
+    import sortnet_amd.functional as F
+    dev = _dev()
+    x = _gen((B, C, HW), 71)
+    rout, rmean = oracle.mean_shift(x.numpy())
+    xd = x.to(dev)
+    y, mean = torch.empty_like(xd), torch.empty(C, device=dev)
+    running = torch.full((C,), 0.5, device=dev)
+    ext.mean_shift_forward(xd, mean, running, 0.1, y)
+    np.testing.assert_allclose(mean.cpu().numpy(), rmean, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(y.cpu().numpy(), rout, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(running.cpu().numpy(), 0.45 + 0.1 * rmean, rtol=1e-5, atol=1e-6)
+    z = torch.empty_like(xd)
+    ext.channel_shift(xd, mean, -1.0, z)
+    assert torch.equal(z, y)
+    # autograd: the gradient of the centring is the centring of the gradient
+    xg = xd.clone().requires_grad_()
+    g = _gen((B, C, HW), 72).to(dev)
+    out, _ = F.mean_shift(xg)
+    out.backward(g)
+    ref = g - g.mean(dim=(0, 2), keepdim=True)
+    np.testing.assert_allclose(xg.grad.cpu().numpy(), ref.cpu().numpy(), rtol=1e-5, atol=1e-6)
+
+
 def test_argument_errors():
     from sortnet_amd import ext
     dev = _dev()
