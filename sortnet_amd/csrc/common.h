@@ -40,6 +40,7 @@ struct FwdArgs {
     int* p0;              // pos / posL / sort pos (K, B, CO, HW)
     int* p1;              // posU
     unsigned long long* packed0;  // (value bits << 32 | ~chunk) merge buffer of split-N position kernels
+    unsigned long long* packed1;  // same for the upper bound of the interval kernel
     const uint32_t* xmask;  // factored mask: keep bits of x rows, one word per (row, chunk), or null
     const uint32_t* wmask;  // same for w rows
     const int* ci_idx;    // (S, G, CIg) or null

@@ -465,14 +465,15 @@ struct LinfPos : PolicyBase {
 // chunk attaining the final value survives.  The (best, chunk) pairs of the split-N slices are
 // merged with a 64-bit atomic max on (value bits << 32 | ~chunk) and resolve_pos_kernel then
 // rescans the one winning chunk of every output for the first input attaining the value.
-__device__ __forceinline__ void store_chunk_winner(const FwdArgs& a, size_t o, float best, int cid) {
+__device__ __forceinline__ void store_chunk_winner(const FwdArgs& a, size_t o, float best, int cid, bool upper = false) {
     if (a.nsplit > 1) {
         if (cid >= 0) {
             unsigned long long key = ((unsigned long long)__float_as_uint(best) << 32) |
                                      (unsigned long long)(0xffffffffu - (uint32_t)cid);
-            atomicMax(a.packed0 + o, key);
+            atomicMax((upper ? a.packed1 : a.packed0) + o, key);
         }
-    } else { a.y0[o] = best; a.p0[o] = cid; }
+    } else if (upper) { a.y1[o] = best; a.p1[o] = cid; }
+    else { a.y0[o] = best; a.p0[o] = cid; }
 }
 
 struct LinfChunk : PolicyBase {
@@ -595,6 +596,37 @@ struct BoundPos : PolicyBase {
     static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
         a.y0[o] = -A.lo; a.y1[o] = A.hi;
         a.p0[o] = (int)A.pl; a.p1[o] = (int)A.pu;
+    }
+};
+
+// interval bounds with indices, chunk-tracked like LinfChunk: the lower side tracks the largest
+// -min(t1,t2) (a positive number once it passes 1e-10), the upper side the largest max(t1,t2);
+// resolve_bound_kernel recovers the exact positions and branch bits
+struct BoundChunk : PolicyBase {
+    static constexpr int NX = 2;
+    static constexpr int PIPE_WAVES = 2;
+    static constexpr int MIN_WAVES = 2;
+    struct Acc { float lo, hi, cl, ch; int il, ih; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
+        A.lo = -kEps; A.hi = kEps; A.cl = 0.f; A.ch = 0.f; A.il = -1; A.ih = -1;
+    }
+    static __device__ __forceinline__ void term(Acc& A, float l, float u, float w) {
+        float t1 = w - l, t2 = u - w;
+        A.cl = fminf(fminf(A.cl, t1), t2);
+        A.ch = fmaxf(fmaxf(A.ch, t1), t2);
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& l, const float4& u,
+                                                 const float4& w, int, int) {
+        term(A, l.x, u.x, w.x); term(A, l.y, u.y, w.y); term(A, l.z, u.z, w.z); term(A, l.w, u.w, w.w);
+    }
+    static __device__ __forceinline__ void chunk_end(Acc& A, const FwdArgs&, int, int k0) {
+        if (A.cl < A.lo) { A.lo = A.cl; A.il = k0 / KT; }
+        if (A.ch > A.hi) { A.hi = A.ch; A.ih = k0 / KT; }
+        A.cl = 0.f; A.ch = 0.f;
+    }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+        store_chunk_winner(a, o, -A.lo, A.il, false);
+        store_chunk_winner(a, o, A.hi, A.ih, true);
     }
 };
 
@@ -880,6 +912,81 @@ __global__ void __launch_bounds__(256) resolve_pos_kernel(FwdArgs a) {
     }
     a.y0[o] = best;
     a.p0[o] = pos;
+}
+
+// Position resolve of the interval kernel: rescans the winning chunk of the lower and of the upper
+// bound for the first input attaining the bound and rebuilds pos = n | (t1 <= t2 ? 0 : 1 << 31);
+// a lower bound that never left its -1e-10 start keeps the 0xffffffff "no gradient" position.
+template <bool PACKED>
+__global__ void __launch_bounds__(256) resolve_bound_kernel(FwdArgs a) {
+    long long total = (long long)a.R * a.G * a.COg;
+    long long o = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (o >= total) return;
+    int hw = (int)(o % a.HW);
+    long long t = o / a.HW;
+    int c = (int)(t % (a.G * a.COg));
+    int b = (int)(t / (a.G * a.COg));
+    int g = c / a.COg;
+    float vl, vu; int cl, cu;
+    if (PACKED) {
+        unsigned long long pl = a.packed0[o], pu = a.packed1[o];
+        uint32_t ll = (uint32_t)pl, lu = (uint32_t)pu;
+        vl = ll ? __uint_as_float((uint32_t)(pl >> 32)) : kEps; cl = ll ? (int)(0xffffffffu - ll) : -1;
+        vu = lu ? __uint_as_float((uint32_t)(pu >> 32)) : kEps; cu = lu ? (int)(0xffffffffu - lu) : -1;
+    } else { vl = a.y0[o]; cl = a.p0[o]; vu = a.y1[o]; cu = a.p1[o]; }
+    const float* wr = a.w + (size_t)c * a.CIg;
+    const size_t xb = ((size_t)(b * a.G + g) * a.CIg) * a.HW + hw;
+    uint32_t posl = kNanId, posu = 0u;
+    #pragma unroll
+    for (int side = 0; side < 2; side++) {
+        const int cid = side ? cu : cl;
+        if (cid < 0) continue;
+        const int n0 = cid * KT, n1 = n0 + KT < a.CIg ? n0 + KT : a.CIg;
+        const float target = side ? vu : vl;
+        uint32_t found = side ? 0u : kNanId;
+        auto probe = [&](float l, float u, float w, int n) {
+            if (l > u) l = u = (l + u) * 0.5f;
+            float t1 = w - l, t2 = u - w;
+            float v = side ? fmaxf(t1, t2) : -fminf(t1, t2);
+            if (v == target) found = (uint32_t)n | (t1 <= t2 ? 0u : kSign);
+        };
+        if (a.fast_x && a.fast_w) {
+            // descending scan over 128-bit loads: the lowest matching input is the one that remains
+            float4 lv[KT / 4], uv[KT / 4], wv[KT / 4];
+            #pragma unroll
+            for (int q4 = 0; q4 < KT / 4; q4++) {
+                int n = n0 + 4 * q4;
+                if (n > a.CIg - 4) n = a.CIg - 4;
+                lv[q4] = *reinterpret_cast<const float4*>(a.x0 + xb + n);
+                uv[q4] = *reinterpret_cast<const float4*>(a.x1 + xb + n);
+                wv[q4] = *reinterpret_cast<const float4*>(wr + n);
+            }
+            #pragma unroll
+            for (int q4 = KT / 4 - 1; q4 >= 0; q4--) {
+                const int n = n0 + 4 * q4;
+                if (n < a.CIg) {
+                    probe(lv[q4].w, uv[q4].w, wv[q4].w, n + 3);
+                    probe(lv[q4].z, uv[q4].z, wv[q4].z, n + 2);
+                    probe(lv[q4].y, uv[q4].y, wv[q4].y, n + 1);
+                    probe(lv[q4].x, uv[q4].x, wv[q4].x, n);
+                }
+            }
+        } else {
+            for (int n = n1 - 1; n >= n0; n--)
+                probe(a.x0[xb + (size_t)n * a.HW], a.x1[xb + (size_t)n * a.HW], wr[n], n);
+        }
+        if (side) posu = found; else posl = found;
+    }
+    a.y0[o] = vl; a.y1[o] = vu;
+    a.p0[o] = (int)posl; a.p1[o] = (int)posu;
+}
+
+inline int launch_resolve_bound(const FwdArgs& a, hipStream_t stream) {
+    long long total = (long long)a.R * a.G * a.COg;
+    dim3 grid((unsigned)((total + 255) / 256));
+    if (a.nsplit > 1) hipLaunchKernelGGL((resolve_bound_kernel<true>), grid, dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL((resolve_bound_kernel<false>), grid, dim3(256), 0, stream, a);
+    return check_launch("resolve_bound_kernel");
 }
 
 inline int launch_resolve(const FwdArgs& a, hipStream_t stream) {

@@ -161,6 +161,16 @@ extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* input
     SD_REQUIRE(outputL && outputU && posL && posU, "bound_inf_dist_forward: null output or pos");
     a.y0 = outputL; a.y1 = outputU; a.p0 = posL; a.p1 = posU;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (a.R <= 32) return launch_fwd<BoundPos, 2, 4>(a, st);
-    return launch_fwd<BoundPos, 4, 4>(a, st);
+    const int TB = a.R <= 32 ? 2 : 4;
+    a.nsplit = pick_nsplit(a, 16 * TB, 64);
+    if (a.nsplit > 1) {
+        size_t n = (size_t)a.R * a.G * a.COg;
+        a.packed0 = static_cast<unsigned long long*>(workspace(n * 16));
+        if (!a.packed0) return SD_ERR_HIP;
+        a.packed1 = a.packed0 + n;
+        if ((rc = fill_zero(a.packed0, n * 4, st))) return rc;
+    }
+    rc = TB == 2 ? launch_fwd<BoundChunk, 2, 4>(a, st) : launch_fwd<BoundChunk, 4, 4>(a, st);
+    if (rc) return rc;
+    return launch_resolve_bound(a, st);
 }
