@@ -41,6 +41,9 @@ struct FwdArgs {
     int* p1;              // posU
     unsigned long long* packed0;  // (value bits << 32 | ~chunk) merge buffer of split-N position kernels
     unsigned long long* packed1;  // same for the upper bound of the interval kernel
+    float* part0;         // split-N partial sums of the l-p forward, [nsplit][part_stride]
+    float* part1;         // split-N partial maxima (online form)
+    size_t part_stride;   // B * CO * HW
     const uint32_t* xmask;  // factored mask: keep bits of x rows, one word per (row, chunk), or null
     const uint32_t* wmask;  // same for w rows
     const int* ci_idx;    // (S, G, CIg) or null

@@ -167,7 +167,7 @@ __global__ void __launch_bounds__(256, P::MIN_WAVES) fwd_kernel(FwdArgs a) {
             int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
             int b = r / a.HW, hw = r - b * a.HW;
             size_t o = ((size_t)(b * a.G + g) * a.COg + m) * a.HW + hw;
-            P::init(acc[i][j], a, o, r < a.R && m < a.COg);
+            P::init(acc[i][j], a, o, r < a.R && m < a.COg, split);
         }
     }
 
@@ -212,7 +212,7 @@ __global__ void __launch_bounds__(256, P::MIN_WAVES) fwd_kernel(FwdArgs a) {
             if (r < a.R && m < a.COg) {
                 int b = r / a.HW, hw = r - b * a.HW;
                 size_t o = ((size_t)(b * a.G + g) * a.COg + m) * a.HW + hw;
-                P::store(acc[i][j], a, o);
+                P::store(acc[i][j], a, o, split);
             }
         }
     }
@@ -340,7 +340,7 @@ __global__ void __launch_bounds__(256, P::PIPE_WAVES) fwd_kernel_pipe(FwdArgs a)
         for (int j = 0; j < TM; j++) {
             int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
             size_t o = (size_t)(r * a.G + g) * a.COg + m;
-            P::init(acc[i][j], a, o, r < a.R && m < a.COg);
+            P::init(acc[i][j], a, o, r < a.R && m < a.COg, split);
         }
     }
 
@@ -389,7 +389,7 @@ __global__ void __launch_bounds__(256, P::PIPE_WAVES) fwd_kernel_pipe(FwdArgs a)
         #pragma unroll
         for (int j = 0; j < TM; j++) {
             int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
-            if (r < a.R && m < a.COg) P::store(acc[i][j], a, (size_t)(r * a.G + g) * a.COg + m);
+            if (r < a.R && m < a.COg) P::store(acc[i][j], a, (size_t)(r * a.G + g) * a.COg + m, split);
         }
     }
 }
@@ -424,7 +424,7 @@ struct LinfNograd : PolicyBase {
     static constexpr int MIN_WAVES = SD_MINW;
     static constexpr int UNROLL4 = SD_UNR;
     struct Acc { float v; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.v = kEps; }
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) { A.v = kEps; }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
                                                  const float4& w, int, int) {
         float v = A.v;
@@ -432,7 +432,7 @@ struct LinfNograd : PolicyBase {
         v = fmaxf(fmaxf(v, fabsf(x.z - w.z)), fabsf(x.w - w.w));
         A.v = v;
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
         // partial maxima are >= 1e-10 > 0, so their bit patterns order like integers
         if (a.nsplit > 1) atomicMax(reinterpret_cast<int*>(a.y0 + o), __float_as_int(A.v));
         else a.y0[o] = A.v;
@@ -444,7 +444,7 @@ struct LinfNograd : PolicyBase {
 // magnitude, so the lowest index wins ties and NaN terms never win.
 struct LinfPos : PolicyBase {
     struct Acc { float bd; int bn; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.bd = kEps; A.bn = 0; }
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) { A.bd = kEps; A.bn = 0; }
     static __device__ __forceinline__ void term(Acc& A, float x, float w, int n) {
         float d = x - w;
         if (fabsf(d) > fabsf(A.bd)) { A.bd = d; A.bn = n; }
@@ -453,7 +453,7 @@ struct LinfPos : PolicyBase {
                                                  const float4& w, int n, int) {
         term(A, x.x, w.x, n); term(A, x.y, w.y, n + 1); term(A, x.z, w.z, n + 2); term(A, x.w, w.w, n + 3);
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
         a.y0[o] = fabsf(A.bd);
         a.p0[o] = A.bn | (A.bd < 0.f ? (int)kSign : 0);
     }
@@ -481,7 +481,7 @@ struct LinfChunk : PolicyBase {
     static constexpr int MIN_WAVES = 2;
     static constexpr int UNROLL4 = 2;
     struct Acc { float best, cm; int cid; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.best = kEps; A.cm = 0.f; A.cid = -1; }
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) { A.best = kEps; A.cm = 0.f; A.cid = -1; }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
                                                  const float4& w, int, int) {
         float v = A.cm;
@@ -493,7 +493,7 @@ struct LinfChunk : PolicyBase {
         if (A.cm > A.best) { A.best = A.cm; A.cid = k0 / KT; }
         A.cm = 0.f;
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) { store_chunk_winner(a, o, A.best, A.cid); }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) { store_chunk_winner(a, o, A.best, A.cid); }
 };
 
 // the per-term masked neuron with the same chunk tracking
@@ -501,7 +501,7 @@ struct MaskedTermChunk : PolicyBase {
     static constexpr int PIPE_WAVES = 2;
     static constexpr int MIN_WAVES = 2;
     struct Acc { float best, cm; int cid; uint32_t key; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool) {
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool, int split = 0) {
         A.best = kEps; A.cm = 0.f; A.cid = -1; A.key = rng_row_key(a.seed, 0u, (uint32_t)o);
     }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
@@ -520,14 +520,14 @@ struct MaskedTermChunk : PolicyBase {
         if (A.cm > A.best) { A.best = A.cm; A.cid = k0 / KT; }
         A.cm = 0.f;
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) { store_chunk_winner(a, o, A.best, A.cid); }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) { store_chunk_winner(a, o, A.best, A.cid); }
 };
 
 // masked neuron, independent draw per term: byte (n & 3) of word(key(output), n >> 2) < t8 keeps
 template <bool POS>
 struct MaskedTerm : PolicyBase {
     struct Acc { float bd; int bn; uint32_t key; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool) {
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool, int split = 0) {
         A.bd = kEps; A.bn = 0; A.key = rng_row_key(a.seed, 0u, (uint32_t)o);
     }
     static __device__ __forceinline__ void term(Acc& A, float x, float w, int n, bool keep) {
@@ -543,7 +543,7 @@ struct MaskedTerm : PolicyBase {
         term(A, x.z, w.z, n + 2, ((word >> 16) & 0xffu) < a.t8);
         term(A, x.w, w.w, n + 3, (word >> 24) < a.t8);
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
         a.y0[o] = fabsf(A.bd);
         if (POS) a.p0[o] = A.bn | (A.bd < 0.f ? (int)kSign : 0);
     }
@@ -556,7 +556,7 @@ struct BoundNograd : PolicyBase {
     static constexpr int MIN_WAVES = SD_MINW;
     static constexpr int UNROLL4 = SD_UNR;
     struct Acc { float lo, hi; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.lo = -kEps; A.hi = kEps; }
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) { A.lo = -kEps; A.hi = kEps; }
     static __device__ __forceinline__ void term(Acc& A, float l, float u, float w) {
         float t1 = w - l, t2 = u - w;
         A.lo = fminf(fminf(A.lo, t1), t2);
@@ -566,7 +566,7 @@ struct BoundNograd : PolicyBase {
                                                  const float4& w, int, int) {
         term(A, l.x, u.x, w.x); term(A, l.y, u.y, w.y); term(A, l.z, u.z, w.z); term(A, l.w, u.w, w.w);
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
         if (a.nsplit > 1) {
             atomicMax(reinterpret_cast<int*>(a.y0 + o), __float_as_int(-A.lo));
             atomicMax(reinterpret_cast<int*>(a.y1 + o), __float_as_int(A.hi));
@@ -578,7 +578,7 @@ struct BoundNograd : PolicyBase {
 struct BoundPos : PolicyBase {
     static constexpr int NX = 2;
     struct Acc { float lo, hi; uint32_t pl, pu; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
         A.lo = -kEps; A.hi = kEps; A.pl = kNanId; A.pu = 0u;
     }
     static __device__ __forceinline__ void term(Acc& A, float l, float u, float w, int n) {
@@ -593,7 +593,7 @@ struct BoundPos : PolicyBase {
         term(A, l.x, u.x, w.x, n); term(A, l.y, u.y, w.y, n + 1);
         term(A, l.z, u.z, w.z, n + 2); term(A, l.w, u.w, w.w, n + 3);
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
         a.y0[o] = -A.lo; a.y1[o] = A.hi;
         a.p0[o] = (int)A.pl; a.p1[o] = (int)A.pu;
     }
@@ -607,7 +607,7 @@ struct BoundChunk : PolicyBase {
     static constexpr int PIPE_WAVES = 2;
     static constexpr int MIN_WAVES = 2;
     struct Acc { float lo, hi, cl, ch; int il, ih; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
         A.lo = -kEps; A.hi = kEps; A.cl = 0.f; A.ch = 0.f; A.il = -1; A.ih = -1;
     }
     static __device__ __forceinline__ void term(Acc& A, float l, float u, float w) {
@@ -624,7 +624,7 @@ struct BoundChunk : PolicyBase {
         if (A.ch > A.hi) { A.hi = A.ch; A.ih = k0 / KT; }
         A.cl = 0.f; A.ch = 0.f;
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
         store_chunk_winner(a, o, -A.lo, A.il, false);
         store_chunk_winner(a, o, A.hi, A.ih, true);
     }
@@ -664,7 +664,7 @@ __device__ __forceinline__ float geo_sum(const float (&res)[K], float q) {
 template <int K>
 struct SortNograd : PolicyBase {
     struct Acc { float res[K]; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
         #pragma unroll
         for (int k = 0; k < K; k++) A.res[k] = 0.f;
     }
@@ -676,13 +676,13 @@ struct SortNograd : PolicyBase {
                                                  const float4& w, int, int) {
         term(A, x.x, w.x); term(A, x.y, w.y); term(A, x.z, w.z); term(A, x.w, w.w);
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) { a.y0[o] = geo_sum<K>(A.res, a.q); }
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) { a.y0[o] = geo_sum<K>(A.res, a.q); }
 };
 
 template <int K>
 struct SortPos : PolicyBase {
     struct Acc { float res[K]; int idx[K]; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
         #pragma unroll
         for (int k = 0; k < K; k++) { A.res[k] = 0.f; A.idx[k] = 0; }
     }
@@ -694,7 +694,7 @@ struct SortPos : PolicyBase {
                                                  const float4& w, int n, int) {
         term(A, x.x, w.x, n); term(A, x.y, w.y, n + 1); term(A, x.z, w.z, n + 2); term(A, x.w, w.w, n + 3);
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
         a.y0[o] = geo_sum<K>(A.res, a.q);
         size_t size = (size_t)a.B * a.G * a.COg * a.HW;
         #pragma unroll
@@ -708,7 +708,7 @@ template <int K>
 struct BoundSort : PolicyBase {
     static constexpr int NX = 2;
     struct Acc { float lo[K], hi[K]; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
         #pragma unroll
         for (int k = 0; k < K; k++) { A.lo[k] = 0.f; A.hi[k] = 0.f; }
     }
@@ -722,7 +722,7 @@ struct BoundSort : PolicyBase {
                                                  const float4& w, int, int) {
         term(A, l.x, u.x, w.x); term(A, l.y, u.y, w.y); term(A, l.z, u.z, w.z); term(A, l.w, u.w, w.w);
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
         a.y0[o] = geo_sum<K>(A.lo, a.q);
         a.y1[o] = geo_sum<K>(A.hi, a.q);
     }
@@ -751,8 +751,10 @@ __device__ __forceinline__ float pow_pos(float a, float p) {
 // p <= 10: y = max(sum |d|^p, FLT_MIN)^(1/p)   (core/cuda/norm_dist_cuda.cu:163-259, no max)
 template <int IP>
 struct LpPlain : PolicyBase {
+    static constexpr int PIPE_WAVES = 3;
+    static constexpr int MIN_WAVES = 3;
     struct Acc { float s; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) { A.s = 0.f; }
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) { A.s = 0.f; }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
                                                  const float4& w, int, int) {
         A.s += pow_pos<IP>(fabsf(x.x - w.x), a.p);
@@ -760,8 +762,9 @@ struct LpPlain : PolicyBase {
         A.s += pow_pos<IP>(fabsf(x.z - w.z), a.p);
         A.s += pow_pos<IP>(fabsf(x.w - w.w), a.p);
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
-        a.y0[o] = powf(fmaxf(A.s, FLT_MIN), a.inv_p);
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
+        if (a.nsplit > 1) a.part0[(size_t)split * a.part_stride + o] = A.s;   // summed by lp_finalize_kernel
+        else a.y0[o] = powf(fmaxf(A.s, FLT_MIN), a.inv_p);
     }
 };
 
@@ -769,10 +772,13 @@ struct LpPlain : PolicyBase {
 // (core/cuda/norm_dist_cuda.cu:36-160): y = M (sum (|d|/M)^p + (1e-10/M)^p)^(1/p).
 template <int IP>
 struct LpOnline : PolicyBase {
+    static constexpr int PIPE_WAVES = 3;
+    static constexpr int MIN_WAVES = 3;
     static constexpr int PASSES = 2;
     struct Acc { float s, M, rinv, cm; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool) {
-        A.s = 1.f; A.M = kEps; A.rinv = 1.f / kEps; A.cm = 0.f;
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
+        // the virtual term of size 1e-10 (res starts at 1 relative to M = 1e-10) belongs to slice 0 only
+        A.s = split == 0 ? 1.f : 0.f; A.M = kEps; A.rinv = 1.f / kEps; A.cm = 0.f;
     }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
                                                  const float4& w, int, int pass) {
@@ -798,8 +804,11 @@ struct LpOnline : PolicyBase {
             A.cm = 0.f;
         }
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
-        a.y0[o] = powf(A.s, a.inv_p) * A.M;
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
+        if (a.nsplit > 1) {
+            a.part0[(size_t)split * a.part_stride + o] = A.s;
+            a.part1[(size_t)split * a.part_stride + o] = A.M;
+        } else a.y0[o] = powf(A.s, a.inv_p) * A.M;
     }
 };
 
@@ -807,7 +816,7 @@ struct LpOnline : PolicyBase {
 template <int IP>
 struct LpWithMax : PolicyBase {
     struct Acc { float s, rinv; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool valid) {
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool valid, int split = 0) {
         A.rinv = valid ? 1.f / a.aux[o] : 1.f;
         A.s = __builtin_amdgcn_exp2f(a.p * __builtin_amdgcn_logf(kEps * A.rinv));
     }
@@ -818,7 +827,7 @@ struct LpWithMax : PolicyBase {
         A.s += pow_pos<IP>(fabsf(x.z - w.z) * A.rinv, a.p);
         A.s += pow_pos<IP>(fabsf(x.w - w.w) * A.rinv, a.p);
     }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o) {
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
         a.y0[o] = powf(A.s, a.inv_p) / A.rinv;
     }
 };

@@ -26,6 +26,48 @@ static int launch_lp(int ip, const FwdArgs& a, hipStream_t st) {
     }
 }
 
+// merges the split-N slices of the l-p forward in slice order (deterministic) and takes the root
+__global__ void __launch_bounds__(256) lp_finalize_kernel(const float* __restrict__ part0, const float* __restrict__ part1,
+                                                          int nsplit, size_t total, float p, float inv_p,
+                                                          float* __restrict__ y) {
+    size_t o = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (o >= total) return;
+    if (part1 == nullptr) {
+        float s = 0.f;
+        for (int k = 0; k < nsplit; k++) s += part0[(size_t)k * total + o];
+        y[o] = powf(fmaxf(s, FLT_MIN), inv_p);
+    } else {
+        float M = kEps;
+        for (int k = 0; k < nsplit; k++) M = fmaxf(M, part1[(size_t)k * total + o]);
+        float s = 0.f;
+        for (int k = 0; k < nsplit; k++) {
+            float Mk = part1[(size_t)k * total + o];
+            s += part0[(size_t)k * total + o] * __builtin_amdgcn_exp2f(p * __builtin_amdgcn_logf(Mk / M));
+        }
+        y[o] = powf(s, inv_p) * M;
+    }
+}
+
+// cuts the reduction range when the output tiles alone cannot fill the device; partial sums go to the
+// library workspace and are merged by lp_finalize_kernel
+static int lp_split_setup(FwdArgs& a, int BB, int BM, bool online) {
+    a.nsplit = pick_nsplit(a, BB, BM);
+    if (a.nsplit > 1) {
+        a.part_stride = (size_t)a.R * a.G * a.COg;
+        a.part0 = static_cast<float*>(workspace(a.part_stride * a.nsplit * (online ? 2 : 1) * sizeof(float)));
+        if (!a.part0) return SD_ERR_HIP;
+        a.part1 = online ? a.part0 + a.part_stride * a.nsplit : nullptr;
+    }
+    return SD_OK;
+}
+
+static int lp_split_finish(const FwdArgs& a, hipStream_t st) {
+    if (a.nsplit <= 1) return SD_OK;
+    hipLaunchKernelGGL(lp_finalize_kernel, dim3((unsigned)((a.part_stride + 255) / 256)), dim3(256), 0, st,
+                       a.part0, a.part1, a.nsplit, a.part_stride, a.p, a.inv_p, a.y0);
+    return check_launch("lp_finalize_kernel");
+}
+
 // ---- backward -------------------------------------------------------------------------------
 // u(b,m,n) = g[b,m] sgn(d) (|d| / y[b,m])^(p-1), d = x[b,n] - w[m,n]
 // grad_x[b,n] = sum_m u,  grad_w[m,n] = - sum_b u      (core/cuda/norm_dist_cuda.cu:261-504)
@@ -45,6 +87,7 @@ struct LpBwdArgs {
     const int* ci_idx; const int* co_idx;
     int B, R, HW, G, COg, CIg, W_COg, W_CIg;
     float pm1;   // p - 1
+    int zsplit;  // slices of the channel range in the dense grad_input kernel
 };
 
 template <int IP>
@@ -166,6 +209,187 @@ __global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
     }
 }
 
+// ---- backward, dense single-group case (G == 1, HW == 1, no index lists, CI % 16 == 0) -------------
+// Two reduction-free kernels instead of the fused one: every work-item owns TN = 16 consecutive input
+// channels of ONE batch row (grad_input) or of ONE weight row (grad_weight) and walks the other
+// axis; the operand that is shared by the whole wavefront (the weight row, resp. the input row) comes in
+// through scalar loads, the per-item (g, 1/y) pair through coalesced vector loads of pre-transposed
+// copies.  No LDS, no atomics, fixed summation order (deterministic gradients).
+typedef float sfloat16 __attribute__((ext_vector_type(16)));
+constexpr int TNB = 16;
+
+__device__ __forceinline__ void sload16(sfloat16& dst, const float* base, int byte_off) {
+    asm volatile("s_load_dwordx16 %0, %1, %2" : "=s"(dst) : "s"(base), "s"(byte_off));
+}
+__device__ __forceinline__ void swait(sfloat16& v) {   // ties the wait to the value so its uses stay behind it
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(v) :: "memory");
+}
+
+// ry = 1/y in (B, M) layout and the (M, B) transposes of g and 1/y
+__global__ void __launch_bounds__(256) lp_prep_kernel(const float* __restrict__ g, const float* __restrict__ y,
+                                                      int B, int M, float* __restrict__ ry,
+                                                      float* __restrict__ gT, float* __restrict__ ryT) {
+    __shared__ float tg[32][33], tr[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
+    const int m0 = blockIdx.x * 32, b0 = blockIdx.y * 32;
+    #pragma unroll
+    for (int k = 0; k < 32; k += 8) {
+        int b = b0 + ty + k, m = m0 + tx;
+        float gv = 0.f, rv = 0.f;
+        if (b < B && m < M) {
+            gv = g[(size_t)b * M + m];
+            rv = 1.f / y[(size_t)b * M + m];
+            if (ry) ry[(size_t)b * M + m] = rv;
+        }
+        tg[ty + k][tx] = gv; tr[ty + k][tx] = rv;
+    }
+    __syncthreads();
+    #pragma unroll
+    for (int k = 0; k < 32; k += 8) {
+        int m = m0 + ty + k, b = b0 + tx;
+        if (b < B && m < M) {
+            gT[(size_t)m * B + b] = tg[tx][ty + k];
+            ryT[(size_t)m * B + b] = tr[tx][ty + k];
+        }
+    }
+}
+
+template <int IP>
+__device__ __forceinline__ void lp_bwd_accumulate(float (&acc)[TNB], const float (&own)[TNB], const sfloat16& shared,
+                                                  bool own_is_x, float gv, float rv, float pm1) {
+    #pragma unroll
+    for (int t = 0; t < TNB; t++) {
+        float d = own_is_x ? own[t] - shared[t] : shared[t] - own[t];   // always x - w
+        acc[t] = fmaf(gv, signed_pow<IP>(d, rv, pm1), acc[t]);
+    }
+}
+
+// grad_x[b, n0..n0+15] = sum_m u(b, m, n): work-item = batch row, scalar operand = weight row m
+template <int IP>
+__global__ void __launch_bounds__(256) lp_bwd_x_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                       const float* __restrict__ gT, const float* __restrict__ ryT,
+                                                       int B, int M, int N, float pm1, float* __restrict__ gx) {
+    const int n0 = blockIdx.x * TNB;
+    const int b = blockIdx.y * 256 + threadIdx.x;
+    const bool ok = b < B;
+    const int bb = ok ? b : B - 1;
+    float xr[TNB], acc[TNB];
+    #pragma unroll
+    for (int q = 0; q < TNB / 4; q++) {
+        float4 v = *reinterpret_cast<const float4*>(x + (size_t)bb * N + n0 + 4 * q);
+        xr[4 * q] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
+    }
+    #pragma unroll
+    for (int t = 0; t < TNB; t++) acc[t] = 0.f;
+    const float* wp = w + n0;
+    const int stride = N * 4;
+    // gridDim.z slices of the channel range keep enough wavefronts in flight for small batches
+    const int per = (M + gridDim.z - 1) / gridDim.z;
+    const int m_lo = blockIdx.z * per, m_hi = m_lo + per < M ? m_lo + per : M;
+    sfloat16 wa, wb;
+    sload16(wa, wp, (m_lo < M ? m_lo : 0) * stride);
+    for (int m = m_lo; m < m_hi; m += 2) {
+        float g0 = gT[(size_t)m * B + bb], r0 = ryT[(size_t)m * B + bb];
+        const bool two = m + 1 < m_hi;
+        const int m1 = two ? m + 1 : m;
+        float g1 = gT[(size_t)m1 * B + bb], r1 = ryT[(size_t)m1 * B + bb];
+        swait(wa);
+        sload16(wb, wp, m1 * stride);
+        lp_bwd_accumulate<IP>(acc, xr, wa, true, g0, r0, pm1);
+        swait(wb);
+        sload16(wa, wp, (m + 2 < m_hi ? m + 2 : m) * stride);
+        if (two) lp_bwd_accumulate<IP>(acc, xr, wb, true, g1, r1, pm1);
+    }
+    swait(wa);
+    if (ok) {
+        if (gridDim.z == 1) {
+            #pragma unroll
+            for (int q = 0; q < TNB / 4; q++)
+                *reinterpret_cast<float4*>(gx + (size_t)b * N + n0 + 4 * q) =
+                    make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+        } else {
+            #pragma unroll
+            for (int t = 0; t < TNB; t++) unsafeAtomicAdd(gx + (size_t)b * N + n0 + t, acc[t]);
+        }
+    }
+}
+
+// grad_w[m, n0..n0+15] = - sum_b u(b, m, n): work-item = weight row, scalar operand = input row b
+template <int IP>
+__global__ void __launch_bounds__(256) lp_bwd_w_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                       const float* __restrict__ g, const float* __restrict__ ry,
+                                                       int B, int M, int N, float pm1, float* __restrict__ gw) {
+    const int n0 = blockIdx.x * TNB;
+    const int m = blockIdx.y * 256 + threadIdx.x;
+    const bool ok = m < M;
+    const int mm = ok ? m : M - 1;
+    float wr[TNB], acc[TNB];
+    #pragma unroll
+    for (int q = 0; q < TNB / 4; q++) {
+        float4 v = *reinterpret_cast<const float4*>(w + (size_t)mm * N + n0 + 4 * q);
+        wr[4 * q] = v.x; wr[4 * q + 1] = v.y; wr[4 * q + 2] = v.z; wr[4 * q + 3] = v.w;
+    }
+    #pragma unroll
+    for (int t = 0; t < TNB; t++) acc[t] = 0.f;
+    const float* xp = x + n0;
+    const int stride = N * 4;
+    sfloat16 xa, xb;
+    sload16(xa, xp, 0);
+    for (int b = 0; b < B; b += 2) {
+        float g0 = g[(size_t)b * M + mm], r0 = ry[(size_t)b * M + mm];
+        const bool two = b + 1 < B;
+        const int b1 = two ? b + 1 : b;
+        float g1 = g[(size_t)b1 * M + mm], r1 = ry[(size_t)b1 * M + mm];
+        swait(xa);
+        sload16(xb, xp, b1 * stride);
+        lp_bwd_accumulate<IP>(acc, wr, xa, false, g0, r0, pm1);
+        swait(xb);
+        sload16(xa, xp, (b + 2 < B ? b + 2 : b) * stride);
+        if (two) lp_bwd_accumulate<IP>(acc, wr, xb, false, g1, r1, pm1);
+    }
+    swait(xa);
+    if (ok) {
+        #pragma unroll
+        for (int q = 0; q < TNB / 4; q++)
+            *reinterpret_cast<float4*>(gw + (size_t)m * N + n0 + 4 * q) =
+                make_float4(-acc[4 * q], -acc[4 * q + 1], -acc[4 * q + 2], -acc[4 * q + 3]);
+    }
+}
+
+template <int IP>
+static void launch_lp_bwd_dense_ip(const LpBwdArgs& a, const float* ry, const float* gT, const float* ryT, hipStream_t st) {
+    const int B = a.R, M = a.COg, N = a.CIg;
+    hipLaunchKernelGGL((lp_bwd_x_kernel<IP>), dim3(N / TNB, (B + 255) / 256, a.zsplit), dim3(256), 0, st,
+                       a.x, a.w, gT, ryT, B, M, N, a.pm1, a.gx);
+    if (a.gw)
+        hipLaunchKernelGGL((lp_bwd_w_kernel<IP>), dim3(N / TNB, (M + 255) / 256), dim3(256), 0, st,
+                           a.x, a.w, a.gy, ry, B, M, N, a.pm1, a.gw);
+}
+
+static int launch_lp_bwd_dense(int ip, const LpBwdArgs& a_in, hipStream_t st) {
+    const size_t n = (size_t)a_in.R * a_in.COg;
+    float* ws = static_cast<float*>(workspace(3 * n * sizeof(float)));
+    if (!ws) return SD_ERR_HIP;
+    float *ry = ws, *gT = ws + n, *ryT = ws + 2 * n;
+    hipLaunchKernelGGL(lp_prep_kernel, dim3((a_in.COg + 31) / 32, (a_in.R + 31) / 32), dim3(256), 0, st,
+                       a_in.gy, a_in.y, a_in.R, a_in.COg, a_in.gw ? ry : nullptr, gT, ryT);
+    int rc = check_launch("lp_prep_kernel");
+    if (rc) return rc;
+    // aim at >= 8 wavefronts per SIMD for the grad_input kernel; its slices merge with atomic adds
+    LpBwdArgs a = a_in;
+    long long waves = (long long)(a.CIg / TNB) * ((a.R + 255) / 256) * 4;
+    a.zsplit = 1;
+    while (a.zsplit < 8 && waves * a.zsplit < 8ll * 4 * num_cus() && a.COg / (a.zsplit * 2) >= 64) a.zsplit *= 2;
+    if (a.zsplit > 1 && (rc = fill_zero(a.gx, (size_t)a.R * a.CIg, st))) return rc;
+#define SD_CASE(k) case k: launch_lp_bwd_dense_ip<k>(a, ry, gT, ryT, st); break;
+    switch (ip) {
+        SD_CASE(0) SD_CASE(1) SD_CASE(2) SD_CASE(3) SD_CASE(4) SD_CASE(5) SD_CASE(6) SD_CASE(7) SD_CASE(8)
+        default: launch_lp_bwd_dense_ip<-1>(a, ry, gT, ryT, st); break;
+    }
+#undef SD_CASE
+    return check_launch("lp_bwd_x/w_kernel");
+}
+
 template <bool WGRAD>
 static int launch_lp_bwd(int ip, const LpBwdArgs& a, hipStream_t st) {
     dim3 grid((a.CIg + 255) / 256, (a.R + RB - 1) / RB, a.G);
@@ -194,6 +418,9 @@ static int lp_backward(const char* who, const float* grad_output, const float* i
     a.pm1 = p - 1.f;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int ip = int_power(p - 1.f);
+    const bool dense = G == 1 && HW == 1 && !ci_idx && !co_idx && f.CIg % TNB == 0 && aligned16(input) &&
+                       aligned16(weight) && aligned16(grad_input) && (!grad_weight || aligned16(grad_weight));
+    if (dense) return launch_lp_bwd_dense(ip, a, st);
     if (grad_weight) {
         if ((rc = fill_zero(grad_weight, (size_t)G * f.W_COg * f.W_CIg, st))) return rc;
         return launch_lp_bwd<true>(ip, a, st);
@@ -218,11 +445,16 @@ extern "C" int sd_norm_dist_forward(const float* input, const float* weight,
     a.y0 = output; a.p = p; a.inv_p = 1.f / p;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = w_index_ci || w_index_co || a.R <= 32;
-    if (p <= 10.f) {   // core/cuda/norm_dist.cpp:4,51-55
+    const bool online = p > 10.f;   // core/cuda/norm_dist.cpp:4,51-55
+    if ((rc = lp_split_setup(a, small ? 32 : 64, 128, online))) return rc;
+    if (!online) {
         int ip = int_power(p);
-        return small ? launch_lp<LpPlain, 2, 8>(ip, a, st) : launch_lp<LpPlain, 4, 8>(ip, a, st);
+        rc = small ? launch_lp<LpPlain, 2, 8>(ip, a, st) : launch_lp<LpPlain, 4, 8>(ip, a, st);
+    } else {
+        rc = small ? launch_fwd<LpOnline<-1>, 2, 8>(a, st) : launch_fwd<LpOnline<-1>, 4, 8>(a, st);
     }
-    return small ? launch_fwd<LpOnline<-1>, 2, 8>(a, st) : launch_fwd<LpOnline<-1>, 4, 8>(a, st);
+    if (rc) return rc;
+    return lp_split_finish(a, st);
 }
 
 extern "C" int sd_norm_dist_forward_with_max(const float* input, const float* weight, const float* max_output,
