@@ -15,15 +15,6 @@
 #include <stdlib.h>
 #include "common.h"
 
-#ifndef SD_MINW
-#define SD_MINW 3
-#endif
-#ifndef SD_UNR
-#define SD_UNR 1
-#endif
-#ifndef SD_PIPEW
-#define SD_PIPEW 3
-#endif
 
 namespace sd {
 
@@ -180,11 +171,7 @@ __global__ void __launch_bounds__(256, P::MIN_WAVES) fwd_kernel(FwdArgs a) {
             #pragma unroll P::UNROLL4
             for (int n4 = 0; n4 < KT; n4 += 4) {
                 float4 wv[TM];
-#ifdef SD_EXP_NOLDS
-                const int n4l = 0;
-#else
                 const int n4l = n4;
-#endif
                 #pragma unroll
                 for (int j = 0; j < TM; j++) wv[j] = *reinterpret_cast<const float4*>(&ws[tm + 16 * j][n4l]);
                 #pragma unroll
@@ -345,19 +332,10 @@ __global__ void __launch_bounds__(256, P::PIPE_WAVES) fwd_kernel_pipe(FwdArgs a)
     }
 
     if (n_begin < n_end) gload(n_begin);
-#if defined(SD_EXP1) || defined(SD_EXP2)
-    sstore(n_begin);
-    __syncthreads();
-#endif
     for (int k0 = n_begin; k0 < n_end; k0 += KT) {
-#if defined(SD_EXP1)
-        __syncthreads();
-#elif defined(SD_EXP2)
-#else
         sstore(k0);
         __syncthreads();
         if (k0 + KT < n_end) gload(k0 + KT);
-#endif
         #pragma unroll
         for (int pass = 0; pass < P::PASSES; pass++) {
             #pragma unroll P::UNROLL4
@@ -379,9 +357,7 @@ __global__ void __launch_bounds__(256, P::PIPE_WAVES) fwd_kernel_pipe(FwdArgs a)
                 for (int j = 0; j < TM; j++) P::chunk_end(acc[i][j], a, pass, k0);
             }
         }
-#if !defined(SD_EXP2)
         __syncthreads();
-#endif
     }
 
     #pragma unroll
@@ -398,8 +374,7 @@ __global__ void __launch_bounds__(256, P::PIPE_WAVES) fwd_kernel_pipe(FwdArgs a)
 template <class P, int TB, int TM>
 int launch_fwd(const FwdArgs& a, hipStream_t stream) {
     dim3 grid((a.COg + 16 * TM - 1) / (16 * TM), (a.R + 16 * TB - 1) / (16 * TB), a.G * a.nsplit);
-    static const bool use_pipe = !getenv("SD_FWD_PIPE") || atoi(getenv("SD_FWD_PIPE")) != 0;
-    if (use_pipe && a.fast_x && a.fast_w && (a.mask_mode != SD_MASK_FACTORED || a.xmask))
+    if (a.fast_x && a.fast_w && (a.mask_mode != SD_MASK_FACTORED || a.xmask))
         hipLaunchKernelGGL((fwd_kernel_pipe<P, TB, TM>), grid, dim3(256), 0, stream, a);
     else
         hipLaunchKernelGGL((fwd_kernel<P, TB, TM>), grid, dim3(256), 0, stream, a);
@@ -420,9 +395,9 @@ struct PolicyBase {
 
 // l-inf forward without indices (core/cuda/inf_dist_cuda.cu:17-107)
 struct LinfNograd : PolicyBase {
-    static constexpr int PIPE_WAVES = SD_PIPEW;
-    static constexpr int MIN_WAVES = SD_MINW;
-    static constexpr int UNROLL4 = SD_UNR;
+    static constexpr int PIPE_WAVES = 3;
+    static constexpr int MIN_WAVES = 3;
+    static constexpr int UNROLL4 = 1;
     struct Acc { float v; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) { A.v = kEps; }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
@@ -439,27 +414,8 @@ struct LinfNograd : PolicyBase {
     }
 };
 
-// l-inf forward with arg-max index and sign (core/cuda/inf_dist_cuda.cu:110-212): the signed
-// difference of the current winner is kept, a later term replaces it only if strictly larger in
-// magnitude, so the lowest index wins ties and NaN terms never win.
-struct LinfPos : PolicyBase {
-    struct Acc { float bd; int bn; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) { A.bd = kEps; A.bn = 0; }
-    static __device__ __forceinline__ void term(Acc& A, float x, float w, int n) {
-        float d = x - w;
-        if (fabsf(d) > fabsf(A.bd)) { A.bd = d; A.bn = n; }
-    }
-    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
-                                                 const float4& w, int n, int) {
-        term(A, x.x, w.x, n); term(A, x.y, w.y, n + 1); term(A, x.z, w.z, n + 2); term(A, x.w, w.w, n + 3);
-    }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
-        a.y0[o] = fabsf(A.bd);
-        a.p0[o] = A.bn | (A.bd < 0.f ? (int)kSign : 0);
-    }
-};
-
-// Same result as LinfPos at a fraction of the cost: inside a chunk of KT inputs only the maximum
+// l-inf forward with arg-max index and sign (core/cuda/inf_dist_cuda.cu:110-212), without paying for
+// index bookkeeping on every term: inside a chunk of KT inputs only the maximum
 // is kept (one subtract per term, one 3-input max per two terms); at the end of the chunk the
 // running (best, chunk index) pair is replaced only on a strictly larger maximum, so the lowest
 // chunk attaining the final value survives.  The (best, chunk) pairs of the split-N slices are
@@ -551,10 +507,10 @@ struct MaskedTerm : PolicyBase {
 
 // interval bounds, values only (core/cuda/bound_inf_dist_cuda.cu:15-118)
 struct BoundNograd : PolicyBase {
-    static constexpr int PIPE_WAVES = SD_PIPEW;
+    static constexpr int PIPE_WAVES = 3;
     static constexpr int NX = 2;
-    static constexpr int MIN_WAVES = SD_MINW;
-    static constexpr int UNROLL4 = SD_UNR;
+    static constexpr int MIN_WAVES = 3;
+    static constexpr int UNROLL4 = 1;
     struct Acc { float lo, hi; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) { A.lo = -kEps; A.hi = kEps; }
     static __device__ __forceinline__ void term(Acc& A, float l, float u, float w) {
@@ -574,32 +530,7 @@ struct BoundNograd : PolicyBase {
     }
 };
 
-// interval bounds with indices (core/cuda/bound_inf_dist_cuda.cu:121-238)
-struct BoundPos : PolicyBase {
-    static constexpr int NX = 2;
-    struct Acc { float lo, hi; uint32_t pl, pu; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
-        A.lo = -kEps; A.hi = kEps; A.pl = kNanId; A.pu = 0u;
-    }
-    static __device__ __forceinline__ void term(Acc& A, float l, float u, float w, int n) {
-        float t1 = w - l, t2 = u - w;
-        float mn = fminf(t1, t2), mx = fmaxf(t1, t2);
-        uint32_t p = (uint32_t)n | (t1 <= t2 ? 0u : kSign);
-        if (mn < A.lo) { A.lo = mn; A.pl = p; }
-        if (mx > A.hi) { A.hi = mx; A.pu = p; }
-    }
-    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& l, const float4& u,
-                                                 const float4& w, int n, int) {
-        term(A, l.x, u.x, w.x, n); term(A, l.y, u.y, w.y, n + 1);
-        term(A, l.z, u.z, w.z, n + 2); term(A, l.w, u.w, w.w, n + 3);
-    }
-    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
-        a.y0[o] = -A.lo; a.y1[o] = A.hi;
-        a.p0[o] = (int)A.pl; a.p1[o] = (int)A.pu;
-    }
-};
-
-// interval bounds with indices, chunk-tracked like LinfChunk: the lower side tracks the largest
+// interval bounds with indices (core/cuda/bound_inf_dist_cuda.cu:121-238), chunk-tracked like LinfChunk: the lower side tracks the largest
 // -min(t1,t2) (a positive number once it passes 1e-10), the upper side the largest max(t1,t2);
 // resolve_bound_kernel recovers the exact positions and branch bits
 struct BoundChunk : PolicyBase {

@@ -4,16 +4,6 @@
 
 using namespace sd;
 
-#ifndef SD_NG_TB
-#define SD_NG_TB 8
-#endif
-#ifndef SD_BD_TM
-#define SD_BD_TM 8
-#endif
-#ifndef SD_BD_TB
-#define SD_BD_TB 4
-#endif
-
 // One work-item per (row, chunk): the 32 keep bits of the factored mask for inputs
 // chunk*32 .. chunk*32+31 of an x row (stream 1) or a w row (stream 2).
 static __global__ void __launch_bounds__(256) build_masks_kernel(uint32_t* __restrict__ out, long long rows, int nchunks,
@@ -61,7 +51,7 @@ extern "C" int sd_inf_dist_forward_nograd(const float* input, const float* weigh
     SD_REQUIRE(output, "inf_dist_forward_nograd: null output");
     a.y0 = output;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int TB = a.R <= 32 ? 2 : a.R <= 64 ? 4 : SD_NG_TB;
+    const int TB = a.R <= 32 ? 2 : a.R <= 64 ? 4 : 8;
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;
     if (TB == 2) return launch_fwd<LinfNograd, 2, 8>(a, st);
@@ -140,14 +130,14 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
     SD_REQUIRE(outputL && outputU, "bound_inf_dist_forward_nograd: null output");
     a.y0 = outputL; a.y1 = outputU;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int TB = a.R <= 32 ? 2 : SD_BD_TB;
-    a.nsplit = pick_nsplit(a, 16 * TB, 16 * SD_BD_TM);
+    const int TB = a.R <= 32 ? 2 : 4;
+    a.nsplit = pick_nsplit(a, 16 * TB, 16 * 8);
     if (a.nsplit > 1) {
         if ((rc = fill_zero(outputL, (size_t)B * CO * HW, st))) return rc;
         if ((rc = fill_zero(outputU, (size_t)B * CO * HW, st))) return rc;
     }
     if (TB == 2) return launch_fwd<BoundNograd, 2, 8>(a, st);
-    return launch_fwd<BoundNograd, SD_BD_TB, SD_BD_TM>(a, st);
+    return launch_fwd<BoundNograd, 4, 8>(a, st);
 }
 
 extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* inputU, const float* weight,
