@@ -170,6 +170,17 @@ int sd_mean_shift_forward(const float* input, int B, int C, int HW, float* mean,
 int sd_channel_shift(const float* input, const float* shift, int B, int C, int HW, float sign,
                      float* output, sd_stream_t stream);
 
+/* ---- device-side mask sampling for the index-list form (replaces sample_mask,
+ * core/models/norm_dist.py:14-17, which draws on the host with a device synchronisation) ---- */
+
+/* Host-only, touches no GPU: the number of kept channels, count = #{c < C : u_c < q} with u_c from
+ * the counter RNG (the reference's (rand(C) < q).sum()). */
+int sd_mask_count(uint32_t seed, int C, float q);
+
+/* out (S, G, count) int32: for every (sub-batch, group) a uniformly random subset of exactly `count`
+ * of the C channels, ascending (the reference's sort(topk(rand(S, G, C), count).indices)). */
+int sd_sample_index_lists(uint32_t seed, int S, int G, int C, int count, int* out, sd_stream_t stream);
+
 /* The counter RNG and the thresholds it is compared with, exposed for verification. */
 uint32_t sd_rng_word(uint32_t seed, uint32_t stream_id, uint32_t row, uint32_t col);
 uint32_t sd_mask_threshold8(float q);

@@ -23,6 +23,7 @@ __all__ = [
     "bound_inf_dist_forward", "bound_inf_dist_backward",
     "sort_neuron_forward", "sort_neuron_backward", "bound_sort_neuron_forward",
     "norm_dist_forward", "norm_dist_backward", "mean_shift", "set_num_threads",
+    "mask_count", "sample_index_lists",
 ]
 
 
@@ -213,3 +214,15 @@ def mean_shift(x):
     out = np.empty_like(x)
     _load().sdo_mean_shift(_p(x), *_c_int(B, C, HW), _p(mean), _p(out))
     return out, mean
+
+
+def mask_count(seed, channels, q):
+    lib = _load()
+    lib.sdo_mask_count.restype = ctypes.c_int
+    return int(lib.sdo_mask_count(ctypes.c_uint32(seed & 0xFFFFFFFF), ctypes.c_int(channels), ctypes.c_float(q)))
+
+
+def sample_index_lists(seed, sub_batches, groups, channels, count):
+    out = np.empty((sub_batches, groups, count), np.int32)
+    _load().sdo_sample_index_lists(ctypes.c_uint32(seed & 0xFFFFFFFF), *_c_int(sub_batches, groups, channels, count), _p(out))
+    return out

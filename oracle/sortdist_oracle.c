@@ -512,3 +512,41 @@ void sdo_mean_shift(const float* x, int B, int C, int HW, float* mean, float* ou
                 out[i] = x[i] - mean[c];
             }
 }
+
+/* ------------------------------------------------------------------------------------------
+ * Mask sampling of the index-list form (core/models/norm_dist.py:14-17 restated on the counter RNG):
+ * count = #{c : word(key(3,0), c) < q 2^32}; list (s,g) = the `count` channels with the smallest
+ * 48-bit keys (word(key(4, s G + g), c) << 16) | c, ascending channel order.
+ * ---------------------------------------------------------------------------------------- */
+int sdo_mask_count(uint32_t seed, int C, float q) {
+    double t = floor((double)q * 4294967296.0 + 0.5);
+    if (t < 0) t = 0;
+    if (t > 4294967296.0) t = 4294967296.0;
+    uint64_t thr = (uint64_t)t;
+    uint32_t key = sdo_row_key(seed, 3u, 0u);
+    int n = 0;
+    for (int c = 0; c < C; c++) n += (uint64_t)sdo_word(key, (uint32_t)c) < thr;
+    return n;
+}
+
+static int sdo_cmp_u64(const void* a, const void* b) {
+    uint64_t x = *(const uint64_t*)a, y = *(const uint64_t*)b;
+    return x < y ? -1 : x > y;
+}
+
+void sdo_sample_index_lists(uint32_t seed, int S, int G, int C, int count, int* out) {
+    uint64_t* keys = (uint64_t*)malloc((size_t)C * sizeof(uint64_t));
+    uint64_t* sorted = (uint64_t*)malloc((size_t)C * sizeof(uint64_t));
+    for (int r = 0; r < S * G; r++) {
+        uint32_t rk = sdo_row_key(seed, 4u, (uint32_t)r);
+        for (int c = 0; c < C; c++) keys[c] = ((uint64_t)sdo_word(rk, (uint32_t)c) << 16) | (uint64_t)c;
+        memcpy(sorted, keys, (size_t)C * sizeof(uint64_t));
+        qsort(sorted, (size_t)C, sizeof(uint64_t), sdo_cmp_u64);
+        int k = 0;
+        if (count > 0) {
+            uint64_t last = sorted[count - 1];
+            for (int c = 0; c < C; c++) if (keys[c] <= last) out[(size_t)r * count + k++] = c;
+        }
+    }
+    free(keys); free(sorted);
+}

@@ -39,6 +39,7 @@ SIGNATURES = {
     "sd_masked_inf_dist_forward": [_F, _F, _i, _i, _i, _i, _i, _F, _I, _f, _u, _i, _S],
     "sd_mean_shift_forward": [_F, _i, _i, _i, _F, _F, _f, _F, _S],
     "sd_channel_shift": [_F, _F, _i, _i, _i, _f, _F, _S],
+    "sd_sample_index_lists": [_u, _i, _i, _i, _i, _I, _S],
 }
 _OTHER = {
     "sd_version": ([], _i),
@@ -46,6 +47,7 @@ _OTHER = {
     "sd_rng_word": ([_u, _u, _u, _u], _u),
     "sd_mask_threshold8": ([_f], _u),
     "sd_mask_threshold16": ([_f], _u),
+    "sd_mask_count": ([_u, _i, _f], _i),
 }
 
 _lib = None

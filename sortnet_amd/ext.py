@@ -176,3 +176,19 @@ def channel_shift(input, shift, sign, output):
     """output = input + sign * shift[c] (evaluation-mode mean shift, bias add)."""
     B, C, HW = input.size(0), input.size(1), input.size(2)
     _run("sd_channel_shift", input, _chk(input, "input"), _chk(shift, "shift"), B, C, HW, sign, _chk(output, "output"))
+
+
+def mask_count(seed, channels, q):
+    """Number of kept channels for keep probability q (host arithmetic only, no GPU work)."""
+    return int(_lib.load().sd_mask_count(seed & 0xFFFFFFFF, channels, q))
+
+
+def sample_index_lists(seed, sub_batches, groups, channels, count, device):
+    """(sub_batches, groups, count) int32 tensor of ascending kept-channel indices, drawn on the
+    device from the counter RNG (the reference's sample_mask without its host synchronisation)."""
+    out = torch.empty(sub_batches, groups, count, device=device, dtype=torch.int32)
+    if count > 0:
+        with torch.cuda.device(out.device):
+            _lib.call("sd_sample_index_lists", seed & 0xFFFFFFFF, sub_batches, groups, channels, count,
+                      out.data_ptr(), torch.cuda.current_stream(out.device).cuda_stream)
+    return out

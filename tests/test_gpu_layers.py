@@ -1,0 +1,130 @@
+"""GPU tests of the layer callers (sortnet_amd.layers) and of the device-side mask sampler:
+a small stack is run in the three modes of the reference's NormDistBase.forward and compared with
+the same computation composed from oracle calls."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+@pytest.mark.parametrize("S,G,C,q", [(3, 1, 100, 0.3), (2, 2, 64, 0.75), (16, 1, 5120, 0.3), (1, 1, 7, 1.0)])
+def test_sampler_matches_oracle(oracle, S, G, C, q):
+    from sortnet_amd import ext
+    dev = _dev()
+    for seed in (0, 12345):
+        count = ext.mask_count(seed, C, q)
+        assert count == oracle.mask_count(seed, C, q)
+        assert abs(count - q * C) <= 6 * np.sqrt(C * q * (1 - q)) + 1
+        idx = ext.sample_index_lists(seed, S, G, C, count, dev).cpu().numpy()
+        ref = oracle.sample_index_lists(seed, S, G, C, count)
+        assert np.array_equal(idx, ref)
+        assert idx.shape == (S, G, count) and (np.diff(idx, axis=-1) > 0).all() and idx.min() >= 0 and idx.max() < C
+    if S > 1 and 0 < count < C:
+        assert not np.array_equal(idx[0], idx[1])    # sub-batches get different subsets
+
+
+def test_plain_stack_value_and_bounds(oracle):
+    from sortnet_amd.layers import NormDist, BoundSequential, DropoutRegistry
+    dev = _dev()
+    reg = DropoutRegistry()
+    torch.manual_seed(0)
+    net = BoundSequential(NormDist(48, 64, bias=False, std=0.2, registry=reg),
+                          NormDist(64, 10, bias=True, mean_shift=False, std=0.2, registry=reg)).to(dev)
+    x = torch.rand(40, 48, device=dev)
+    eps = 0.02
+    net.train()
+    y, _, _ = net((x, None, None))
+    w0, w1 = net[0].weight.detach().cpu().numpy(), net[1].weight.detach().cpu().numpy()
+    h = oracle.inf_dist_forward(x.cpu().numpy()[:, :, None], w0, need_pos=False)
+    h, mean = oracle.mean_shift(h)
+    ref = oracle.inf_dist_forward(h, w1, need_pos=False)[:, :, 0]
+    np.testing.assert_allclose(y.detach().cpu().numpy(), ref, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(net[0].mean_shift.running_mean.cpu().numpy(), 0.1 * mean, rtol=1e-5, atol=1e-7)
+    y.sum().backward()
+    assert net[0].weight.grad is not None and torch.isfinite(net[0].weight.grad).all()
+    net.eval()
+    with torch.no_grad():
+        v, lo, up = net((x, x - eps, x + eps))
+    rm = net[0].mean_shift.running_mean.cpu().numpy()
+    xl, xu = (x - eps).cpu().numpy()[:, :, None], (x + eps).cpu().numpy()[:, :, None]
+    l1, u1 = oracle.bound_inf_dist_forward(xl, xu, w0, need_pos=False)
+    l2, u2 = oracle.bound_inf_dist_forward(l1 - rm[None, :, None], u1 - rm[None, :, None], w1, need_pos=False)
+    np.testing.assert_allclose(lo.cpu().numpy(), l2[:, :, 0], rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(up.cpu().numpy(), u2[:, :, 0], rtol=1e-6, atol=1e-6)
+    assert bool((lo <= v + 1e-6).all()) and bool((v <= up + 1e-6).all())
+
+
+def test_index_list_training_and_sort_eval(oracle):
+    from sortnet_amd.layers import NormDist, BoundSequential, DropoutRegistry, set_mask_seed
+    dev = _dev()
+    reg = DropoutRegistry()
+    torch.manual_seed(1)
+    q = 0.6
+    net = BoundSequential(NormDist(40, 96, bias=False, std=0.2, registry=reg),
+                          NormDist(96, 64, bias=False, std=0.2, dropout=q, registry=reg),
+                          NormDist(64, 10, bias=True, mean_shift=False, std=0.2, dropout=q, registry=reg)).to(dev)
+    x = torch.rand(70, 40, device=dev)
+    set_mask_seed(7, reg)
+    net.train()
+    y, _, _ = net((x, None, None))
+    y.sum().backward()
+    for m in net:
+        assert m.weight.grad is not None and torch.isfinite(m.weight.grad).all()
+    # recompute with the oracle: layer 0 drops outputs (= inputs of layer 1), layer 1 drops outputs too
+    S = 3
+    seeds = [(7 * 1000003 + d) & 0xFFFFFFFF for d in (1, 2)]
+    c1 = oracle.mask_count(seeds[0], 96, q)
+    i1 = oracle.sample_index_lists(seeds[0], S, 1, 96, c1)
+    c2 = oracle.mask_count(seeds[1], 64, q)
+    i2 = oracle.sample_index_lists(seeds[1], S, 1, 64, c2)
+    w = [m.weight.detach().cpu().numpy() for m in net]
+    rows = np.arange(70) // 32
+
+    def index_mean_shift(h, idx, channels):
+        tot, cnt = np.zeros(channels), np.full(channels, 1e-10)
+        for b in range(h.shape[0]):
+            tot[idx[rows[b], 0]] += h[b, :, 0]
+            cnt[idx[rows[b], 0]] += 1
+        mean = (tot / cnt).astype(np.float32)
+        return h - mean[idx[rows, 0]][:, :, None]
+
+    h0 = oracle.inf_dist_forward(x.cpu().numpy()[:, :, None], w[0], 1, False, None, i1)
+    h0 = index_mean_shift(h0, i1, 96)
+    h1 = oracle.inf_dist_forward(h0, w[1], 1, False, i1, i2)
+    h1 = index_mean_shift(h1, i2, 64)
+    h2 = oracle.inf_dist_forward(h1, w[2], 1, False, i2, None)
+    np.testing.assert_allclose(y.detach().cpu().numpy(), h2[:, :, 0], rtol=2e-5, atol=2e-6)
+    # evaluation mode: sort neuron for the value, its interval version for the bounds
+    net.eval()
+    eps = 0.01
+    with torch.no_grad():
+        v, lo, up = net((x, x - eps, x + eps))
+    rm = [m.mean_shift.running_mean.cpu().numpy() if m.mean_shift is not None else None for m in net]
+    xv = x.cpu().numpy()[:, :, None]
+    a = oracle.inf_dist_forward(xv, w[0], need_pos=False) - rm[0][None, :, None]
+    a = oracle.sort_neuron_forward(a, w[1], q, 10, need_pos=False) - rm[1][None, :, None]
+    a = oracle.sort_neuron_forward(a, w[2], q, 10, need_pos=False)
+    np.testing.assert_allclose(v.cpu().numpy(), a[:, :, 0], rtol=1e-5, atol=1e-6)
+    assert bool((lo <= v + 1e-5).all()) and bool((v <= up + 1e-5).all())
+
+
+def test_conv_layer_shapes_and_value(oracle):
+    from sortnet_amd.layers import NormDistConv, DropoutRegistry
+    dev = _dev()
+    torch.manual_seed(2)
+    layer = NormDistConv(3, 8, 3, stride=2, bias=False, mean_shift=False, std=0.3, registry=DropoutRegistry()).to(dev)
+    x = torch.rand(4, 3, 9, 9, device=dev)
+    with torch.no_grad():
+        y, lo, up = layer(x, x - 0.01, x + 0.01)
+    assert y.shape == (4, 8, 4, 4) and lo.shape == y.shape
+    cols = torch.nn.functional.unfold(x, 3, stride=2).cpu().numpy()          # (4, 27, 16)
+    ref = oracle.inf_dist_forward(cols, layer.weight.detach().cpu().numpy(), need_pos=False)
+    assert np.array_equal(y.cpu().numpy().reshape(4, 8, 16), ref)
+    assert bool((lo <= y).all()) and bool((y <= up).all())
