@@ -40,14 +40,29 @@ inline int make_fwd_args(FwdArgs& a, const char* who, const float* x0, const flo
     return SD_OK;
 }
 
-// how many slices to cut the reduction range in so that the grid covers the device a few times
+// how many slices to cut the reduction range in so that the grid covers the device a few times;
+// a slice keeps at least four LDS chunks (128 inputs)
 inline int pick_nsplit(const FwdArgs& a, int BB, int BM) {
     long long tiles = (long long)((a.R + BB - 1) / BB) * ((a.COg + BM - 1) / BM) * a.G;
     int chunks = (a.CIg + 31) / 32;
     long long want = 4ll * num_cus();
+    int max_ns = chunks / 4;
+    if (max_ns > 16) max_ns = 16;
     int ns = 1;
-    while (ns < 16 && tiles * ns < want && chunks / (ns * 2) >= 8) ns *= 2;
+    while (ns * 2 <= max_ns && tiles * ns < want) ns *= 2;
     return ns;
+}
+
+// rows per work-item (batch tile = 16 * TB rows): the largest candidate whose tiles, after split-N,
+// still give the device about four workgroups per compute unit; small problems fall to the smallest
+inline int pick_tb(const FwdArgs& a, const int* candidates, int n, int BM) {
+    for (int k = 0; k < n; k++) {
+        int BB = 16 * candidates[k];
+        if (a.R <= BB / 2 && k + 1 < n) continue;   // tile mostly padding
+        long long tiles = (long long)((a.R + BB - 1) / BB) * ((a.COg + BM - 1) / BM) * a.G;
+        if (tiles * pick_nsplit(a, BB, BM) >= 4ll * num_cus()) return candidates[k];
+    }
+    return candidates[n - 1];
 }
 
 }  // namespace sd

@@ -27,7 +27,8 @@ static __global__ void __launch_bounds__(256) build_masks_kernel(uint32_t* __res
 template <class P>
 static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st) {
     // with index lists a batch tile must stay inside one 32-sample sub-batch
-    const int TB = (index_lists || a.R <= 32) ? 2 : 4;
+    static const int kTb42[] = {4, 2};
+    const int TB = index_lists ? 2 : pick_tb(a, kTb42, 2, 128);
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     int rc;
     if (a.nsplit > 1) {
@@ -51,7 +52,8 @@ extern "C" int sd_inf_dist_forward_nograd(const float* input, const float* weigh
     SD_REQUIRE(output, "inf_dist_forward_nograd: null output");
     a.y0 = output;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int TB = a.R <= 32 ? 2 : a.R <= 64 ? 4 : 8;
+    static const int kTb842[] = {8, 4, 2};
+    const int TB = pick_tb(a, kTb842, 3, 128);
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;
     if (TB == 2) return launch_fwd<LinfNograd, 2, 8>(a, st);
@@ -111,7 +113,8 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
         a.xmask = xm; a.wmask = wm;
     }
     if (pos) return run_chunk_pos<LinfChunk>(a, false, st);
-    const int TB = a.R <= 32 ? 2 : a.R <= 64 ? 4 : 8;
+    static const int kTb842[] = {8, 4, 2};
+    const int TB = pick_tb(a, kTb842, 3, 128);
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;
     if (TB == 2) return launch_fwd<LinfNograd, 2, 8>(a, st);
@@ -130,7 +133,8 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
     SD_REQUIRE(outputL && outputU, "bound_inf_dist_forward_nograd: null output");
     a.y0 = outputL; a.y1 = outputU;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int TB = a.R <= 32 ? 2 : 4;
+    static const int kTb42[] = {4, 2};
+    const int TB = pick_tb(a, kTb42, 2, 128);
     a.nsplit = pick_nsplit(a, 16 * TB, 16 * 8);
     if (a.nsplit > 1) {
         if ((rc = fill_zero(outputL, (size_t)B * CO * HW, st))) return rc;
@@ -151,7 +155,8 @@ extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* input
     SD_REQUIRE(outputL && outputU && posL && posU, "bound_inf_dist_forward: null output or pos");
     a.y0 = outputL; a.y1 = outputU; a.p0 = posL; a.p1 = posU;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int TB = a.R <= 32 ? 2 : 4;
+    static const int kTb42[] = {4, 2};
+    const int TB = pick_tb(a, kTb42, 2, 64);
     a.nsplit = pick_nsplit(a, 16 * TB, 64);
     if (a.nsplit > 1) {
         size_t n = (size_t)a.R * a.G * a.COg;

@@ -444,7 +444,8 @@ extern "C" int sd_norm_dist_forward(const float* input, const float* weight,
     SD_REQUIRE(p > 0.f && !std::isinf(p), "norm_dist_forward: p=%g must be positive and finite", (double)p);
     a.y0 = output; a.p = p; a.inv_p = 1.f / p;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const bool small = w_index_ci || w_index_co || a.R <= 32;
+    static const int kTb42[] = {4, 2};
+    const bool small = w_index_ci || w_index_co || pick_tb(a, kTb42, 2, 128) == 2;
     const bool online = p > 10.f;   // core/cuda/norm_dist.cpp:4,51-55
     if ((rc = lp_split_setup(a, small ? 32 : 64, 128, online))) return rc;
     if (!online) {
