@@ -15,6 +15,16 @@
 #include <stdlib.h>
 #include "common.h"
 
+#ifndef SD_MT_WAVES
+#define SD_MT_WAVES 2
+#endif
+#ifndef SD_MT_TB
+#define SD_MT_TB 4
+#endif
+#ifndef SD_MT_TM
+#define SD_MT_TM 8
+#endif
+
 
 namespace sd {
 
@@ -390,6 +400,7 @@ struct PolicyBase {
     static constexpr int MIN_WAVES = 1;   // waves per SIMD the register budget must allow
     static constexpr int PIPE_WAVES = 2;  // same for the pipelined kernel
     static constexpr int UNROLL4 = 2;     // unroll factor of the loop over groups of four inputs
+    static constexpr int WIDE_TB = 4, WIDE_TM = 8;   // register tile of the large-batch launch of position kernels
     template <class A> static __device__ __forceinline__ void chunk_end(A&, const FwdArgs&, int, int) {}
 };
 
@@ -454,8 +465,9 @@ struct LinfChunk : PolicyBase {
 
 // the per-term masked neuron with the same chunk tracking
 struct MaskedTermChunk : PolicyBase {
-    static constexpr int PIPE_WAVES = 2;
-    static constexpr int MIN_WAVES = 2;
+    static constexpr int WIDE_TB = SD_MT_TB, WIDE_TM = SD_MT_TM;
+    static constexpr int PIPE_WAVES = SD_MT_WAVES;
+    static constexpr int MIN_WAVES = SD_MT_WAVES;
     struct Acc { float best, cm; int cid; uint32_t key; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool, int split = 0) {
         A.best = kEps; A.cm = 0.f; A.cid = -1; A.key = rng_row_key(a.seed, 0u, (uint32_t)o);
@@ -479,29 +491,30 @@ struct MaskedTermChunk : PolicyBase {
     static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) { store_chunk_winner(a, o, A.best, A.cid); }
 };
 
-// masked neuron, independent draw per term: byte (n & 3) of word(key(output), n >> 2) < t8 keeps
-template <bool POS>
-struct MaskedTerm : PolicyBase {
-    struct Acc { float bd; int bn; uint32_t key; };
+// masked neuron without positions, independent draw per term: byte (n & 3) of
+// word(key(output), n >> 2) < t8 keeps; dropped terms enter the maximum as 0
+struct MaskedTermMax : PolicyBase {
+    static constexpr int PIPE_WAVES = SD_MT_WAVES;
+    static constexpr int MIN_WAVES = SD_MT_WAVES;
+    struct Acc { float v; uint32_t key; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool, int split = 0) {
-        A.bd = kEps; A.bn = 0; A.key = rng_row_key(a.seed, 0u, (uint32_t)o);
-    }
-    static __device__ __forceinline__ void term(Acc& A, float x, float w, int n, bool keep) {
-        float d = x - w;
-        if (POS) { if (keep && fabsf(d) > fabsf(A.bd)) { A.bd = d; A.bn = n; } }
-        else A.bd = fmaxf(A.bd, keep ? fabsf(d) : 0.f);
+        A.v = kEps; A.key = rng_row_key(a.seed, 0u, (uint32_t)o);
     }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
                                                  const float4& w, int n, int) {
         uint32_t word = rng_word(A.key, (uint32_t)n >> 2);
-        term(A, x.x, w.x, n, (word & 0xffu) < a.t8);
-        term(A, x.y, w.y, n + 1, ((word >> 8) & 0xffu) < a.t8);
-        term(A, x.z, w.z, n + 2, ((word >> 16) & 0xffu) < a.t8);
-        term(A, x.w, w.w, n + 3, (word >> 24) < a.t8);
+        float d0 = (word & 0xffu) < a.t8 ? x.x - w.x : 0.f;
+        float d1 = ((word >> 8) & 0xffu) < a.t8 ? x.y - w.y : 0.f;
+        float d2 = ((word >> 16) & 0xffu) < a.t8 ? x.z - w.z : 0.f;
+        float d3 = (word >> 24) < a.t8 ? x.w - w.w : 0.f;
+        float v = A.v;
+        v = fmaxf(fmaxf(v, fabsf(d0)), fabsf(d1));
+        v = fmaxf(fmaxf(v, fabsf(d2)), fabsf(d3));
+        A.v = v;
     }
     static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
-        a.y0[o] = fabsf(A.bd);
-        if (POS) a.p0[o] = A.bn | (A.bd < 0.f ? (int)kSign : 0);
+        if (a.nsplit > 1) atomicMax(reinterpret_cast<int*>(a.y0 + o), __float_as_int(A.v));
+        else a.y0[o] = A.v;
     }
 };
 

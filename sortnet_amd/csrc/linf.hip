@@ -29,7 +29,7 @@ static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st) {
     // with index lists a batch tile must stay inside one 32-sample sub-batch
     static const int kTb42[] = {4, 2};
     const int TB = index_lists ? 2 : pick_tb(a, kTb42, 2, 128);
-    a.nsplit = pick_nsplit(a, 16 * TB, 128);
+    a.nsplit = TB == 2 ? pick_nsplit(a, 32, 128) : pick_nsplit(a, 16 * P::WIDE_TB, 16 * P::WIDE_TM);
     int rc;
     if (a.nsplit > 1) {
         // the merge buffer sits at the start of the workspace; a factored-mask call has already sized
@@ -39,7 +39,8 @@ static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st) {
         if (!a.packed0) return SD_ERR_HIP;
         if ((rc = fill_zero(a.packed0, n * 2, st))) return rc;
     }
-    rc = TB == 2 ? launch_fwd<P, 2, 8>(a, st) : launch_fwd<P, 4, 8>(a, st);
+    if (TB == 2) rc = launch_fwd<P, 2, 8>(a, st);
+    else rc = launch_fwd<P, P::WIDE_TB, P::WIDE_TM>(a, st);
     if (rc) return rc;
     return launch_resolve(a, st);
 }
@@ -91,7 +92,10 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (mode == SD_MASK_TERM) {
         if (pos) return run_chunk_pos<MaskedTermChunk>(a, false, st);
-        return small ? launch_fwd<MaskedTerm<false>, 2, 8>(a, st) : launch_fwd<MaskedTerm<false>, 4, 8>(a, st);
+        const int TBm = small ? 2 : SD_MT_TB;
+        a.nsplit = pick_nsplit(a, 16 * TBm, small ? 128 : 16 * SD_MT_TM);
+        if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;
+        return small ? launch_fwd<MaskedTermMax, 2, 8>(a, st) : launch_fwd<MaskedTermMax, SD_MT_TB, SD_MT_TM>(a, st);
     }
     // factored mask: dropped inputs / weights are replaced by NaN while staging the tiles and
     // NaN terms never win the maximum, so the plain l-inf policies apply unchanged.  On the
