@@ -366,7 +366,7 @@ def test_full_size_properties():
     assert torch.equal(y, y2)
     idx = (pos & 0x7FFFFFFF).long().squeeze(-1)
     xv = torch.gather(x.squeeze(-1), 1, idx)
-    wv = torch.gather(w.t().contiguous(), 0, idx.clamp(max=N - 1)) if False else w[torch.arange(M, device=dev)[None, :], idx]
+    wv = w[torch.arange(M, device=dev)[None, :], idx]
     d = xv - wv
     assert torch.equal(d.abs(), y.squeeze(-1))
     assert torch.equal(d < 0, (pos.squeeze(-1) < 0))
