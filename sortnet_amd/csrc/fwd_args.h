@@ -40,12 +40,14 @@ inline int make_fwd_args(FwdArgs& a, const char* who, const float* x0, const flo
     return SD_OK;
 }
 
-// how many slices to cut the reduction range in so that the grid covers the device a few times;
-// a slice keeps at least four LDS chunks (128 inputs)
+// how many slices to cut the reduction range in.  A compute unit holds two to four of these
+// workgroups at a time and a workgroup runs about as long alone as with neighbours, so the last,
+// partly filled round of workgroups costs a full round: eight workgroups per compute unit keep that
+// tail below a fifth of the run.  A slice keeps at least four LDS chunks (128 inputs).
 inline int pick_nsplit(const FwdArgs& a, int BB, int BM) {
     long long tiles = (long long)((a.R + BB - 1) / BB) * ((a.COg + BM - 1) / BM) * a.G;
     int chunks = (a.CIg + 31) / 32;
-    long long want = 4ll * num_cus();
+    long long want = 8ll * num_cus();
     int max_ns = chunks / 4;
     if (max_ns > 16) max_ns = 16;
     int ns = 1;
