@@ -582,7 +582,7 @@ template <int K>
 __device__ __forceinline__ void topk_insert_values(float (&res)[K], float v) {
     #pragma unroll
     for (int k = 0; k < K - 1; k++) res[k] = __builtin_amdgcn_fmed3f(res[k], v, res[k + 1]);
-    res[K - 1] = fmaxf(res[K - 1], v);
+    res[K - 1] = __builtin_amdgcn_fmed3f(res[K - 1], v, __builtin_inff());   // max without the NaN-quieting moves of fmaxf
 }
 template <int K>
 __device__ __forceinline__ void topk_insert(float (&res)[K], int (&idx)[K], float v, int p) {

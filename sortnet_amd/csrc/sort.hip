@@ -16,6 +16,12 @@ static int check_qk(const char* who, float q, int K, int CIg) {
     return SD_OK;
 }
 
+// few output tiles: 16 x 32 tiles instead of 32 x 64 (the top-K lists do not merge across a split reduction)
+static bool few_tiles(const FwdArgs& a, int BB, int BM) {
+    long long tiles = (long long)((a.R + BB - 1) / BB) * ((a.COg + BM - 1) / BM) * a.G;
+    return tiles < 2ll * num_cus();
+}
+
 extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* weight,
                                              int B, int CO, int CI, int G, int HW, float* output, float q, int K,
                                              sd_stream_t stream) {
@@ -26,8 +32,9 @@ extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* we
     SD_REQUIRE(output, "sort_neuron_forward_nograd: null output");
     a.y0 = output; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool small = few_tiles(a, 32, 64);
     switch (K) {
-#define X(k) case k: return launch_fwd<SortNograd<k>, 2, 4>(a, st);
+#define X(k) case k: return small ? launch_fwd<SortNograd<k>, 1, 2>(a, st) : launch_fwd<SortNograd<k>, 2, 4>(a, st);
         SD_FOR_EACH_K(X)
 #undef X
     }
@@ -45,8 +52,9 @@ extern "C" int sd_sort_neuron_forward(const float* input, const float* weight,
     SD_REQUIRE((long long)K * B * CO * HW < (1ll << 31), "sort_neuron_forward: pos too large for 32-bit indexing");
     a.y0 = output; a.p0 = pos; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool small = few_tiles(a, 32, 32);
     switch (K) {
-#define X(k) case k: return launch_fwd<SortPos<k>, 2, 2>(a, st);
+#define X(k) case k: return small ? launch_fwd<SortPos<k>, 1, 2>(a, st) : launch_fwd<SortPos<k>, 2, 2>(a, st);
         SD_FOR_EACH_K(X)
 #undef X
     }
@@ -64,8 +72,9 @@ extern "C" int sd_bound_sort_neuron_forward(const float* inputL, const float* in
     SD_REQUIRE(outputL && outputU, "bound_sort_neuron_forward: null output");
     a.y0 = outputL; a.y1 = outputU; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool small = few_tiles(a, 32, 32);
     switch (K) {
-#define X(k) case k: return launch_fwd<BoundSort<k>, 2, 2>(a, st);
+#define X(k) case k: return small ? launch_fwd<BoundSort<k>, 1, 2>(a, st) : launch_fwd<BoundSort<k>, 2, 2>(a, st);
         SD_FOR_EACH_K(X)
 #undef X
     }
