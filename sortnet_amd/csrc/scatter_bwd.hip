@@ -1,7 +1,8 @@
 // Backward of the arg-max style ops (l-inf, sort neuron, interval bounds): every output sends its
 // upstream gradient to the saved input position(s) of grad_input and grad_weight
 // (core/cuda/inf_dist_cuda.cu:214-271, sort_neuron.cu:316-375, bound_inf_dist_cuda.cu:240-299).
-// Both targets are zero-filled here and accumulated with hardware fp32 atomic adds.
+// Dense layers accumulate both gradients in LDS row histograms and write every row once; index lists and
+// very long rows fall back to a zero-fill pass and hardware fp32 atomic adds on device memory.
 #include <cmath>
 #include "common.h"
 
@@ -149,6 +150,65 @@ __global__ void __launch_bounds__(256) bound_bwd_rows_kernel(BwdArgs a) {
     }
 }
 
+// grad_weight by rows (dense layers, no index lists): one workgroup owns WR consecutive weight rows,
+// accumulates in LDS whatever any (sample, position, slot) sends into them and writes the rows out once, so
+// grad_weight needs neither a zero-fill pass nor global atomics.  Work-item = (row j = tid % WR, batch rows
+// tid / WR + i * 256 / WR): the WR positions of one batch row are adjacent in memory when HW == 1.
+// MODE 0: l-inf, 1: sort neuron (K slots, geometric coefficients), 2: interval bounds (two positions).
+constexpr int kMaxWRowsLds = 15360;   // floats of LDS the weight-row histograms of one workgroup may take
+
+template <int MODE>
+__global__ void __launch_bounds__(256) wrows_bwd_kernel(BwdArgs a, int WR) {
+    extern __shared__ float hist[];             // [WR][CIg]
+    const int CO = a.G * a.COg;
+    const int c0 = blockIdx.x * WR;
+    const int nrows = CO - c0 < WR ? CO - c0 : WR;
+    for (int n = threadIdx.x; n < WR * a.CIg; n += 256) hist[n] = 0.f;
+    __syncthreads();
+    const int j = threadIdx.x % WR, rstep = 256 / WR;
+    const int R = a.B * a.HW;
+    if (j < nrows) {
+        float* h = hist + (size_t)j * a.CIg;
+        for (int r = threadIdx.x / WR; r < R; r += rstep) {
+            int b = r, hw = 0;
+            if (a.HW > 1) { b = r / a.HW; hw = r - b * a.HW; }
+            const size_t o = ((size_t)b * CO + c0 + j) * a.HW + hw;
+            if (MODE == 2) {
+                int pl = a.p0[o], pu = a.p1[o];
+                float gl = a.g0[o], gu = a.g1[o];
+                if ((uint32_t)pl != kNanId) atomicAdd(&h[pl & 0x7fffffff], pl >= 0 ? -gl : gl);
+                atomicAdd(&h[pu & 0x7fffffff], pu >= 0 ? -gu : gu);
+            } else {
+                const float grad = a.g0[o];
+                float coef = a.coef0;
+                const int K = MODE == 1 ? a.K : 1;
+                for (int k = 0; k < K; k++) {
+                    int pr = a.p0[(size_t)k * a.total + o];
+                    float v = pr >= 0 ? grad : -grad;
+                    if (MODE == 1) { v = v * coef * a.q; coef *= 1.f - a.q; }
+                    atomicAdd(&h[pr & 0x7fffffff], -v);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    float* out = a.gw + (size_t)c0 * a.CIg;
+    for (int n = threadIdx.x; n < nrows * a.CIg; n += 256) out[n] = hist[n];
+}
+
+// launches wrows_bwd_kernel when the layer is dense and a row fits; returns false when the caller has to
+// take the zero-fill + atomics path for grad_weight
+template <int MODE>
+static bool launch_wrows(const BwdArgs& a, hipStream_t st) {
+    if (a.ci_idx || a.co_idx || a.CIg > kMaxWRowsLds) return false;
+    int WR = 1;
+    while (WR < 8 && 2 * WR * a.CIg <= kMaxWRowsLds) WR *= 2;
+    const int CO = a.G * a.COg;
+    hipLaunchKernelGGL((wrows_bwd_kernel<MODE>), dim3((unsigned)((CO + WR - 1) / WR)), dim3(256),
+                       (size_t)WR * a.CIg * sizeof(float), st, a, WR);
+    return true;
+}
+
 static int make_bwd_args(BwdArgs& a, const char* who, int B, int CO, int CI, int G, int HW,
                          const int* ci_idx, const int* co_idx, int W_CO, int W_CI) {
     SD_REQUIRE(B > 0 && CO > 0 && CI > 0 && G > 0 && HW > 0, "%s: sizes must be positive", who);
@@ -170,18 +230,25 @@ static int make_bwd_args(BwdArgs& a, const char* who, int B, int CO, int CI, int
 template <bool SORT>
 static int run_scatter(BwdArgs& a, hipStream_t st) {
     int rc;
-    if (a.gw && (rc = fill_zero(a.gw, (size_t)a.G * a.W_COg * a.W_CIg, st))) return rc;
+    float* gw_atomic = a.gw;      // grad_weight target of the atomics path, null once the row kernel has taken it
+    if (a.gw && launch_wrows<SORT ? 1 : 0>(a, st)) {
+        if ((rc = check_launch("wrows_bwd_kernel"))) return rc;
+        gw_atomic = nullptr;
+    }
+    if (gw_atomic && (rc = fill_zero(gw_atomic, (size_t)a.G * a.W_COg * a.W_CIg, st))) return rc;
+    BwdArgs x = a;
+    x.gw = gw_atomic;
     if (a.CIg <= kMaxRowLds) {
         dim3 rows((unsigned)(a.B * a.G * a.HW));
         size_t lds = (size_t)a.CIg * sizeof(float);
-        if (a.gw) hipLaunchKernelGGL((scatter_bwd_rows_kernel<SORT, true>), rows, dim3(256), lds, st, a);
-        else hipLaunchKernelGGL((scatter_bwd_rows_kernel<SORT, false>), rows, dim3(256), lds, st, a);
+        if (x.gw) hipLaunchKernelGGL((scatter_bwd_rows_kernel<SORT, true>), rows, dim3(256), lds, st, x);
+        else hipLaunchKernelGGL((scatter_bwd_rows_kernel<SORT, false>), rows, dim3(256), lds, st, x);
         return check_launch("scatter_bwd_rows_kernel");
     }
     if ((rc = fill_zero(a.gx0, (size_t)a.B * a.G * a.CIg * a.HW, st))) return rc;
     dim3 grid((unsigned)((a.total + 255) / 256));
-    if (a.gw) hipLaunchKernelGGL((scatter_bwd_kernel<SORT, true>), grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((scatter_bwd_kernel<SORT, false>), grid, dim3(256), 0, st, a);
+    if (x.gw) hipLaunchKernelGGL((scatter_bwd_kernel<SORT, true>), grid, dim3(256), 0, st, x);
+    else hipLaunchKernelGGL((scatter_bwd_kernel<SORT, false>), grid, dim3(256), 0, st, x);
     return check_launch("scatter_bwd_kernel");
 }
 
@@ -249,6 +316,10 @@ static int bound_bwd(const char* who, const float* gL, const float* gU, const in
     a.g0 = gL; a.g1 = gU; a.p0 = posL; a.p1 = posU; a.gx0 = gxL; a.gx1 = gxU; a.gw = gw;
     hipStream_t st = static_cast<hipStream_t>(stream);
     size_t nx = (size_t)B * CI * HW;
+    if (gw && launch_wrows<2>(a, st)) {
+        if ((rc = check_launch("wrows_bwd_kernel"))) return rc;
+        a.gw = gw = nullptr;
+    }
     if (gw && (rc = fill_zero(gw, (size_t)CO * a.CIg, st))) return rc;
     if (2 * a.CIg <= kMaxRowLds) {
         dim3 rows((unsigned)(B * G * HW));
