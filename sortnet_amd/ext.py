@@ -178,6 +178,11 @@ def channel_shift(input, shift, sign, output):
     _run("sd_channel_shift", input, _chk(input, "input"), _chk(shift, "shift"), B, C, HW, sign, _chk(output, "output"))
 
 
+def rng_word(seed, stream, row, col):
+    """One 32-bit word of the library's counter RNG (host arithmetic; the kernels use the same function)."""
+    return int(_lib.load().sd_rng_word(seed & 0xFFFFFFFF, stream, row & 0xFFFFFFFF, col & 0xFFFFFFFF))
+
+
 def mask_count(seed, channels, q):
     """Number of kept channels for keep probability q (host arithmetic only, no GPU work)."""
     return int(_lib.load().sd_mask_count(seed & 0xFFFFFFFF, channels, q))
