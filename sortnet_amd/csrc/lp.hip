@@ -356,6 +356,147 @@ __global__ void __launch_bounds__(256) lp_bwd_w_kernel(const float* __restrict__
     }
 }
 
+// Fused dense backward for grad_input AND grad_weight: u(b, m, n) is formed once and feeds both sums.
+// A workgroup owns FN = 8 consecutive input channels and a range of at most FMR weight rows; its 256
+// work-items are 16 (row of W: m = tm + 16 j) x 16 (batch row: b = tb + 16 i) with a 4 x 2 x 8 block of terms
+// each per (batch tile, weight tile) pair.  Outer loop = batch tiles, inner loop = weight tiles:
+//   grad_x partial sums of the 4 batch rows stay in registers across the inner loop, are reduced over the 16
+//   work-items that share the rows and added to memory (one atomic per row and channel and weight range);
+//   grad_w partial sums of a pair are combined through LDS into an accumulator that covers the whole weight
+//   range and is written out once at the end (the workgroup sees every batch row, so grad_weight needs no
+//   global atomics).
+// All operands sit in vector registers; the only LDS traffic is that combination.
+constexpr int FN = 8, FMR = 1024;
+
+__global__ void __launch_bounds__(256) lp_recip_kernel(const float* __restrict__ y, size_t n, float* __restrict__ ry) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) ry[i] = 1.f / y[i];
+}
+
+template <int IP>
+__global__ void __launch_bounds__(256, 3) lp_bwd_fused_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                              const float* __restrict__ g, const float* __restrict__ ry,
+                                                              int B, int M, int N, int mr, float pm1,
+                                                              float* __restrict__ gx, float* __restrict__ gw) {
+    constexpr int TI = 4, TJ = 2;                 // batch rows / weight rows per work-item
+    constexpr int PSTRIDE = FN * 16 * TJ + 16;    // plane of one batch-row group, skewed by 16 banks
+    constexpr int GSTRIDE = FMR + 32;
+    static_assert(FN * 16 * TJ == 256, "one accumulator per work-item and weight tile");
+    __shared__ float gwl[FN * GSTRIDE];
+    __shared__ float part[16 * PSTRIDE];
+    const int tid = threadIdx.x, tm = tid & 15, tb = tid >> 4;
+    const int n0 = blockIdx.x * FN;
+    const int m_lo = blockIdx.y * mr, m_hi = m_lo + mr < M ? m_lo + mr : M;
+    for (int e = tid; e < FN * GSTRIDE; e += 256) gwl[e] = 0.f;
+    __syncthreads();
+
+    for (int b0 = 0; b0 < B; b0 += 16 * TI) {
+        float xr[TI][FN], gxp[TI][FN];
+        int bi[TI];
+        #pragma unroll
+        for (int i = 0; i < TI; i++) {
+            int b = b0 + tb + 16 * i;
+            bi[i] = b < B ? b : -1;
+            const float* xp = x + (size_t)(b < B ? b : B - 1) * N + n0;
+            float4 v0 = *reinterpret_cast<const float4*>(xp), v1 = *reinterpret_cast<const float4*>(xp + 4);
+            xr[i][0] = v0.x; xr[i][1] = v0.y; xr[i][2] = v0.z; xr[i][3] = v0.w;
+            xr[i][4] = v1.x; xr[i][5] = v1.y; xr[i][6] = v1.z; xr[i][7] = v1.w;
+            #pragma unroll
+            for (int t = 0; t < FN; t++) gxp[i][t] = 0.f;
+        }
+        for (int m0 = m_lo; m0 < m_hi; m0 += 16 * TJ) {
+            float wr[TJ][FN], gwp[TJ][FN];
+            int mj[TJ];
+            #pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                int m = m0 + tm + 16 * j;
+                mj[j] = m < m_hi ? m : -1;
+                const float* wp = w + (size_t)(m < m_hi ? m : m_hi - 1) * N + n0;
+                float4 v0 = *reinterpret_cast<const float4*>(wp), v1 = *reinterpret_cast<const float4*>(wp + 4);
+                wr[j][0] = v0.x; wr[j][1] = v0.y; wr[j][2] = v0.z; wr[j][3] = v0.w;
+                wr[j][4] = v1.x; wr[j][5] = v1.y; wr[j][6] = v1.z; wr[j][7] = v1.w;
+                #pragma unroll
+                for (int t = 0; t < FN; t++) gwp[j][t] = 0.f;
+            }
+            #pragma unroll
+            for (int i = 0; i < TI; i++) {
+                #pragma unroll
+                for (int j = 0; j < TJ; j++) {
+                    const bool ok = bi[i] >= 0 && mj[j] >= 0;
+                    // padded rows reuse the last valid row of x / w and its own 1/y, so the ratio stays <= 1
+                    const size_t o = (size_t)(bi[i] >= 0 ? bi[i] : B - 1) * M + (mj[j] >= 0 ? mj[j] : m_hi - 1);
+                    const float gv = ok ? g[o] : 0.f, rv = ry[o];
+                    #pragma unroll
+                    for (int t = 0; t < FN; t++) {
+                        float pw = signed_pow<IP>(xr[i][t] - wr[j][t], rv, pm1);
+                        gxp[i][t] = fmaf(gv, pw, gxp[i][t]);
+                        gwp[j][t] = fmaf(gv, pw, gwp[j][t]);
+                    }
+                }
+            }
+            // the 16 work-items that share a weight row publish their partial sums; work-item (t, row) of the
+            // tile then adds the 16 of them to the accumulator it owns (LDS float atomics are far too slow)
+            #pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                #pragma unroll
+                for (int t = 0; t < FN; t++) part[tb * PSTRIDE + t * (16 * TJ) + tm + 16 * j] = gwp[j][t];
+            }
+            __syncthreads();
+            {
+                const int t = tid / (16 * TJ), ml = tid % (16 * TJ);
+                float sum = 0.f;
+                #pragma unroll
+                for (int k = 0; k < 16; k++) sum += part[k * PSTRIDE + t * (16 * TJ) + ml];
+                if (m0 + ml < m_hi) gwl[t * GSTRIDE + (m0 - m_lo) + ml] += sum;
+            }
+            __syncthreads();
+        }
+        // sum over the 16 work-items that share the batch rows, then one atomic per row and channel
+        #pragma unroll
+        for (int i = 0; i < TI; i++) {
+            #pragma unroll
+            for (int t = 0; t < FN; t++) {
+                float v = gxp[i][t];
+                v += __shfl_xor(v, 1); v += __shfl_xor(v, 2); v += __shfl_xor(v, 4); v += __shfl_xor(v, 8);
+                gxp[i][t] = v;
+            }
+        }
+        if (tm == 0) {
+            #pragma unroll
+            for (int i = 0; i < TI; i++) {
+                if (bi[i] >= 0) {
+                    #pragma unroll
+                    for (int t = 0; t < FN; t++) unsafeAtomicAdd(gx + (size_t)bi[i] * N + n0 + t, gxp[i][t]);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < (m_hi - m_lo) * 2; e += 256) {
+        int row = e >> 1, h = (e & 1) * 4;
+        const float* src = gwl + h * GSTRIDE + row;
+        *reinterpret_cast<float4*>(gw + (size_t)(m_lo + row) * N + n0 + h) =
+            make_float4(-src[0], -src[GSTRIDE], -src[2 * GSTRIDE], -src[3 * GSTRIDE]);
+    }
+}
+
+static int launch_lp_bwd_fused(int ip, const LpBwdArgs& a, hipStream_t st) {
+    const int B = a.R, M = a.COg, N = a.CIg;
+    const size_t n = (size_t)B * M;
+    float* ry = static_cast<float*>(workspace(n * sizeof(float)));
+    if (!ry) return SD_ERR_HIP;
+    hipLaunchKernelGGL(lp_recip_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a.y, n, ry);
+    int rc = check_launch("lp_recip_kernel");
+    if (rc) return rc;
+    if ((rc = fill_zero(a.gx, (size_t)B * N, st))) return rc;
+    const int ranges = (M + FMR - 1) / FMR;
+    const int mr = (((M + ranges - 1) / ranges) + 31) / 32 * 32;   // equal ranges, whole weight tiles
+    dim3 grid(N / FN, (M + mr - 1) / mr);
+    (void)ip;
+    hipLaunchKernelGGL((lp_bwd_fused_kernel<-1>), grid, dim3(256), 0, st, a.x, a.w, a.gy, ry, B, M, N, mr, a.pm1, a.gx, a.gw);
+    return check_launch("lp_bwd_fused_kernel");
+}
+
 template <int IP>
 static void launch_lp_bwd_dense_ip(const LpBwdArgs& a, const float* ry, const float* gT, const float* ryT, hipStream_t st) {
     const int B = a.R, M = a.COg, N = a.CIg;
@@ -420,6 +561,9 @@ static int lp_backward(const char* who, const float* grad_output, const float* i
     int ip = int_power(p - 1.f);
     const bool dense = G == 1 && HW == 1 && !ci_idx && !co_idx && f.CIg % TNB == 0 && aligned16(input) &&
                        aligned16(weight) && aligned16(grad_input) && (!grad_weight || aligned16(grad_weight));
+    // general p: the two transcendentals per term are worth sharing between both gradients; integral
+    // p - 1 <= 8 (multiply chains) is faster through the two reduction-free kernels
+    if (dense && grad_weight && ip < 0) return launch_lp_bwd_fused(ip, a, st);
     if (dense) return launch_lp_bwd_dense(ip, a, st);
     if (grad_weight) {
         if ((rc = fill_zero(grad_weight, (size_t)G * f.W_COg * f.W_CIg, st))) return rc;
