@@ -21,7 +21,7 @@ PEAK = 157.3e12
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--shape", type=int, nargs=3, default=[512, 5120, 5120], metavar=("B", "N", "M"))
-    ap.add_argument("--ops", default="linf,mask,bwd,bound,sort,lp,shift")
+    ap.add_argument("--ops", default="linf,mask,bwd,bound,sort,lp,shift,idx")
     ap.add_argument("--reps", type=int, default=5)
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
@@ -99,6 +99,30 @@ def main():
             t("norm_dist_backward_input_weight p=%g" % p,
               lambda: ext.norm_dist_backward_input_weight(gy, xn, w, y, gx, gw, 1, p), fb)
             t("norm_dist_backward_input p=%g" % p, lambda: ext.norm_dist_backward_input(gy, xn, w, y, gx, 1, p), fb / 2)
+    if "idx" in on:
+        # index-list ("dropout") form: every 32-sample sub-batch keeps its own ~q share of the inputs and outputs
+        qk = 0.3
+        S = (B + 31) // 32
+        cn, cm = ext.mask_count(1, N, qk), ext.mask_count(2, M, qk)
+        ci = ext.sample_index_lists(1, S, 1, N, cn, dev)
+        co = ext.sample_index_lists(2, S, 1, M, cm, dev)
+        xc = torch.rand(B, cn, 1, generator=g).to(dev)
+        gyc = torch.randn(B, cm, 1, generator=g).to(dev)
+        yc = torch.empty(B, cm, 1, device=dev)
+        posc = torch.empty(B, cm, 1, device=dev, dtype=torch.int32)
+        gxc = torch.empty_like(xc)
+        sub = B * cn * cm
+        scale = terms / sub          # the helper divides by the dense term count
+        t("index lists: %d of %d in, %d of %d out" % (cn, N, cm, M), lambda: None)
+        rows.pop()
+        t("  sample_index_lists (both)", lambda: (ext.sample_index_lists(1, S, 1, N, cn, dev),
+                                                   ext.sample_index_lists(2, S, 1, M, cm, dev)))
+        t("  inf_dist_forward (+pos, lists)", lambda: ext.inf_dist_forward(xc, w, yc, posc, 1, ci, co), 2 / scale)
+        t("  inf_dist_backward_input_weight (lists)",
+          lambda: ext.inf_dist_backward_input_weight(gyc, posc, gxc, gw, 1, ci, co))
+        t("  norm_dist_forward p=8 (lists)", lambda: ext.norm_dist_forward(xc, w, yc, 1, 8.0, ci, co), 5 / scale)
+        t("  norm_dist_backward_input_weight p=8 (lists)",
+          lambda: ext.norm_dist_backward_input_weight(gyc, xc, w, yc, gxc, gw, 1, 8.0, ci, co), 9 / scale)
     if "shift" in on:
         t("mean_shift_forward", lambda: ext.mean_shift_forward(y, mean, None, 0.1, y2), None, 4 * (3 * B * M))
     if args.json:
