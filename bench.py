@@ -20,8 +20,8 @@ if ROOT not in sys.path:
 
 FP32_VECTOR_PEAK_TFLOPS = 157.3     # MI355X published fp32 vector peak
 # HBM bytes of one 512x5120x5120 interval-bound launch from the FETCH_SIZE / WRITE_SIZE counter runs
-# (2.00 * 176252 KiB + 81920 KiB); only reported when the benchmark runs at that shape
-IBP_LAUNCH_TRAFFIC_BYTES = 444.8e6
+# (2.00 * 171079 KiB + 163840 KiB); only reported when the benchmark runs at that shape
+IBP_LAUNCH_TRAFFIC_BYTES = 518.0e6
 VALU_LANE_RATE = 39.32e12           # 256 CUs x 4 SIMD x 16 lanes x 2.4 GHz lane-instructions/s
 
 
