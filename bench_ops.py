@@ -121,6 +121,8 @@ def main():
         t("  inf_dist_backward_input_weight (lists)",
           lambda: ext.inf_dist_backward_input_weight(gyc, posc, gxc, gw, 1, ci, co))
         t("  norm_dist_forward p=8 (lists)", lambda: ext.norm_dist_forward(xc, w, yc, 1, 8.0, ci, co), 5 / scale)
+        t("  norm_dist_backward_input p=8 (lists)",
+          lambda: ext.norm_dist_backward_input(gyc, xc, w, yc, gxc, 1, 8.0, ci, co), 4.5 / scale)
         t("  norm_dist_backward_input_weight p=8 (lists)",
           lambda: ext.norm_dist_backward_input_weight(gyc, xc, w, yc, gxc, gw, 1, 8.0, ci, co), 9 / scale)
     if "shift" in on:

@@ -87,7 +87,7 @@ struct LpBwdArgs {
     const int* ci_idx; const int* co_idx;
     int B, R, HW, G, COg, CIg, W_COg, W_CIg;
     float pm1;   // p - 1
-    int zsplit;  // slices of the channel range in the dense grad_input kernel
+    int zsplit;  // slices of the output-channel range (grad_input then merges with atomic adds)
 };
 
 template <int IP>
@@ -116,7 +116,10 @@ __global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
     __shared__ float2 gr[MC][RB];   // (g, 1/y) of output channel m0+k, row r0+i
 
     const int tid = threadIdx.x;
-    const int g = blockIdx.z;
+    const int g = blockIdx.z % a.G, slice = blockIdx.z / a.G;
+    // output channels of this slice, whole LDS chunks
+    const int per = ((a.COg + a.zsplit - 1) / a.zsplit + MC - 1) / MC * MC;
+    const int m_lo = slice * per, m_hi = m_lo + per < a.COg ? m_lo + per : a.COg;
     const int r0 = blockIdx.y * RB;
     const int n = blockIdx.x * 256 + tid;
     const bool n_ok = n < a.CIg;
@@ -139,7 +142,7 @@ __global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
         acc[i] = 0.f;
     }
 
-    for (int m0 = 0; m0 < a.COg; m0 += MC) {
+    for (int m0 = m_lo; m0 < m_hi; m0 += MC) {
         __syncthreads();
         // stage (g, 1/y): MC * RB = 512 pairs, two per work-item; consecutive work-items take
         // consecutive channels of one row when HW == 1
@@ -148,7 +151,7 @@ __global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
             int k = e % MC, i = e / MC;
             int m = m0 + k, r = r0 + i;
             float2 v = make_float2(0.f, 0.f);
-            if (m < a.COg && i < rows) {
+            if (m < m_hi && i < rows) {
                 int b = r / a.HW, hw = r - b * a.HW;
                 size_t o = ((size_t)(b * a.G + g) * a.COg + m) * a.HW + hw;
                 v.x = a.gy[o];
@@ -161,14 +164,14 @@ __global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
         for (int k = 0; k < MC; k++) {
             int m = m0 + k;
             float v = 0.f;
-            if (n_ok && m < a.COg) {
+            if (n_ok && m < m_hi) {
                 int wrow = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + m] : m;
                 v = a.w[(size_t)(g * a.W_COg + wrow) * a.W_CIg + wcol];
             }
             wv[k] = v;
         }
         __syncthreads();
-        const int mcount = a.COg - m0 < MC ? a.COg - m0 : MC;
+        const int mcount = m_hi - m0 < MC ? m_hi - m0 : MC;
         for (int k = 0; k < mcount; k++) {
             float wsum = 0.f;
             if (rows == RB) {
@@ -203,7 +206,9 @@ __global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
             if (i < rows) {
                 int r = r0 + i;
                 int b = r / a.HW, hw = r - b * a.HW;
-                a.gx[((size_t)(b * a.G + g) * a.CIg + n) * a.HW + hw] = acc[i];
+                float* dst = a.gx + ((size_t)(b * a.G + g) * a.CIg + n) * a.HW + hw;
+                if (a.zsplit > 1) unsafeAtomicAdd(dst, acc[i]);
+                else *dst = acc[i];
             }
         }
     }
@@ -532,8 +537,17 @@ static int launch_lp_bwd_dense(int ip, const LpBwdArgs& a_in, hipStream_t st) {
 }
 
 template <bool WGRAD>
-static int launch_lp_bwd(int ip, const LpBwdArgs& a, hipStream_t st) {
-    dim3 grid((a.CIg + 255) / 256, (a.R + RB - 1) / RB, a.G);
+static int launch_lp_bwd(int ip, const LpBwdArgs& a_in, hipStream_t st) {
+    // a workgroup covers 256 input channels x 32 rows and walks the output channels; when that leaves the
+    // device mostly idle (index lists: a few hundred kept inputs per sub-batch) the output-channel range is
+    // cut in slices that merge into grad_input with atomic adds
+    LpBwdArgs a = a_in;
+    const long long blocks = (long long)((a.CIg + 255) / 256) * ((a.R + RB - 1) / RB) * a.G;
+    a.zsplit = 1;
+    while (a.zsplit < 16 && blocks * a.zsplit < 4ll * num_cus() && a.COg / (a.zsplit * 2) >= 4 * MC) a.zsplit *= 2;
+    int rc;
+    if (a.zsplit > 1 && (rc = fill_zero(a.gx, (size_t)a.R * a.G * a.CIg, st))) return rc;
+    dim3 grid((a.CIg + 255) / 256, (a.R + RB - 1) / RB, a.G * a.zsplit);
 #define SD_CASE(k) case k: hipLaunchKernelGGL((lp_bwd_kernel<k, WGRAD>), grid, dim3(256), 0, st, a); break;
     switch (ip) {
         SD_CASE(0) SD_CASE(1) SD_CASE(2) SD_CASE(3) SD_CASE(4) SD_CASE(5) SD_CASE(6) SD_CASE(7) SD_CASE(8)
