@@ -126,13 +126,16 @@ __device__ __forceinline__ void load_w_tile(float (*ws)[LDP], const FwdArgs& a,
             *reinterpret_cast<float4*>(&ws[row][c4]) = v;
         }
     } else {
-        for (int e = tid; e < BM * KT; e += 256) {
-            int row = e / KT, c = e - row * KT;
-            int m = m0 + row, n = k0 + c;
+        // a work-item stages one column of the chunk (256 is a multiple of KT): its input index is looked up once
+        const int c = tid % KT, n = k0 + c;
+        const bool n_ok = n < n_end;
+        const int wcol = n_ok ? (a.ci_idx ? a.ci_idx[(s * a.G + g) * a.CIg + n] : n) : 0;
+        #pragma unroll
+        for (int row = tid / KT; row < BM; row += 256 / KT) {
+            int m = m0 + row;
             float v = 0.f;
-            if (m < a.COg && n < n_end) {
+            if (m < a.COg && n_ok) {
                 int wrow = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + m] : m;
-                int wcol = a.ci_idx ? a.ci_idx[(s * a.G + g) * a.CIg + n] : n;
                 v = a.w[(size_t)(g * a.W_COg + wrow) * a.W_CIg + wcol];
                 if (masked) v = mask_value(v, rng_row_key(a.seed, 2u, (uint32_t)(g * a.COg + m)), n, a.t16);
             }
