@@ -649,6 +649,64 @@ struct SortPos : PolicyBase {
     }
 };
 
+// First pass of the two-level sort neuron.  The hot loop only keeps the maximum of |x - w| over a chunk of
+// KT inputs (like LinfChunk); at the end of a chunk that maximum, with its low kKeyIdBits mantissa bits
+// replaced by the chunk number, enters a sorted list of the K + kKeySlack largest such keys (branch-free
+// 3-input medians on the integer patterns; all keys differ because the chunk numbers do).
+// Why the list is enough: truncation is monotone, so the K-th largest truncated maximum is the truncation of
+// the K-th largest maximum, and every term that can belong to the K largest terms lies in a chunk whose
+// truncated maximum reaches that value.  Unless more than kKeySlack further chunks share that truncated
+// value (then the smallest kept key still has it and the second pass scans every chunk instead), all those
+// chunks are in the list; the second pass (sort_rows_kernel) looks at their K * KT or so candidates only.
+// Keys go to p0 as K + kKeySlack planes of (channel, sample) layout.
+constexpr int kKeyIdBits = 10;          // chunk numbers below 1024
+constexpr int kKeySlack = 6;
+
+__device__ __forceinline__ uint32_t umed3(uint32_t a, uint32_t b, uint32_t c) {
+    uint32_t r;
+    asm("v_med3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+template <int KP>
+__device__ __forceinline__ void key_insert(uint32_t (&key)[KP], uint32_t v) {
+    #pragma unroll
+    for (int k = 0; k < KP - 1; k++) key[k] = umed3(key[k], v, key[k + 1]);
+    key[KP - 1] = key[KP - 1] > v ? key[KP - 1] : v;
+}
+
+template <int K>
+struct SortChunkKeys : PolicyBase {
+    static constexpr int KP = K + kKeySlack;
+    static constexpr int PIPE_WAVES = 2;
+    static constexpr int MIN_WAVES = 2;
+    struct Acc { float cm; uint32_t key[KP]; };
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
+        A.cm = 0.f;
+        #pragma unroll
+        for (int k = 0; k < KP; k++) A.key[k] = 0u;
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
+                                                 const float4& w, int, int) {
+        float v = A.cm;
+        v = fmaxf(fmaxf(v, fabsf(x.x - w.x)), fabsf(x.y - w.y));
+        v = fmaxf(fmaxf(v, fabsf(x.z - w.z)), fabsf(x.w - w.w));
+        A.cm = v;
+    }
+    static __device__ __forceinline__ void chunk_end(Acc& A, const FwdArgs&, int, int k0) {
+        const uint32_t v = (__float_as_uint(A.cm) & ~((1u << kKeyIdBits) - 1u)) | (uint32_t)(k0 / KT);
+        A.cm = 0.f;
+        key_insert<KP>(A.key, v);
+    }
+    // plane k, then output channel, then sample: the second pass reads one channel for consecutive samples
+    static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
+        const int channels = a.G * a.COg;                 // HW == 1 on this path
+        const int b = (int)(o / channels), c = (int)(o - (size_t)b * channels);
+        #pragma unroll
+        for (int k = 0; k < KP; k++) a.p0[((size_t)k * channels + c) * a.B + b] = (int)A.key[k];
+    }
+};
+
 // interval bounds of the sort neuron (core/cuda/sort_neuron.cu:216-314).  The lower side keeps
 // the negated K most negative values of min(t1,t2), so both sides share the insertion routine.
 template <int K>

@@ -16,6 +16,115 @@ static int check_qk(const char* who, float q, int K, int CIg) {
     return SD_OK;
 }
 
+// Second pass of the two-level sort neuron.  One workgroup per weight row: the row is staged in LDS once
+// (chunks of KT floats, each followed by 4 floats of padding so that work-items reading different chunks hit
+// different banks) and every work-item resolves one output of that row at a time, reading the candidate
+// chunks of its input row (128-bit loads) against the staged weights.  VALUES: the K largest candidate values
+// by branch-free insertion; otherwise the reference's ordered insertion with indices over the candidates in
+// ascending input order (the chunk numbers are sorted first), which ends in the same list as the scan over
+// all inputs because every left-out term is smaller than the final K-th value.
+constexpr int kSortRowMax = 12288;   // inputs per weight row this path stages
+constexpr int kChunkPad = KT + 4;
+
+template <int K, bool VALUES>
+__global__ void __launch_bounds__(256) sort_rows_kernel(FwdArgs a, const int* __restrict__ keys) {
+    constexpr int KP = K + kKeySlack;
+    extern __shared__ __attribute__((aligned(16))) float wrow[];
+    const int c = blockIdx.x;                      // g * COg + m
+    const int g = c / a.COg;
+    const float* wsrc = a.w + (size_t)c * a.CIg;
+    for (int n = threadIdx.x * 4; n < a.CIg; n += 1024)
+        *reinterpret_cast<float4*>(wrow + (n / KT) * kChunkPad + (n % KT)) = *reinterpret_cast<const float4*>(wsrc + n);
+    __syncthreads();
+    const size_t size = (size_t)a.B * a.G * a.COg;
+    const int nchunks = (a.CIg + KT - 1) / KT;
+    for (int b = threadIdx.x; b < a.B; b += 256) {
+        const size_t o = (size_t)b * a.G * a.COg + c;
+        const float* xr = a.x0 + (size_t)(b * a.G + g) * a.CIg;
+        float res[K];
+        int idx[K];
+        #pragma unroll
+        for (int k = 0; k < K; k++) { res[k] = 0.f; idx[k] = 0; }
+        auto chunk = [&](int cid) {
+            const int n0 = cid * KT;
+            const float* wc = wrow + cid * kChunkPad;
+            #pragma unroll
+            for (int q4 = 0; q4 < KT / 4; q4++) {
+                int n = n0 + 4 * q4;
+                const bool in = n < a.CIg;           // CIg is a multiple of 4 on this path
+                if (!in) n = a.CIg - 4;
+                const float4 xv = *reinterpret_cast<const float4*>(xr + n);
+                const float4 wv = *reinterpret_cast<const float4*>(wc + (n - n0));
+                const float d[4] = {xv.x - wv.x, xv.y - wv.y, xv.z - wv.z, xv.w - wv.w};
+                #pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float v = in ? fabsf(d[e]) : 0.f;
+                    if (VALUES) topk_insert_values<K>(res, v);
+                    else if (v > res[0]) topk_insert<K>(res, idx, v, (n + e) | (d[e] >= 0.f ? 0 : (int)kSign));
+                }
+            }
+        };
+        uint32_t key[KP];
+        #pragma unroll
+        for (int k = 0; k < KP; k++) key[k] = (uint32_t)keys[((size_t)k * a.G * a.COg + c) * a.B + b];
+        // keys ascend: key[KP - K] is the K-th largest; chunks whose truncated maximum reaches it are candidates
+        const uint32_t cut = key[KP - K] >> kKeyIdBits;
+        if (cut != 0u && (key[0] >> kKeyIdBits) == cut) {
+            for (int cid = 0; cid < nchunks; cid++) chunk(cid);     // too many chunks share the cut value
+        } else {
+            int ids[KP];
+            #pragma unroll
+            for (int k = 0; k < KP; k++) {
+                const uint32_t bucket = key[k] >> kKeyIdBits;
+                ids[k] = (bucket != 0u && bucket >= cut) ? (int)(key[k] & ((1u << kKeyIdBits) - 1u)) : 0x7fffffff;
+            }
+            if (!VALUES) {
+                // ascending chunk numbers (odd-even transposition network; skipped slots sort to the end)
+                #pragma unroll
+                for (int i = 0; i < KP; i++) {
+                    #pragma unroll
+                    for (int k = i & 1; k + 1 < KP; k += 2) {
+                        int lo = min(ids[k], ids[k + 1]), hi = max(ids[k], ids[k + 1]);
+                        ids[k] = lo; ids[k + 1] = hi;
+                    }
+                }
+            }
+            #pragma unroll
+            for (int k = 0; k < KP; k++) {
+                if (ids[k] < nchunks) chunk(ids[k]);
+            }
+        }
+        a.y0[o] = geo_sum<K>(res, a.q);
+        if (!VALUES) {
+            #pragma unroll
+            for (int k = K - 1; k >= 0; k--) a.p0[(size_t)(K - 1 - k) * size + o] = idx[k];
+        }
+    }
+}
+
+// two-level path: dense vector-load case with a reduction long enough for the chunk lists to pay
+static bool two_level_ok(const FwdArgs& a, int K) {
+    const int nchunks = (a.CIg + KT - 1) / KT;
+    return a.HW == 1 && a.fast_x && a.fast_w && a.CIg <= kSortRowMax && K <= 12 && nchunks >= 4 * K &&
+           nchunks <= (1 << kKeyIdBits);
+}
+
+template <int K, bool VALUES>
+static int run_two_level(FwdArgs& a, bool small, hipStream_t st) {
+    constexpr int KP = K + kKeySlack;
+    const size_t total = (size_t)a.R * a.G * a.COg;
+    int* keys = static_cast<int*>(workspace((size_t)KP * total * sizeof(int)));
+    if (!keys) return SD_ERR_HIP;
+    FwdArgs t = a;
+    t.p0 = keys;
+    int rc = small ? launch_fwd<SortChunkKeys<K>, 1, 2>(t, st) : launch_fwd<SortChunkKeys<K>, 2, 4>(t, st);
+    if (rc) return rc;
+    const int nchunks = (a.CIg + KT - 1) / KT;
+    hipLaunchKernelGGL((sort_rows_kernel<K, VALUES>), dim3((unsigned)(a.G * a.COg)), dim3(256),
+                       (size_t)nchunks * kChunkPad * sizeof(float), st, a, keys);
+    return check_launch("sort_rows_kernel");
+}
+
 // few output tiles: 16 x 32 tiles instead of 32 x 64 (the top-K lists do not merge across a split reduction)
 static bool few_tiles(const FwdArgs& a, int BB, int BM) {
     long long tiles = (long long)((a.R + BB - 1) / BB) * ((a.COg + BM - 1) / BM) * a.G;
@@ -34,7 +143,8 @@ extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* we
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 64);
     switch (K) {
-#define X(k) case k: return small ? launch_fwd<SortNograd<k>, 1, 2>(a, st) : launch_fwd<SortNograd<k>, 2, 4>(a, st);
+#define X(k) case k: if (k <= 12 && two_level_ok(a, k)) return run_two_level<(k <= 12 ? k : 2), true>(a, small, st); \
+                     return small ? launch_fwd<SortNograd<k>, 1, 2>(a, st) : launch_fwd<SortNograd<k>, 2, 4>(a, st);
         SD_FOR_EACH_K(X)
 #undef X
     }
@@ -54,7 +164,8 @@ extern "C" int sd_sort_neuron_forward(const float* input, const float* weight,
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 32);
     switch (K) {
-#define X(k) case k: return small ? launch_fwd<SortPos<k>, 1, 2>(a, st) : launch_fwd<SortPos<k>, 2, 2>(a, st);
+#define X(k) case k: if (k <= 12 && two_level_ok(a, k)) return run_two_level<(k <= 12 ? k : 2), false>(a, few_tiles(a, 32, 64), st); \
+                     return small ? launch_fwd<SortPos<k>, 1, 2>(a, st) : launch_fwd<SortPos<k>, 2, 2>(a, st);
         SD_FOR_EACH_K(X)
 #undef X
     }

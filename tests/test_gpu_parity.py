@@ -275,6 +275,39 @@ def test_sort_neuron_tie_order(oracle):
     _close(y, ry)
 
 
+@pytest.mark.parametrize("case", ["random", "grid", "flat", "sparse", "groups"])
+@pytest.mark.parametrize("K", [10, 4, 12])
+def test_sort_neuron_long_rows(oracle, case, K):
+    """Rows long enough for the two-level path (chunk lists, then a candidate scan): continuous data, data
+    on a coarse grid (exact ties inside and across chunks), chunk maxima that are all equal (the exhaustive
+    scan of the second pass), rows with fewer than K non-zero terms, and groups."""
+    from sortnet_amd import ext
+    dev = _dev()
+    G = 2 if case == "groups" else 1
+    B, CI, CO = 37, 2048 * G, 24 * G
+    x, w = _gen((B, CI, 1), 51, "rand"), _gen((CO, CI // G), 52, scale=0.3)
+    if case == "grid":
+        x, w = torch.round(x * 8) / 8, torch.round(w * 4) / 4
+    elif case == "flat":
+        x, w = torch.round(x * 2) / 2, torch.zeros_like(w)       # every chunk maximum is 1
+    elif case == "sparse":
+        keep = torch.zeros(CI)
+        keep[[5, 700, 701, 1500]] = 1.0
+        x, w = x * keep.view(1, -1, 1), w * 0
+    x, w = x.contiguous(), w.contiguous()
+    q = 0.3
+    ry, rpos = oracle.sort_neuron_forward(x.numpy(), w.numpy(), q, K, G)
+    xd, wd = x.to(dev), w.to(dev)
+    y = torch.empty(B, CO, 1, device=dev)
+    pos = torch.empty(K, B, CO, 1, device=dev, dtype=torch.int32)
+    ext.sort_neuron_forward(xd, wd, y, pos, G, q, K)
+    assert np.array_equal(pos.cpu().numpy(), rpos)
+    _close(y, ry)
+    y2 = torch.empty_like(y)
+    ext.sort_neuron_forward_nograd(xd, wd, y2, G, q, K)
+    _close(y2, ry)
+
+
 @pytest.mark.parametrize("p", [1.0, 2.0, 3.0, 7.0, 8.0, 9.5, 11.3, 64.0, 300.0])
 @pytest.mark.parametrize("B,CI,CO,G,HW", [SHAPES[1], SHAPES[3], SHAPES[4]])
 def test_norm_dist(oracle, p, B, CI, CO, G, HW):
