@@ -308,6 +308,25 @@ def test_sort_neuron_long_rows(oracle, case, K):
     _close(y2, ry)
 
 
+def test_sort_neuron_widest_rows(oracle):
+    """12288 inputs per row (the widest first layer): the candidate scan needs more than 64 KiB of LDS; the
+    row length is not a multiple of the chunk size in the second case."""
+    from sortnet_amd import ext
+    dev = _dev()
+    for CI in (12288, 12268):
+        B, CO, K, q = 70, 9, 10, 0.3
+        x, w = _gen((B, CI, 1), 61, "rand"), _gen((CO, CI), 62, scale=0.3)
+        ry, rpos = oracle.sort_neuron_forward(x.numpy(), w.numpy(), q, K)
+        xd, wd = x.to(dev), w.to(dev)
+        y = torch.empty(B, CO, 1, device=dev)
+        pos = torch.empty(K, B, CO, 1, device=dev, dtype=torch.int32)
+        ext.sort_neuron_forward(xd, wd, y, pos, 1, q, K)
+        assert np.array_equal(pos.cpu().numpy(), rpos)
+        _close(y, ry)
+        ext.sort_neuron_forward_nograd(xd, wd, y, 1, q, K)
+        _close(y, ry)
+
+
 @pytest.mark.parametrize("p", [1.0, 2.0, 3.0, 7.0, 8.0, 9.5, 11.3, 64.0, 300.0])
 @pytest.mark.parametrize("B,CI,CO,G,HW", [SHAPES[1], SHAPES[3], SHAPES[4]])
 def test_norm_dist(oracle, p, B, CI, CO, G, HW):
