@@ -817,13 +817,17 @@ struct LpOnline : PolicyBase {
     }
 };
 
-// caller-supplied maximum (core/cuda/norm_dist_cuda.cu:163-259 with has_max)
+// caller-supplied maximum (core/cuda/norm_dist_cuda.cu:163-259 with has_max); also the second step of the
+// general-p forward, whose first step is the l-inf kernel
 template <int IP>
 struct LpWithMax : PolicyBase {
+    static constexpr int PIPE_WAVES = 3;
+    static constexpr int MIN_WAVES = 3;
     struct Acc { float s, rinv; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool valid, int split = 0) {
         A.rinv = valid ? 1.f / a.aux[o] : 1.f;
-        A.s = __builtin_amdgcn_exp2f(a.p * __builtin_amdgcn_logf(kEps * A.rinv));
+        // the virtual term of size 1e-10 belongs to slice 0 only
+        A.s = split == 0 ? __builtin_amdgcn_exp2f(a.p * __builtin_amdgcn_logf(kEps * A.rinv)) : 0.f;
     }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
                                                  const float4& w, int, int) {
@@ -833,7 +837,8 @@ struct LpWithMax : PolicyBase {
         A.s += pow_pos<IP>(fabsf(x.w - w.w) * A.rinv, a.p);
     }
     static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
-        a.y0[o] = powf(A.s, a.inv_p) / A.rinv;
+        if (a.nsplit > 1) a.part0[(size_t)split * a.part_stride + o] = A.s;   // merged by lp_finalize_kernel
+        else a.y0[o] = powf(A.s, a.inv_p) / A.rinv;
     }
 };
 

@@ -26,8 +26,10 @@ static int launch_lp(int ip, const FwdArgs& a, hipStream_t st) {
     }
 }
 
-// merges the split-N slices of the l-p forward in slice order (deterministic) and takes the root
+// merges the split-N slices of the l-p forward in slice order (deterministic) and takes the root:
+// plain sums, sums relative to a known maximum (scale), or (sum, running maximum) pairs of the online form
 __global__ void __launch_bounds__(256) lp_finalize_kernel(const float* __restrict__ part0, const float* __restrict__ part1,
+                                                          const float* __restrict__ scale,
                                                           int nsplit, size_t total, float p, float inv_p,
                                                           float* __restrict__ y) {
     size_t o = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -35,7 +37,7 @@ __global__ void __launch_bounds__(256) lp_finalize_kernel(const float* __restric
     if (part1 == nullptr) {
         float s = 0.f;
         for (int k = 0; k < nsplit; k++) s += part0[(size_t)k * total + o];
-        y[o] = powf(fmaxf(s, FLT_MIN), inv_p);
+        y[o] = scale ? powf(s, inv_p) * scale[o] : powf(fmaxf(s, FLT_MIN), inv_p);
     } else {
         float M = kEps;
         for (int k = 0; k < nsplit; k++) M = fmaxf(M, part1[(size_t)k * total + o]);
@@ -64,8 +66,32 @@ static int lp_split_setup(FwdArgs& a, int BB, int BM, bool online) {
 static int lp_split_finish(const FwdArgs& a, hipStream_t st) {
     if (a.nsplit <= 1) return SD_OK;
     hipLaunchKernelGGL(lp_finalize_kernel, dim3((unsigned)((a.part_stride + 255) / 256)), dim3(256), 0, st,
-                       a.part0, a.part1, a.nsplit, a.part_stride, a.p, a.inv_p, a.y0);
+                       a.part0, a.part1, a.part1 ? nullptr : a.aux, a.nsplit, a.part_stride, a.p, a.inv_p, a.y0);
     return check_launch("lp_finalize_kernel");
+}
+
+// General p on the vector path: the exact maximum of |x - w| per output first (l-inf kernel, 1.5
+// instructions per term), then one pass of sums relative to it, instead of the online form's two passes over
+// every LDS chunk.  Workspace: the maxima, then the partial sums of the split reduction.
+static int lp_forward_max_first(FwdArgs& a, bool small, hipStream_t st) {
+    const size_t total = (size_t)a.R * a.G * a.COg;
+    FwdArgs m = a;
+    m.nsplit = pick_nsplit(m, small ? 32 : 64, 128);
+    a.nsplit = m.nsplit;
+    float* base = static_cast<float*>(workspace(total * (size_t)(1 + (a.nsplit > 1 ? a.nsplit : 0)) * sizeof(float)));
+    if (!base) return SD_ERR_HIP;
+    m.y0 = base;
+    int rc;
+    if (m.nsplit > 1 && (rc = fill_zero(base, total, st))) return rc;
+    rc = small ? launch_fwd<LinfNograd, 2, 8>(m, st) : launch_fwd<LinfNograd, 4, 8>(m, st);
+    if (rc) return rc;
+    a.aux = base;
+    a.part_stride = total;
+    a.part0 = a.nsplit > 1 ? base + total : nullptr;
+    a.part1 = nullptr;
+    rc = small ? launch_fwd<LpWithMax<-1>, 2, 8>(a, st) : launch_fwd<LpWithMax<-1>, 4, 8>(a, st);
+    if (rc) return rc;
+    return lp_split_finish(a, st);
 }
 
 // ---- backward -------------------------------------------------------------------------------
@@ -605,6 +631,7 @@ extern "C" int sd_norm_dist_forward(const float* input, const float* weight,
     static const int kTb42[] = {4, 2};
     const bool small = w_index_ci || w_index_co || pick_tb(a, kTb42, 2, 128) == 2;
     const bool online = p > 10.f;   // core/cuda/norm_dist.cpp:4,51-55
+    if (online && a.fast_x && a.fast_w && !w_index_co) return lp_forward_max_first(a, small, st);
     if ((rc = lp_split_setup(a, small ? 32 : 64, 128, online))) return rc;
     if (!online) {
         int ip = int_power(p);
