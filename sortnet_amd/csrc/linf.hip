@@ -53,13 +53,12 @@ extern "C" int sd_inf_dist_forward_nograd(const float* input, const float* weigh
     SD_REQUIRE(output, "inf_dist_forward_nograd: null output");
     a.y0 = output;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    static const int kTb842[] = {8, 4, 2};
-    const int TB = pick_tb(a, kTb842, 3, 128);
+    static const int kTb42[] = {4, 2};   // 8 rows per work-item measured slower (168 registers, three waves per SIMD)
+    const int TB = pick_tb(a, kTb42, 2, 128);
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;
     if (TB == 2) return launch_fwd<LinfNograd, 2, 8>(a, st);
-    if (TB == 4) return launch_fwd<LinfNograd, 4, 8>(a, st);
-    return launch_fwd<LinfNograd, 8, 8>(a, st);
+    return launch_fwd<LinfNograd, 4, 8>(a, st);
 }
 
 extern "C" int sd_inf_dist_forward(const float* input, const float* weight,
@@ -117,13 +116,12 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
         a.xmask = xm; a.wmask = wm;
     }
     if (pos) return run_chunk_pos<LinfChunk>(a, false, st);
-    static const int kTb842[] = {8, 4, 2};
-    const int TB = pick_tb(a, kTb842, 3, 128);
+    static const int kTb42[] = {4, 2};   // 8 rows per work-item measured slower (168 registers, three waves per SIMD)
+    const int TB = pick_tb(a, kTb42, 2, 128);
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;
     if (TB == 2) return launch_fwd<LinfNograd, 2, 8>(a, st);
-    if (TB == 4) return launch_fwd<LinfNograd, 4, 8>(a, st);
-    return launch_fwd<LinfNograd, 8, 8>(a, st);
+    return launch_fwd<LinfNograd, 4, 8>(a, st);
 }
 
 extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float* inputU, const float* weight,
