@@ -15,16 +15,6 @@
 #include <stdlib.h>
 #include "common.h"
 
-#ifndef SD_MT_WAVES
-#define SD_MT_WAVES 2
-#endif
-#ifndef SD_MT_TB
-#define SD_MT_TB 4
-#endif
-#ifndef SD_MT_TM
-#define SD_MT_TM 8
-#endif
-
 
 namespace sd {
 
@@ -468,9 +458,8 @@ struct LinfChunk : PolicyBase {
 
 // the per-term masked neuron with the same chunk tracking
 struct MaskedTermChunk : PolicyBase {
-    static constexpr int WIDE_TB = SD_MT_TB, WIDE_TM = SD_MT_TM;
-    static constexpr int PIPE_WAVES = SD_MT_WAVES;
-    static constexpr int MIN_WAVES = SD_MT_WAVES;
+    static constexpr int PIPE_WAVES = 2;   // hash-bound: timings were flat over 2..4 waves and 4x8 / 4x4 / 2x8 tiles
+    static constexpr int MIN_WAVES = 2;
     struct Acc { float best, cm; int cid; uint32_t key; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool, int split = 0) {
         A.best = kEps; A.cm = 0.f; A.cid = -1; A.key = rng_row_key(a.seed, 0u, (uint32_t)o);
@@ -497,8 +486,8 @@ struct MaskedTermChunk : PolicyBase {
 // masked neuron without positions, independent draw per term: byte (n & 3) of
 // word(key(output), n >> 2) < t8 keeps; dropped terms enter the maximum as 0
 struct MaskedTermMax : PolicyBase {
-    static constexpr int PIPE_WAVES = SD_MT_WAVES;
-    static constexpr int MIN_WAVES = SD_MT_WAVES;
+    static constexpr int PIPE_WAVES = 2;   // hash-bound: timings were flat over 2..4 waves and 4x8 / 4x4 / 2x8 tiles
+    static constexpr int MIN_WAVES = 2;
     struct Acc { float v; uint32_t key; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool, int split = 0) {
         A.v = kEps; A.key = rng_row_key(a.seed, 0u, (uint32_t)o);

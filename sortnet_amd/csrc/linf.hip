@@ -91,10 +91,9 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (mode == SD_MASK_TERM) {
         if (pos) return run_chunk_pos<MaskedTermChunk>(a, false, st);
-        const int TBm = small ? 2 : SD_MT_TB;
-        a.nsplit = pick_nsplit(a, 16 * TBm, small ? 128 : 16 * SD_MT_TM);
+        a.nsplit = pick_nsplit(a, small ? 32 : 64, 128);
         if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;
-        return small ? launch_fwd<MaskedTermMax, 2, 8>(a, st) : launch_fwd<MaskedTermMax, SD_MT_TB, SD_MT_TM>(a, st);
+        return small ? launch_fwd<MaskedTermMax, 2, 8>(a, st) : launch_fwd<MaskedTermMax, 4, 8>(a, st);
     }
     // factored mask: dropped inputs / weights are replaced by NaN while staging the tiles and
     // NaN terms never win the maximum, so the plain l-inf policies apply unchanged.  On the
