@@ -1,0 +1,121 @@
+"""The reference's SortNet model zoo on top of sortnet_amd.layers / sortnet_amd.heads
+(ell_inf_models.py:18-240): same constructor arguments, same `forward(x, targets, eps, up, down)` contract,
+same sub-module names (`fc_dist`, `fc_linear`, `fc_final`, `scalar`) so that reference checkpoints load.
+Extra keyword `registry`: the DropoutRegistry the distance layers share (default: the process-wide one).
+
+forward(x)                              -> logits (training / plain evaluation)
+forward(x, targets, eps)                -> (logits, worst-case margins): radius-eps ball around the distance
+                                           features (1-Lipschitz argument) when no input box is propagated
+forward(x, targets, eps, up, down)      -> the same with interval bounds propagated from the clipped input box
+                                           through every layer; only in evaluation mode with p = inf
+"""
+import math
+
+import torch
+import torch.nn as nn
+
+from .heads import BoundFinalLinear, BoundLinear, BoundTanh
+from .layers import BoundSequential, NormDist, NormDistBase, NormDistConv, apply_if_not_none
+
+
+def check_inf_and_eval(model):
+    """True when every distance layer is an evaluation-mode l-inf layer (ell_inf_models.py:10-14)."""
+    return all(math.isinf(m.p) and not m.training for m in model.modules() if isinstance(m, NormDistBase))
+
+
+def _make_scalar(scalar):
+    if isinstance(scalar, float):
+        return scalar
+    return nn.Parameter(torch.ones(1)) if scalar else 1
+
+
+class _SortNet(nn.Module):
+    """Input-box handling shared by the models; subclasses build `fc_dist` (and the head) and say whether the
+    distance stack works on flattened inputs."""
+
+    flatten_input = True
+
+    def _distance_features(self, x, eps, up, down):
+        certify = up is not None and down is not None and check_inf_and_eval(self)
+        paras = (x, torch.maximum(x - eps, down), torch.minimum(x + eps, up)) if certify else (x, None, None)
+        flat = lambda z: z.reshape(z.size(0), -1)
+        if self.flatten_input:
+            paras = apply_if_not_none(paras, flat)
+        paras = self.fc_dist(paras)
+        return apply_if_not_none(paras, flat)
+
+
+class SortMLPModel(_SortNet):
+    """Distance layers only; the negated last-layer distances are the logits (ell_inf_models.py:17-51)."""
+
+    def __init__(self, depth, width, input_dim, num_classes=10, dropout=0.7, std=1.0, identity_val=None, scalar=False,
+                 registry=None):
+        super().__init__()
+        kw = {"std": std, "identity_val": identity_val, "registry": registry}
+        pixels = input_dim[0] * input_dim[1] * input_dim[2]
+        stack = [NormDist(pixels, width, bias=False, mean_shift=True, **kw)]
+        stack += [NormDist(width, width, bias=False, mean_shift=True, dropout=dropout, **kw) for _ in range(depth - 2)]
+        stack.append(NormDist(width, num_classes, bias=True, mean_shift=False, dropout=dropout, **kw))
+        self.fc_dist = BoundSequential(*stack)
+        self.scalar = _make_scalar(scalar)
+
+    def forward(self, x=None, targets=None, eps=0, up=None, down=None):
+        dist, lower, upper = self._distance_features(x, eps, up, down)
+        if targets is None:
+            return -dist * self.scalar
+        lower = dist - eps if lower is None else lower
+        upper = dist + eps if upper is None else upper
+        # logits are negated distances: the largest rival logit against the smallest target logit
+        t = targets.view(-1, 1)
+        margin = (-lower) - torch.gather(-upper, 1, t)
+        margin = margin.scatter(1, t, 0)
+        return -dist * self.scalar, margin / (2 * eps)
+
+
+class _HybridNet(_SortNet):
+    """Distance stack, then BoundLinear + tanh, then the margin layer (ell_inf_models.py:54-96)."""
+
+    def _build_head(self, features, hidden, num_classes, scalar):
+        self.fc_linear = BoundSequential(BoundLinear(features, hidden, bias=True), BoundTanh())
+        self.fc_final = BoundFinalLinear(hidden, num_classes, bias=True)
+        self.scalar = _make_scalar(scalar)
+
+    def forward(self, x=None, targets=None, eps=0, up=None, down=None):
+        paras = self._distance_features(x, eps, up, down)
+        if targets is not None and (paras[1] is None or paras[2] is None):
+            paras = paras[0], paras[0] - eps, paras[0] + eps
+        paras = self.fc_linear(paras)
+        out = self.fc_final(*paras, targets=targets)
+        if targets is None:
+            return out * self.scalar
+        return out[0] * self.scalar, out[1]
+
+
+class SortHybridModel(_HybridNet):
+    def __init__(self, depth, width, input_dim, hidden=512, num_classes=10, dropout=0.7, std=1.0,
+                 identity_val=None, scalar=True, registry=None):
+        super().__init__()
+        kw = {"std": std, "identity_val": identity_val, "registry": registry}
+        pixels = input_dim[0] * input_dim[1] * input_dim[2]
+        stack = [NormDist(pixels, width, bias=False, mean_shift=True, **kw)]
+        stack += [NormDist(width, width, bias=False, mean_shift=True, dropout=dropout, **kw) for _ in range(depth - 3)]
+        self.fc_dist = BoundSequential(*stack)
+        self._build_head(width, hidden, num_classes, scalar)
+
+
+class SortHybridModel2(_HybridNet):
+    """First layer is a distance convolution with a (H - stride) x (W - stride) window and the given stride,
+    i.e. four positions; later layers are 1 x 1 (ell_inf_models.py:99-137)."""
+
+    flatten_input = False
+
+    def __init__(self, depth, width, input_dim, hidden=512, num_classes=10, dropout=0.7, stride=2, std=1.0,
+                 identity_val=None, scalar=True, registry=None):
+        super().__init__()
+        kw = {"std": std, "identity_val": identity_val, "registry": registry}
+        window = (input_dim[1] - stride, input_dim[2] - stride)
+        stack = [NormDistConv(input_dim[0], width, window, stride=stride, bias=False, mean_shift=True, **kw)]
+        stack += [NormDistConv(width, width, 1, bias=False, mean_shift=True, dropout=dropout, **kw)
+                  for _ in range(depth - 3)]
+        self.fc_dist = BoundSequential(*stack)
+        self._build_head(width * 4, hidden, num_classes, scalar)

@@ -1,0 +1,102 @@
+"""Interval-bound versions of the dense head that follows the distance layers in the hybrid models
+(core/models/bound_basic_module.py:11-103): ReLU / tanh, a linear layer and the final linear layer that
+returns worst-case margins against the target class.  Same constructor arguments, parameter names
+(`weight`, `bias`), scaling (`w_scale = w_lr / sqrt(in_features)`, `b_scale = b_lr`) and
+`(x, lower, upper)` protocol as the reference, so its checkpoints load.
+
+These layers are matrix products, so they run on the library GEMMs behind torch.  The one difference in
+formulation: the reference builds the (batch, classes, features) tensor `weight - weight[target]` for the
+margin radius; here samples are grouped by target class (one `(classes, features)` difference matrix and one
+GEMM per class present) or, with many classes, processed in bounded chunks, so memory stays O(classes x
+features) instead of O(batch x classes x features).
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as TF
+
+from .layers import apply_if_not_none
+
+
+class BoundReLU(nn.ReLU):
+    def forward(self, x=None, lower=None, upper=None):      # monotone: bounds map to bounds
+        return apply_if_not_none((x, lower, upper), TF.relu)
+
+
+class BoundTanh(nn.Tanh):
+    def forward(self, x=None, lower=None, upper=None):
+        return apply_if_not_none((x, lower, upper), torch.tanh)
+
+
+def _affine(inp, weight, bias, w_scale, b_scale):
+    if bias is None:
+        return torch.mm(inp, weight.t()) * w_scale
+    return torch.addmm(bias, inp, weight.t(), alpha=w_scale, beta=b_scale)
+
+
+class _ScaledLinear(nn.Linear):
+    """nn.Linear with N(0, w_scale^2) weights, zero bias and the reference's run-time scaling."""
+
+    def __init__(self, in_features, out_features, bias=True, w_scale=1.0, w_lr=1.0, b_lr=1.0):
+        super().__init__(in_features, out_features, bias=bias)
+        with torch.no_grad():
+            self.weight.normal_().mul_(w_scale)
+            if self.bias is not None:
+                self.bias.zero_()
+        self.w_scale = w_lr / math.sqrt(in_features)
+        self.b_scale = b_lr
+
+    def _center_radius(self, lower, upper):
+        center = (lower + upper) * 0.5
+        radius = (upper - lower) * 0.5
+        return _affine(center, self.weight, self.bias, self.w_scale, self.b_scale), radius
+
+
+class BoundLinear(_ScaledLinear):
+    """core/models/bound_basic_module.py:27-47: W c + b -/+ |W| r for the box of centre c and radius r."""
+
+    def forward(self, x=None, lower=None, upper=None):
+        if x is not None:
+            x = _affine(x, self.weight, self.bias, self.w_scale, self.b_scale)
+        if lower is not None and upper is not None:
+            z, radius = self._center_radius(lower, upper)
+            spread = torch.mm(radius, self.weight.abs().t()) * self.w_scale
+            lower, upper = z - spread, z + spread
+        return x, lower, upper
+
+
+class BoundFinalLinear(_ScaledLinear):
+    """core/models/bound_basic_module.py:79-103.  Without bounds or targets: the logits.  With both:
+    `(logits, res)`, `res[b, j]` = upper bound over the box of `logit_j - logit_target(b)` (0 at j = target)."""
+
+    group_by_class_upto = 32     # classes up to which samples are grouped by target class
+
+    def forward(self, x=None, lower=None, upper=None, targets=None):
+        if x is not None:
+            x = _affine(x, self.weight, self.bias, self.w_scale, self.b_scale)
+            if lower is None or upper is None or targets is None:
+                return x
+        res = None
+        if lower is not None and upper is not None and targets is not None:
+            z, radius = self._center_radius(lower, upper)
+            z = z - torch.gather(z, 1, targets.unsqueeze(1))
+            res = z + self._margin_radius(radius, targets) * self.w_scale
+        return x, res
+
+    def _margin_radius(self, radius, targets):
+        """sum_i |W[j, i] - W[target_b, i]| radius[b, i] for every sample b and class j."""
+        w = self.weight
+        out = radius.new_zeros(radius.size(0), w.size(0))
+        if w.size(0) <= self.group_by_class_upto:
+            for y in torch.unique(targets).tolist():
+                rows = (targets == y).nonzero(as_tuple=True)[0]
+                diff = (w - w[y]).abs()
+                out = out.index_add(0, rows, torch.mm(radius.index_select(0, rows), diff.t()))
+            return out
+        pieces = []
+        for start in range(0, radius.size(0), 64):
+            t = targets[start:start + 64]
+            diff = (w.unsqueeze(0) - w.index_select(0, t).unsqueeze(1)).abs()      # (chunk, classes, features)
+            pieces.append(torch.bmm(diff, radius[start:start + 64].unsqueeze(-1)).squeeze(-1))
+        return torch.cat(pieces)

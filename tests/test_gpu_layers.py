@@ -128,3 +128,52 @@ def test_conv_layer_shapes_and_value(oracle):
     ref = oracle.inf_dist_forward(cols, layer.weight.detach().cpu().numpy(), need_pos=False)
     assert np.array_equal(y.cpu().numpy().reshape(4, 8, 16), ref)
     assert bool((lo <= y).all()) and bool((y <= up).all())
+
+
+@pytest.mark.parametrize("kind", ["mlp", "hybrid", "hybrid_conv"])
+def test_model_zoo_modes(kind):
+    """The three uses of a model: training step through the index-list path, plain evaluation, and
+    certification with an input box.  Certified margins must dominate the margins at sampled points of the
+    box, and the 1-Lipschitz margins (no box) must dominate the certified ones' nominal margins as well."""
+    from sortnet_amd.ell_inf_models import SortMLPModel, SortHybridModel, SortHybridModel2
+    from sortnet_amd.layers import DropoutRegistry, set_mask_seed
+    dev = _dev()
+    reg = DropoutRegistry()
+    torch.manual_seed(3)
+    dims = (3, 8, 8)
+    if kind == "mlp":
+        net = SortMLPModel(4, 64, dims, num_classes=10, dropout=0.7, std=0.3, registry=reg)
+    elif kind == "hybrid":
+        net = SortHybridModel(5, 64, dims, hidden=32, num_classes=10, dropout=0.7, std=0.3, registry=reg)
+    else:
+        net = SortHybridModel2(5, 64, dims, hidden=32, num_classes=10, dropout=0.7, std=0.3, registry=reg)
+    net = net.to(dev)
+    B, eps = 70, 2.0 / 255
+    x = torch.rand(B, *dims, device=dev)
+    targets = torch.randint(0, 10, (B,), device=dev)
+    set_mask_seed(11, reg)
+    net.train()
+    logits = net(x)
+    assert logits.shape == (B, 10)
+    torch.nn.functional.cross_entropy(logits, targets).backward()
+    grads = [p.grad for p in net.parameters() if p.requires_grad]
+    assert all(g is not None and torch.isfinite(g).all() for g in grads)
+    # training-mode margins from the 1-Lipschitz ball around the distance features
+    logits2, margin = net(x, targets=targets, eps=eps)
+    assert margin.shape == (B, 10) and torch.isfinite(margin).all()
+    net.eval()
+    with torch.no_grad():
+        plain = net(x)
+        up, down = torch.ones_like(x), torch.zeros_like(x)
+        cl, certified = net(x, targets=targets, eps=eps, up=up, down=down)
+        torch.testing.assert_close(cl, plain, rtol=1e-5, atol=1e-6)
+        scale = 2 * eps if kind == "mlp" else 1.0                 # the MLP reports margins in units of 2 eps
+        g = torch.Generator().manual_seed(5)
+        for _ in range(5):
+            noise = (torch.rand(x.shape, generator=g) * 2 - 1).to(dev) * eps
+            xp = torch.minimum(torch.maximum(x + noise, down), up)
+            out = net(xp)
+            m = out - out.gather(1, targets.view(-1, 1))
+            s = net.scalar if not isinstance(net.scalar, (int, float)) else torch.tensor(float(net.scalar), device=dev)
+            assert bool((m <= certified * scale * s + 1e-4).all())
+        assert bool((certified.gather(1, targets.view(-1, 1)).abs() < 1e-6).all())

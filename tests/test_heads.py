@@ -1,0 +1,84 @@
+"""Interval-bound dense head (sortnet_amd.heads) against float64 interval arithmetic on the CPU: these layers
+are plain torch matrix products, so no GPU is needed."""
+import pytest
+import torch
+
+from sortnet_amd.heads import BoundFinalLinear, BoundLinear, BoundReLU, BoundTanh
+
+
+def _box(batch, features, seed, radius=0.1):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(batch, features, generator=g)
+    r = torch.rand(batch, features, generator=g) * radius
+    return x, x - r, x + r
+
+
+def test_bound_linear_matches_interval_arithmetic_and_contains_samples():
+    torch.manual_seed(0)
+    layer = BoundLinear(24, 10, bias=True, w_scale=0.7)
+    with torch.no_grad():
+        layer.bias.normal_()
+    x, lo, up = _box(6, 24, 1)
+    y, ylo, yup = layer(x, lo, up)
+    w = layer.weight.double() * layer.w_scale
+    b = layer.bias.double() * layer.b_scale
+    pos, neg = w.clamp(min=0), w.clamp(max=0)
+    ref_lo = lo.double() @ pos.t() + up.double() @ neg.t() + b
+    ref_up = up.double() @ pos.t() + lo.double() @ neg.t() + b
+    torch.testing.assert_close(ylo.double(), ref_lo, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(yup.double(), ref_up, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(y.double(), x.double() @ w.t() + b, rtol=1e-5, atol=1e-5)
+    g = torch.Generator().manual_seed(2)
+    for _ in range(20):
+        p = lo + (up - lo) * torch.rand(lo.shape, generator=g)
+        out = layer(p)[0]
+        assert bool((out >= ylo - 1e-5).all()) and bool((out <= yup + 1e-5).all())
+    assert layer(x)[1] is None and layer(None, lo, up)[0] is None
+
+
+def test_monotone_activations_map_bounds():
+    x, lo, up = _box(4, 7, 3)
+    for act, fn in ((BoundTanh(), torch.tanh), (BoundReLU(), torch.relu)):
+        y, ylo, yup = act(x, lo, up)
+        assert torch.equal(y, fn(x)) and torch.equal(ylo, fn(lo)) and torch.equal(yup, fn(up))
+        assert bool((ylo <= y).all()) and bool((y <= yup).all())
+
+
+@pytest.mark.parametrize("classes", [10, 40])      # grouped by target class / chunked
+def test_final_linear_margins(classes):
+    torch.manual_seed(1)
+    layer = BoundFinalLinear(16, classes, bias=True)
+    with torch.no_grad():
+        layer.bias.normal_()
+    batch = 70
+    x, lo, up = _box(batch, 16, 4)
+    targets = torch.randint(0, classes, (batch,), generator=torch.Generator().manual_seed(5))
+    logits, res = layer(x, lo, up, targets=targets)
+    w = layer.weight.double() * layer.w_scale
+    b = layer.bias.double() * layer.b_scale
+    dw = w.unsqueeze(0) - w[targets].unsqueeze(1)                    # (batch, classes, features)
+    db = b.unsqueeze(0) - b[targets].unsqueeze(1)
+    c, r = (lo.double() + up.double()) / 2, (up.double() - lo.double()) / 2
+    ref = torch.einsum("bjf,bf->bj", dw, c) + db + torch.einsum("bjf,bf->bj", dw.abs(), r)
+    torch.testing.assert_close(res.double(), ref, rtol=1e-5, atol=1e-5)
+    assert bool((res.gather(1, targets.unsqueeze(1)).abs() < 1e-5).all())
+    # the bound dominates the margin at any point of the box
+    g = torch.Generator().manual_seed(6)
+    for _ in range(10):
+        p = lo + (up - lo) * torch.rand(lo.shape, generator=g)
+        out = layer(p)
+        margin = out - out.gather(1, targets.unsqueeze(1))
+        assert bool((margin <= res + 1e-4).all())
+    torch.testing.assert_close(logits, layer(x))
+    # both formulations of the radius term agree
+    layer.group_by_class_upto = 0 if classes <= 32 else 1000
+    torch.testing.assert_close(layer(x, lo, up, targets=targets)[1], res, rtol=1e-5, atol=1e-5)
+
+
+def test_final_linear_is_differentiable():
+    layer = BoundFinalLinear(8, 5)
+    x, lo, up = _box(9, 8, 7)
+    targets = torch.arange(9) % 5
+    _, res = layer(x, lo, up, targets=targets)
+    res.sum().backward()
+    assert layer.weight.grad is not None and torch.isfinite(layer.weight.grad).all()
