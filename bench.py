@@ -39,6 +39,10 @@ def parse():
     ap.add_argument("--eps", type=float, default=8.0 / 255)
     ap.add_argument("--mask", choices=["term", "factored"], default="factored",
                     help="granularity of the Bernoulli keep mask of the masked neuron")
+    ap.add_argument("--workload", choices=["masked", "index-lists"], default="masked",
+                    help="masked: the headline step (fused masked neuron).  index-lists: the reference's own training "
+                         "form (kept-channel lists per 32-sample sub-batch, SortMLPModel) plus its certification pass "
+                         "(sort neuron and interval sort neuron); a secondary figure, without roofline / cpu_baseline")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain device copy of a width x width fp32 matrix after the timed steps "
@@ -88,12 +92,70 @@ def cpu_baseline(args, model_dims):
                       "bounds of all %d layers; no optimizer), %.1f s" % (nb, len(ws), t)}
 
 
+def index_list_workload(args):
+    """Training step of SortMLPModel in the reference's index-list form and the certification pass of the same
+    model in evaluation mode (sort neuron for the value, interval sort neuron for the bounds)."""
+    import torch
+    from sortnet_amd.ell_inf_models import SortMLPModel
+    from sortnet_amd.layers import DropoutRegistry, set_mask_seed
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    reg = DropoutRegistry()
+    torch.manual_seed(0)
+    side = int(round((args.in_features / 3) ** 0.5))
+    assert 3 * side * side == args.in_features, "--in-features must be 3 x side x side for this workload"
+    net = SortMLPModel(args.depth, args.width, (3, side, side), num_classes=args.classes, dropout=args.q,
+                       registry=reg).to(dev)
+    opt = torch.optim.AdamW(net.parameters(), lr=1e-4, fused=True)
+    g = torch.Generator().manual_seed(0)
+    x = torch.rand(args.batch, 3, side, side, generator=g).to(dev)
+    t = torch.randint(0, args.classes, (args.batch,), generator=g).to(dev)
+    up, down = torch.ones_like(x), torch.zeros_like(x)
+    set_mask_seed(1, reg)
+
+    def train_step():
+        net.train()
+        loss = torch.nn.functional.cross_entropy(net(x), t)
+        opt.zero_grad(set_to_none=True)
+        loss.backward()
+        opt.step()
+
+    def certify():
+        net.eval()
+        with torch.no_grad():
+            return net(x, targets=t, eps=args.eps, up=up, down=down)
+
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+
+    for _ in range(args.warmup):
+        train_step()
+    step_s = timed(train_step, args.steps)
+    certify()
+    cert_s = timed(certify, max(2, args.steps // 4))
+    print(json.dumps({
+        "metric": "train samples/s, SortMLPModel in the reference's index-list form", "value": args.batch / step_s,
+        "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": step_s * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "SortMLPModel depth %d width %d, B=%d, keep probability %.2f: forward + cross entropy + "
+                               "backward + AdamW through kept-channel index lists" % (args.depth, args.width, args.batch, args.q)},
+        "certification_ms": cert_s * 1e3,
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collective path exists); run with --gpus 1",
               file=sys.stderr)
         sys.exit(2)
+    if args.workload == "index-lists":
+        return index_list_workload(args)
     import torch
     from sortnet_amd import ext
     from sortnet_amd.model import DistanceMLP, margins, hinge_loss
