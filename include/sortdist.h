@@ -21,6 +21,12 @@
  * scatters into (grad_input, grad_weight), as the reference launchers do, and owns no
  * caller-visible memory.  pos packs the arg-max input index in bits 0..30 and a branch/sign
  * flag in bit 31.
+ *
+ * Scratch memory: the library keeps one device buffer per GPU for partial results (split
+ * reductions, mask bits, candidate lists, per-slice sums) and grows it on demand with
+ * hipMalloc; growing waits for the device to go idle first.  Calls are asynchronous on
+ * `stream`, but two calls that use the buffer must not overlap on different streams of one
+ * GPU.  Outputs that are zero-filled or merged with 128-bit stores must be 16-byte aligned.
  */
 #ifndef SORTDIST_H
 #define SORTDIST_H

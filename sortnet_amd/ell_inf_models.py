@@ -75,13 +75,17 @@ class SortMLPModel(_SortNet):
 class _HybridNet(_SortNet):
     """Distance stack, then BoundLinear + tanh, then the margin layer (ell_inf_models.py:54-96)."""
 
+    @staticmethod
+    def _pool(z):      # hook between the distance stack and the head
+        return z
+
     def _build_head(self, features, hidden, num_classes, scalar):
         self.fc_linear = BoundSequential(BoundLinear(features, hidden, bias=True), BoundTanh())
         self.fc_final = BoundFinalLinear(hidden, num_classes, bias=True)
         self.scalar = _make_scalar(scalar)
 
     def forward(self, x=None, targets=None, eps=0, up=None, down=None):
-        paras = self._distance_features(x, eps, up, down)
+        paras = apply_if_not_none(self._distance_features(x, eps, up, down), self._pool)
         if targets is not None and (paras[1] is None or paras[2] is None):
             paras = paras[0], paras[0] - eps, paras[0] + eps
         paras = self.fc_linear(paras)
@@ -108,6 +112,7 @@ class SortHybridModel2(_HybridNet):
     i.e. four positions; later layers are 1 x 1 (ell_inf_models.py:99-137)."""
 
     flatten_input = False
+    head_inputs_per_channel = 4
 
     def __init__(self, depth, width, input_dim, hidden=512, num_classes=10, dropout=0.7, stride=2, std=1.0,
                  identity_val=None, scalar=True, registry=None):
@@ -118,4 +123,15 @@ class SortHybridModel2(_HybridNet):
         stack += [NormDistConv(width, width, 1, bias=False, mean_shift=True, dropout=dropout, **kw)
                   for _ in range(depth - 3)]
         self.fc_dist = BoundSequential(*stack)
-        self._build_head(width * 4, hidden, num_classes, scalar)
+        self._build_head(width * self.head_inputs_per_channel, hidden, num_classes, scalar)
+
+
+class SortHybridModelAvg(SortHybridModel2):
+    """SortHybridModel2 whose head sees the mean over the four window positions of every channel instead of
+    all of them (ell_inf_models.py:131-164); means of bounds are bounds of the mean."""
+
+    head_inputs_per_channel = 1
+
+    @staticmethod
+    def _pool(z):
+        return z.view(z.size(0), -1, 4).mean(dim=2)

@@ -1,6 +1,6 @@
 """Interval-bound versions of the dense head that follows the distance layers in the hybrid models
-(core/models/bound_basic_module.py:11-103): ReLU / tanh, a linear layer and the final linear layer that
-returns worst-case margins against the target class.  Same constructor arguments, parameter names
+(core/models/bound_basic_module.py:11-103): ReLU / tanh, a linear layer, a convolution and the final linear
+layer that returns worst-case margins against the target class.  Same constructor arguments, parameter names
 (`weight`, `bias`), scaling (`w_scale = w_lr / sqrt(in_features)`, `b_scale = b_lr`) and
 `(x, lower, upper)` protocol as the reference, so its checkpoints load.
 
@@ -62,6 +62,38 @@ class BoundLinear(_ScaledLinear):
         if lower is not None and upper is not None:
             z, radius = self._center_radius(lower, upper)
             spread = torch.mm(radius, self.weight.abs().t()) * self.w_scale
+            lower, upper = z - spread, z + spread
+        return x, lower, upper
+
+
+class BoundConv2d(nn.Conv2d):
+    """core/models/bound_basic_module.py:50-76: the convolution counterpart of BoundLinear, with
+    `w_scale = w_lr / sqrt(in_channels * kernel_size^2)`; the box is propagated as centre and radius
+    (radius through |W|, no bias)."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1, groups=1, bias=True,
+                 w_scale=1.0, w_lr=1.0, b_lr=1.0):
+        super().__init__(in_channels, out_channels, kernel_size, stride=stride, padding=padding, dilation=dilation,
+                         groups=groups, bias=bias)
+        with torch.no_grad():
+            self.weight.normal_().mul_(w_scale)
+            if self.bias is not None:
+                self.bias.zero_()
+        self.w_scale = w_lr / math.sqrt(in_channels * kernel_size * kernel_size)
+        self.b_scale = b_lr
+
+    def _conv(self, inp, weight, with_bias):
+        bias = self.bias * self.b_scale if with_bias and self.bias is not None else None
+        return TF.conv2d(inp, weight, bias, stride=self.stride, padding=self.padding, dilation=self.dilation,
+                         groups=self.groups)
+
+    def forward(self, x=None, lower=None, upper=None):
+        if x is not None:
+            x = self._conv(x, self.weight * self.w_scale, True)
+        if lower is not None and upper is not None:
+            half = self.w_scale / 2
+            z = self._conv(lower + upper, self.weight * half, True)
+            spread = self._conv(upper - lower, self.weight.abs() * half, False)
             lower, upper = z - spread, z + spread
         return x, lower, upper
 

@@ -130,12 +130,12 @@ def test_conv_layer_shapes_and_value(oracle):
     assert bool((lo <= y).all()) and bool((y <= up).all())
 
 
-@pytest.mark.parametrize("kind", ["mlp", "hybrid", "hybrid_conv"])
+@pytest.mark.parametrize("kind", ["mlp", "hybrid", "hybrid_conv", "hybrid_avg"])
 def test_model_zoo_modes(kind):
-    """The three uses of a model: training step through the index-list path, plain evaluation, and
+    """The three uses of a model of every family: training step through the index-list path, plain evaluation, and
     certification with an input box.  Certified margins must dominate the margins at sampled points of the
     box, and the 1-Lipschitz margins (no box) must dominate the certified ones' nominal margins as well."""
-    from sortnet_amd.ell_inf_models import SortMLPModel, SortHybridModel, SortHybridModel2
+    from sortnet_amd.ell_inf_models import SortMLPModel, SortHybridModel, SortHybridModel2, SortHybridModelAvg
     from sortnet_amd.layers import DropoutRegistry, set_mask_seed
     dev = _dev()
     reg = DropoutRegistry()
@@ -145,8 +145,11 @@ def test_model_zoo_modes(kind):
         net = SortMLPModel(4, 64, dims, num_classes=10, dropout=0.7, std=0.3, registry=reg)
     elif kind == "hybrid":
         net = SortHybridModel(5, 64, dims, hidden=32, num_classes=10, dropout=0.7, std=0.3, registry=reg)
-    else:
+    elif kind == "hybrid_conv":
         net = SortHybridModel2(5, 64, dims, hidden=32, num_classes=10, dropout=0.7, std=0.3, registry=reg)
+    else:
+        net = SortHybridModelAvg(5, 64, dims, hidden=32, num_classes=10, dropout=0.7, std=0.3, registry=reg)
+        assert net.fc_linear[0].in_features == 64
     net = net.to(dev)
     B, eps = 70, 2.0 / 255
     x = torch.rand(B, *dims, device=dev)

@@ -3,7 +3,7 @@ are plain torch matrix products, so no GPU is needed."""
 import pytest
 import torch
 
-from sortnet_amd.heads import BoundFinalLinear, BoundLinear, BoundReLU, BoundTanh
+from sortnet_amd.heads import BoundConv2d, BoundFinalLinear, BoundLinear, BoundReLU, BoundTanh
 
 
 def _box(batch, features, seed, radius=0.1):
@@ -82,3 +82,28 @@ def test_final_linear_is_differentiable():
     _, res = layer(x, lo, up, targets=targets)
     res.sum().backward()
     assert layer.weight.grad is not None and torch.isfinite(layer.weight.grad).all()
+
+
+def test_bound_conv2d_matches_interval_arithmetic_and_contains_samples():
+    torch.manual_seed(2)
+    layer = BoundConv2d(3, 5, 3, stride=2, padding=1, bias=True, w_scale=0.5)
+    with torch.no_grad():
+        layer.bias.normal_()
+    assert abs(layer.w_scale - 1.0 / (3 * 3 * 3) ** 0.5) < 1e-12
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(4, 3, 9, 9, generator=g)
+    r = torch.rand(4, 3, 9, 9, generator=g) * 0.2
+    lo, up = x - r, x + r
+    y, ylo, yup = layer(x, lo, up)
+    w = layer.weight.double() * layer.w_scale
+    b = layer.bias.double() * layer.b_scale
+    conv = lambda inp, k, bias=None: torch.nn.functional.conv2d(inp.double(), k, bias, stride=2, padding=1)
+    pos, neg = w.clamp(min=0), w.clamp(max=0)
+    torch.testing.assert_close(y.double(), conv(x, w, b), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(ylo.double(), conv(lo, pos, b) + conv(up, neg), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(yup.double(), conv(up, pos, b) + conv(lo, neg), rtol=1e-5, atol=1e-5)
+    for _ in range(10):
+        p = lo + (up - lo) * torch.rand(lo.shape, generator=g)
+        out = layer(p)[0]
+        assert bool((out >= ylo - 1e-5).all()) and bool((out <= yup + 1e-5).all())
+    assert layer(x)[1] is None and layer(None, lo, up)[0] is None
