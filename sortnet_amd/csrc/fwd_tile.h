@@ -833,93 +833,111 @@ struct LpWithMax : PolicyBase {
 
 
 // -------------------------------------------------------------------------------------------
-// resolve_pos_kernel: one work-item per output.  Reads the winning (value, chunk) pair left by a
-// chunk-tracking policy (from y/pos when the reduction was not split, else from the packed
-// workspace), rescans that chunk in ascending input order for the first kept term whose
-// magnitude equals the value bit for bit, and writes the final value and position.
+// resolve_pos_kernel: a wavefront owns 64 consecutive outputs.  Each lane first reads the winning
+// (value, chunk) pair of its own output left by a chunk-tracking policy (from y/pos when the reduction
+// was not split, else from the packed workspace) and posts the row offsets and keep information
+// of that output in LDS.  The wavefront then walks its outputs two at a time, 32 lanes per output and
+// one input of the winning chunk per lane, so that a chunk is fetched with one coalesced load per
+// operand instead of one cache line per lane; a ballot finds the first kept input whose magnitude equals
+// the value bit for bit, and the owner lane writes the final value and position.
 // -------------------------------------------------------------------------------------------
+struct ResolveSlot { int cid; float best; int xoff, woff, coff; uint32_t keep; int pad0, pad1; };
+
+// keep bits of the 32 inputs of chunk `cid` of output `o` (input row xrow, weight row c) under the active mask mode
+__device__ __forceinline__ uint32_t chunk_keep_bits(const FwdArgs& a, long long o, int xrow, int c, int cid, int nchunks) {
+    if (a.mask_mode == SD_MASK_TERM) {
+        const uint32_t key_t = rng_row_key(a.seed, 0u, (uint32_t)o);
+        uint32_t keep = 0u;
+        #pragma unroll
+        for (int q4 = 0; q4 < KT / 4; q4++) {
+            const uint32_t word = rng_word(key_t, (uint32_t)(cid * (KT / 4) + q4));
+            #pragma unroll
+            for (int c4 = 0; c4 < 4; c4++)
+                if (((word >> (8 * c4)) & 0xffu) < a.t8) keep |= 1u << (q4 * 4 + c4);
+        }
+        return keep;
+    }
+    if (a.mask_mode == SD_MASK_FACTORED) {
+        if (a.xmask) return a.xmask[(size_t)xrow * nchunks + cid] & a.wmask[(size_t)c * nchunks + cid];
+        const uint32_t key_x = rng_row_key(a.seed, 1u, (uint32_t)xrow), key_w = rng_row_key(a.seed, 2u, (uint32_t)c);
+        uint32_t keep = 0u;
+        for (int k = 0; k < KT; k++) {
+            const uint32_t n = (uint32_t)(cid * KT + k);
+            if ((rng_word(key_x, n) >> 16) < a.t16 && (rng_word(key_w, n) >> 16) < a.t16) keep |= 1u << k;
+        }
+        return keep;
+    }
+    return 0xffffffffu;
+}
+
 template <bool PACKED>
 __global__ void __launch_bounds__(256) resolve_pos_kernel(FwdArgs a) {
-    long long total = (long long)a.R * a.G * a.COg;
-    long long o = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (o >= total) return;
-    int hw = (int)(o % a.HW);
-    long long t = o / a.HW;
-    int c = (int)(t % (a.G * a.COg));
-    int b = (int)(t / (a.G * a.COg));
-    int g = c / a.COg, m = c - g * a.COg;
-    float best; int cid;
-    if (PACKED) {
-        unsigned long long v = a.packed0[o];
-        uint32_t low = (uint32_t)v;
-        best = low ? __uint_as_float((uint32_t)(v >> 32)) : kEps;
-        cid = low ? (int)(0xffffffffu - low) : -1;
-    } else { best = a.y0[o]; cid = a.p0[o]; }
-    int pos = 0;
-    if (cid >= 0) {
-        const int s = b / kSubBatch;
-        const int wrow = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + m] : m;
-        const float* wr = a.w + (size_t)(g * a.W_COg + wrow) * a.W_CIg;
-        const float* xr = a.x0 + ((size_t)(b * a.G + g) * a.CIg) * a.HW + hw;
-        const int* cidx = a.ci_idx ? a.ci_idx + (size_t)(s * a.G + g) * a.CIg : nullptr;
-        const int n0 = cid * KT;
-        // keep bits of the 32 inputs of the chunk
-        uint32_t keep = 0xffffffffu;
-        if (a.mask_mode == SD_MASK_TERM) {
-            const uint32_t key_t = rng_row_key(a.seed, 0u, (uint32_t)o);
-            keep = 0u;
-            #pragma unroll
-            for (int q4 = 0; q4 < KT / 4; q4++) {
-                uint32_t word = rng_word(key_t, (uint32_t)(n0 >> 2) + q4);
-                #pragma unroll
-                for (int c4 = 0; c4 < 4; c4++)
-                    if (((word >> (8 * c4)) & 0xffu) < a.t8) keep |= 1u << (q4 * 4 + c4);
-            }
-        } else if (a.mask_mode == SD_MASK_FACTORED) {
-            if (a.xmask) {
-                const int nchunks = (a.CIg + KT - 1) / KT;
-                keep = a.xmask[(size_t)((b * a.G + g) * a.HW + hw) * nchunks + cid] & a.wmask[(size_t)c * nchunks + cid];
-            } else {
-                const uint32_t key_x = rng_row_key(a.seed, 1u, (uint32_t)((b * a.G + g) * a.HW + hw));
-                const uint32_t key_w = rng_row_key(a.seed, 2u, (uint32_t)c);
-                keep = 0u;
-                for (int k = 0; k < KT; k++)
-                    if ((rng_word(key_x, (uint32_t)(n0 + k)) >> 16) < a.t16 && (rng_word(key_w, (uint32_t)(n0 + k)) >> 16) < a.t16)
-                        keep |= 1u << k;
-            }
+    __shared__ __attribute__((aligned(16))) ResolveSlot slots[4][64];
+    const long long total = (long long)a.R * a.G * a.COg;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long long o_base = ((long long)blockIdx.x * 4 + wave) * 64;
+    if (o_base >= total) return;                       // whole wavefront; no workgroup barrier below
+    const long long o = o_base + lane;
+    const bool mine = o < total;
+    ResolveSlot me;
+    me.cid = -1; me.best = kEps; me.xoff = me.woff = me.coff = 0; me.keep = 0u; me.pad0 = me.pad1 = 0;
+    if (mine) {
+        const int hw = (int)(o % a.HW);
+        const long long t = o / a.HW;
+        const int c = (int)(t % (a.G * a.COg));
+        const int b = (int)(t / (a.G * a.COg));
+        const int g = c / a.COg, m = c - g * a.COg;
+        if (PACKED) {
+            unsigned long long v = a.packed0[o];
+            uint32_t low = (uint32_t)v;
+            me.best = low ? __uint_as_float((uint32_t)(v >> 32)) : kEps;
+            me.cid = low ? (int)(0xffffffffu - low) : -1;
+        } else { me.best = a.y0[o]; me.cid = a.p0[o]; }
+        if (me.cid >= 0) {
+            const int s = b / kSubBatch;
+            const int wrow = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + m] : m;
+            me.woff = (g * a.W_COg + wrow) * a.W_CIg;
+            me.xoff = (b * a.G + g) * a.CIg * a.HW + hw;
+            me.coff = (s * a.G + g) * a.CIg;
+            me.keep = chunk_keep_bits(a, o, (b * a.G + g) * a.HW + hw, c, me.cid, (a.CIg + KT - 1) / KT);
         }
-        if (a.fast_x && a.fast_w) {
-            // 128-bit loads of the whole chunk, then a branch-free scan from the top so that the
-            // lowest matching input is the one that remains
-            float4 xv[KT / 4], wv[KT / 4];
-            #pragma unroll
-            for (int q4 = 0; q4 < KT / 4; q4++) {
-                int n = n0 + 4 * q4;
-                if (n > a.CIg - 4) n = a.CIg - 4;
-                xv[q4] = *reinterpret_cast<const float4*>(xr + n);
-                wv[q4] = *reinterpret_cast<const float4*>(wr + n);
-            }
-            #pragma unroll
-            for (int q4 = KT / 4 - 1; q4 >= 0; q4--) {
-                const int n = n0 + 4 * q4;
-                const bool in = n < a.CIg;
-                float d3 = xv[q4].w - wv[q4].w, d2 = xv[q4].z - wv[q4].z, d1 = xv[q4].y - wv[q4].y, d0 = xv[q4].x - wv[q4].x;
-                uint32_t kb = keep >> (4 * q4);
-                if (in && (kb & 8u) && fabsf(d3) == best) pos = (n + 3) | (d3 < 0.f ? (int)kSign : 0);
-                if (in && (kb & 4u) && fabsf(d2) == best) pos = (n + 2) | (d2 < 0.f ? (int)kSign : 0);
-                if (in && (kb & 2u) && fabsf(d1) == best) pos = (n + 1) | (d1 < 0.f ? (int)kSign : 0);
-                if (in && (kb & 1u) && fabsf(d0) == best) pos = n | (d0 < 0.f ? (int)kSign : 0);
-            }
-        } else {
-            const int n1 = n0 + KT < a.CIg ? n0 + KT : a.CIg;
-            for (int n = n0; n < n1; n++) {
-                float d = xr[(size_t)n * a.HW] - wr[cidx ? cidx[n] : n];
-                if (((keep >> (n - n0)) & 1u) && fabsf(d) == best) { pos = n | (d < 0.f ? (int)kSign : 0); break; }
+    }
+    slots[wave][lane] = me;
+    __builtin_amdgcn_wave_barrier();                   // LDS operations of one wavefront complete in order
+
+    // slots without a winning chunk keep offset 0 and keep bits 0: their loads hit element 0 and never match
+    constexpr int U = 8;
+    const int half = lane >> 5, l = lane & 31;
+    int pos = 0;
+    for (int it0 = 0; it0 < 32; it0 += U) {
+        float d[U];
+        bool cand[U];
+        float best[U];
+        #pragma unroll
+        for (int u = 0; u < U; u++) {
+            const ResolveSlot q = slots[wave][2 * (it0 + u) + half];
+            int n = (q.cid < 0 ? 0 : q.cid) * KT + l;
+            cand[u] = n < a.CIg && ((q.keep >> l) & 1u) != 0u;
+            if (n >= a.CIg) n = 0;
+            const int col = a.ci_idx ? a.ci_idx[q.coff + n] : n;
+            d[u] = a.x0[(size_t)q.xoff + (size_t)n * a.HW] - a.w[q.woff + col];
+            best[u] = q.best;
+        }
+        #pragma unroll
+        for (int u = 0; u < U; u++) {
+            const unsigned long long hit = __ballot(cand[u] && fabsf(d[u]) == best[u]);
+            const unsigned long long neg = __ballot(d[u] < 0.f);
+            if ((lane >> 1) == it0 + u) {              // the two owner lanes of this step
+                const uint32_t h32 = (lane & 1) ? (uint32_t)(hit >> 32) : (uint32_t)hit;
+                const uint32_t n32 = (lane & 1) ? (uint32_t)(neg >> 32) : (uint32_t)neg;
+                if (h32) {
+                    const int first = __ffs((int)h32) - 1;
+                    pos = (me.cid * KT + first) | (((n32 >> first) & 1u) ? (int)kSign : 0);
+                }
             }
         }
     }
-    a.y0[o] = best;
-    a.p0[o] = pos;
+    if (mine) { a.y0[o] = me.best; a.p0[o] = pos; }
 }
 
 // Position resolve of the interval kernel: rescans the winning chunk of the lower and of the upper

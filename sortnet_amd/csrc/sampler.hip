@@ -15,47 +15,101 @@ __host__ __device__ __forceinline__ unsigned long long sample_key(uint32_t rowke
     return ((unsigned long long)rng_word(rowkey, c) << 16) | (unsigned long long)c;
 }
 
+// sum of one wave-uniform value per wavefront over the four wavefronts of a workgroup.  `part` holds one slot
+// per wavefront and call parity, so one barrier per call is enough.
+__device__ __forceinline__ int block_sum_uniform(int v, int (*part)[4], int parity) {
+    if ((threadIdx.x & 63) == 0) part[parity][threadIdx.x >> 6] = v;
+    __syncthreads();
+    return part[parity][0] + part[parity][1] + part[parity][2] + part[parity][3];
+}
+__device__ __forceinline__ int wave_sum(int v) {
+    #pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+// exclusive prefix over the 256 work-items in work-item order
+__device__ __forceinline__ int block_exclusive_scan(int mine, int* wave_total) {
+    const int tid = threadIdx.x;
+    int incl = mine;
+    #pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int v = __shfl_up(incl, off);
+        if ((tid & 63) >= off) incl += v;
+    }
+    if ((tid & 63) == 63) wave_total[tid >> 6] = incl;
+    __syncthreads();
+    int before = incl - mine;
+    for (int w = 0; w < (tid >> 6); w++) before += wave_total[w];
+    return before;
+}
+
+// One workgroup per (sub-batch, group); work-item t owns the channels [t * per, (t + 1) * per).
+// The `count` smallest 48-bit keys (word << 16 | channel) are the keys whose word is below the count-th smallest
+// word w, plus the lowest channels among the keys whose word equals w.
+//
+// CACHED (C <= 256 * kCached): the words stay in registers; w is found by bisection over the 32-bit word range
+// with one ballot and population count per register slot, and ties on w are ranked by the ordered scan.
+// Otherwise the words are recomputed and the threshold is found by bisection over the whole 48-bit key range.
+constexpr int kCached = 32;
+
+template <bool CACHED>
 __global__ void __launch_bounds__(256) sample_index_lists_kernel(uint32_t seed, int C, int count, int* __restrict__ out) {
-    __shared__ int red[256];
-    __shared__ unsigned long long s_lo, s_hi;
+    __shared__ int part[2][4];
+    __shared__ int wave_total[4];
     const int tid = threadIdx.x;
     const uint32_t rowkey = rng_row_key(seed, 4u, blockIdx.x);
-    // smallest T with #{keys < T} >= count, by bisection on the 48-bit key range (keys are distinct)
-    if (tid == 0) { s_lo = 0ull; s_hi = 1ull << 48; }
-    __syncthreads();
-    for (int it = 0; it < 48; it++) {
-        const unsigned long long lo = s_lo, hi = s_hi;
-        const unsigned long long mid = lo + ((hi - lo) >> 1);
-        int cnt = 0;
-        for (int c = tid; c < C; c += 256) cnt += sample_key(rowkey, (uint32_t)c) < mid ? 1 : 0;
-        red[tid] = cnt;
-        __syncthreads();
-        for (int s = 128; s > 0; s >>= 1) {
-            if (tid < s) red[tid] += red[tid + s];
-            __syncthreads();
-        }
-        if (tid == 0) {
-            if (red[0] >= count) s_hi = mid; else s_lo = mid + 1;
-        }
-        __syncthreads();
-    }
-    const unsigned long long T = s_hi;    // #{keys < T} == count
-    // ordered compaction: work-item t owns channels [t * per, (t + 1) * per)
     const int per = (C + 255) / 256;
     const int c0 = tid * per, c1 = c0 + per < C ? c0 + per : C;
-    int mine = 0;
-    for (int c = c0; c < c1; c++) mine += sample_key(rowkey, (uint32_t)c) < T ? 1 : 0;
-    red[tid] = mine;
-    __syncthreads();
-    if (tid == 0) {
-        int run = 0;
-        for (int t = 0; t < 256; t++) { int v = red[t]; red[t] = run; run += v; }
-    }
-    __syncthreads();
-    int pos = red[tid];
     int* dst = out + (size_t)blockIdx.x * count;
-    for (int c = c0; c < c1; c++)
-        if (sample_key(rowkey, (uint32_t)c) < T) dst[pos++] = c;
+    if (CACHED) {
+        uint32_t word[kCached];
+        #pragma unroll
+        for (int i = 0; i < kCached; i++) word[i] = rng_word(rowkey, (uint32_t)(c0 + i));
+        // smallest w with #{word <= w} >= count
+        uint32_t lo = 0u, hi = 0xffffffffu;
+        for (int it = 0; it < 32; it++) {
+            const uint32_t mid = lo + ((hi - lo) >> 1);
+            int cnt = 0;
+            #pragma unroll
+            for (int i = 0; i < kCached; i++) cnt += __popcll(__ballot(c0 + i < c1 && word[i] <= mid));
+            if (block_sum_uniform(cnt, part, it & 1) >= count) hi = mid; else lo = mid + 1u;
+        }
+        const uint32_t w = hi;
+        int below = 0, ties = 0;
+        #pragma unroll
+        for (int i = 0; i < kCached; i++) {
+            below += (c0 + i < c1 && word[i] < w) ? 1 : 0;
+            ties += (c0 + i < c1 && word[i] == w) ? 1 : 0;
+        }
+        const int all_below = block_sum_uniform(wave_sum(below), part, 0);     // parity 0 was last written 2 calls ago
+        const int take = count - all_below;                                    // ties to keep, >= 1
+        const int before = block_exclusive_scan(below | (ties << 16), wave_total);
+        int tie_rank = before >> 16;
+        int pos = (before & 0xffff) + (tie_rank < take ? tie_rank : take);
+        #pragma unroll
+        for (int i = 0; i < kCached; i++) {
+            if (c0 + i < c1) {
+                bool keep = word[i] < w;
+                if (word[i] == w) keep = tie_rank++ < take;
+                if (keep) dst[pos++] = c0 + i;
+            }
+        }
+    } else {
+        auto below = [&](unsigned long long T) {
+            int cnt = 0;
+            for (int c = c0; c < c1; c++) cnt += sample_key(rowkey, (uint32_t)c) < T ? 1 : 0;
+            return cnt;
+        };
+        // smallest T with #{keys < T} >= count (keys are distinct); every work-item follows the same interval
+        unsigned long long lo = 0ull, hi = 1ull << 48;
+        for (int it = 0; it < 48; it++) {
+            const unsigned long long mid = lo + ((hi - lo) >> 1);
+            if (block_sum_uniform(wave_sum(below(mid)), part, it & 1) >= count) hi = mid; else lo = mid + 1;
+        }
+        int pos = block_exclusive_scan(below(hi), wave_total);
+        for (int c = c0; c < c1; c++)
+            if (sample_key(rowkey, (uint32_t)c) < hi) dst[pos++] = c;
+    }
 }
 
 }  // namespace sd
@@ -79,7 +133,11 @@ extern "C" int sd_sample_index_lists(uint32_t seed, int S, int G, int C, int cou
     SD_REQUIRE(count >= 0 && count <= C, "sample_index_lists: count=%d outside 0..C=%d", count, C);
     if (count == 0) return SD_OK;
     SD_REQUIRE(out, "sample_index_lists: null output");
-    hipLaunchKernelGGL(sample_index_lists_kernel, dim3(S * G), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       seed, C, count, out);
+    if (C <= 256 * kCached)
+        hipLaunchKernelGGL(sample_index_lists_kernel<true>, dim3(S * G), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           seed, C, count, out);
+    else
+        hipLaunchKernelGGL(sample_index_lists_kernel<false>, dim3(S * G), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           seed, C, count, out);
     return check_launch("sample_index_lists_kernel");
 }

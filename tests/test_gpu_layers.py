@@ -14,7 +14,8 @@ def _dev():
     return torch.device("cuda:0")
 
 
-@pytest.mark.parametrize("S,G,C,q", [(3, 1, 100, 0.3), (2, 2, 64, 0.75), (16, 1, 5120, 0.3), (1, 1, 7, 1.0)])
+@pytest.mark.parametrize("S,G,C,q", [(3, 1, 100, 0.3), (2, 2, 64, 0.75), (16, 1, 5120, 0.3), (1, 1, 7, 1.0),
+                                     (2, 1, 8192, 0.5), (2, 1, 8193, 0.1), (1, 2, 20000, 0.9)])
 def test_sampler_matches_oracle(oracle, S, G, C, q):
     from sortnet_amd import ext
     dev = _dev()
