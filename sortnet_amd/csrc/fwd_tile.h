@@ -373,14 +373,134 @@ __global__ void __launch_bounds__(256, P::PIPE_WAVES) fwd_kernel_pipe(FwdArgs a)
     }
 }
 
+// -------------------------------------------------------------------------------------------
+// Pipelined variant for scalar loads with HW == 1: kept-channel index lists on either side (the weight
+// element of input n is w[co_idx[m]][ci_idx[n]]), reduction lengths that are not a multiple of 4, unaligned
+// rows.  Work-item t stages column t % 32 of the chunk for the rows t / 32 + 8 k, so a row of the input tile
+// is one 128-byte segment and the index of the column is looked up once.  As in fwd_kernel_pipe the loads of
+// chunk k+1 (index, then the gathered weights) are in flight while chunk k is consumed.
+// -------------------------------------------------------------------------------------------
+template <class P, int TB, int TM>
+__global__ void __launch_bounds__(256, P::PIPE_WAVES) fwd_kernel_lists(FwdArgs a) {
+    static_assert(P::NX == 1 && KT == 32, "one input tile, 32 columns per chunk");
+    constexpr int BB = 16 * TB, BM = 16 * TM;
+    constexpr int NXR = BB / 8, NWR = BM / 8;
+    __shared__ __attribute__((aligned(16))) float xs[BB][LDP];
+    __shared__ __attribute__((aligned(16))) float ws[BM][LDP];
+
+    const int tid = threadIdx.x, tm = tid & 15, tb = tid >> 4;
+    const int g = blockIdx.z % a.G, split = blockIdx.z / a.G;
+    const int r0 = blockIdx.y * BB, m0 = blockIdx.x * BM;
+    const int s = r0 / kSubBatch;
+
+    const int nchunks = (a.CIg + KT - 1) / KT;
+    const int n_begin = (int)((long long)split * nchunks / a.nsplit) * KT;
+    int n_end = (int)((long long)(split + 1) * nchunks / a.nsplit) * KT;
+    if (n_end > a.CIg) n_end = a.CIg;
+
+    const int col = tid & 31, lrow = tid >> 5;
+    int xoff[NXR], woff[NWR];
+    uint32_t okx = 0u, okw = 0u;
+    #pragma unroll
+    for (int k = 0; k < NXR; k++) {
+        const int r = r0 + lrow + 8 * k;
+        const bool ok = r < a.R;
+        okx |= ok ? 1u << k : 0u;
+        xoff[k] = ((ok ? r : r0) * a.G + g) * a.CIg;
+    }
+    #pragma unroll
+    for (int k = 0; k < NWR; k++) {
+        const int m = m0 + lrow + 8 * k;
+        const bool ok = m < a.COg;
+        okw |= ok ? 1u << k : 0u;
+        const int mm = ok ? m : m0;
+        const int wrow = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + mm] : mm;
+        woff[k] = (g * a.W_COg + wrow) * a.W_CIg;
+    }
+    const int* cidx = a.ci_idx ? a.ci_idx + (size_t)(s * a.G + g) * a.CIg : nullptr;
+
+    float px[NXR], pw[NWR];
+    auto gload = [&](int k0) {
+        int n = k0 + col;
+        if (n >= n_end) n = n_begin;                  // a legal column; zeroed in sstore()
+        const int wcol = cidx ? cidx[n] : n;
+        #pragma unroll
+        for (int k = 0; k < NXR; k++) px[k] = a.x0[xoff[k] + n];
+        #pragma unroll
+        for (int k = 0; k < NWR; k++) pw[k] = a.w[woff[k] + wcol];
+    };
+    auto sstore = [&](int k0) {
+        const bool in = k0 + col < n_end;
+        #pragma unroll
+        for (int k = 0; k < NXR; k++) xs[lrow + 8 * k][col] = (in && ((okx >> k) & 1u)) ? px[k] : 0.f;
+        #pragma unroll
+        for (int k = 0; k < NWR; k++) ws[lrow + 8 * k][col] = (in && ((okw >> k) & 1u)) ? pw[k] : 0.f;
+    };
+
+    typename P::Acc acc[TB][TM];
+    #pragma unroll
+    for (int i = 0; i < TB; i++) {
+        #pragma unroll
+        for (int j = 0; j < TM; j++) {
+            int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
+            size_t o = (size_t)(r * a.G + g) * a.COg + m;
+            P::init(acc[i][j], a, o, r < a.R && m < a.COg, split);
+        }
+    }
+
+    if (n_begin < n_end) gload(n_begin);
+    for (int k0 = n_begin; k0 < n_end; k0 += KT) {
+        sstore(k0);
+        __syncthreads();
+        if (k0 + KT < n_end) gload(k0 + KT);
+        #pragma unroll
+        for (int pass = 0; pass < P::PASSES; pass++) {
+            #pragma unroll P::UNROLL4
+            for (int n4 = 0; n4 < KT; n4 += 4) {
+                float4 wv[TM];
+                #pragma unroll
+                for (int j = 0; j < TM; j++) wv[j] = *reinterpret_cast<const float4*>(&ws[tm + 16 * j][n4]);
+                #pragma unroll
+                for (int i = 0; i < TB; i++) {
+                    float4 xl = *reinterpret_cast<const float4*>(&xs[tb + 16 * i][n4]);
+                    #pragma unroll
+                    for (int j = 0; j < TM; j++) P::step4(acc[i][j], a, xl, xl, wv[j], k0 + n4, pass);
+                }
+            }
+            #pragma unroll
+            for (int i = 0; i < TB; i++) {
+                #pragma unroll
+                for (int j = 0; j < TM; j++) P::chunk_end(acc[i][j], a, pass, k0);
+            }
+        }
+        __syncthreads();
+    }
+
+    #pragma unroll
+    for (int i = 0; i < TB; i++) {
+        #pragma unroll
+        for (int j = 0; j < TM; j++) {
+            int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
+            if (r < a.R && m < a.COg) P::store(acc[i][j], a, (size_t)(r * a.G + g) * a.COg + m, split);
+        }
+    }
+}
+
 // host-side launcher; the caller has validated shapes
 template <class P, int TB, int TM>
 int launch_fwd(const FwdArgs& a, hipStream_t stream) {
     dim3 grid((a.COg + 16 * TM - 1) / (16 * TM), (a.R + 16 * TB - 1) / (16 * TB), a.G * a.nsplit);
-    if (a.fast_x && a.fast_w && (a.mask_mode != SD_MASK_FACTORED || a.xmask))
+    if (a.fast_x && a.fast_w && (a.mask_mode != SD_MASK_FACTORED || a.xmask)) {
         hipLaunchKernelGGL((fwd_kernel_pipe<P, TB, TM>), grid, dim3(256), 0, stream, a);
-    else
-        hipLaunchKernelGGL((fwd_kernel<P, TB, TM>), grid, dim3(256), 0, stream, a);
+        return check_launch("fwd_kernel");
+    }
+    if constexpr (P::LISTS && TB == 2) {
+        if (a.HW == 1 && a.mask_mode != SD_MASK_FACTORED) {
+            hipLaunchKernelGGL((fwd_kernel_lists<P, TB, TM>), grid, dim3(256), 0, stream, a);
+            return check_launch("fwd_kernel");
+        }
+    }
+    hipLaunchKernelGGL((fwd_kernel<P, TB, TM>), grid, dim3(256), 0, stream, a);
     return check_launch("fwd_kernel");
 }
 
@@ -394,11 +514,13 @@ struct PolicyBase {
     static constexpr int PIPE_WAVES = 2;  // same for the pipelined kernel
     static constexpr int UNROLL4 = 2;     // unroll factor of the loop over groups of four inputs
     static constexpr int WIDE_TB = 4, WIDE_TM = 8;   // register tile of the large-batch launch of position kernels
+    static constexpr bool LISTS = false;  // also built as fwd_kernel_lists (ops that accept kept-channel index lists)
     template <class A> static __device__ __forceinline__ void chunk_end(A&, const FwdArgs&, int, int) {}
 };
 
 // l-inf forward without indices (core/cuda/inf_dist_cuda.cu:17-107)
 struct LinfNograd : PolicyBase {
+    static constexpr bool LISTS = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int MIN_WAVES = 3;
     static constexpr int UNROLL4 = 1;
@@ -437,6 +559,7 @@ __device__ __forceinline__ void store_chunk_winner(const FwdArgs& a, size_t o, f
 }
 
 struct LinfChunk : PolicyBase {
+    static constexpr bool LISTS = true;
     static constexpr int PIPE_WAVES = 2;   // three accumulator registers per output: no room for more waves
     static constexpr int MIN_WAVES = 2;
     static constexpr int UNROLL4 = 2;
@@ -745,6 +868,7 @@ __device__ __forceinline__ float pow_pos(float a, float p) {
 // p <= 10: y = max(sum |d|^p, FLT_MIN)^(1/p)   (core/cuda/norm_dist_cuda.cu:163-259, no max)
 template <int IP>
 struct LpPlain : PolicyBase {
+    static constexpr bool LISTS = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int MIN_WAVES = 3;
     struct Acc { float s; };
@@ -766,6 +890,7 @@ struct LpPlain : PolicyBase {
 // (core/cuda/norm_dist_cuda.cu:36-160): y = M (sum (|d|/M)^p + (1e-10/M)^p)^(1/p).
 template <int IP>
 struct LpOnline : PolicyBase {
+    static constexpr bool LISTS = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int MIN_WAVES = 3;
     static constexpr int PASSES = 2;
@@ -810,6 +935,7 @@ struct LpOnline : PolicyBase {
 // general-p forward, whose first step is the l-inf kernel
 template <int IP>
 struct LpWithMax : PolicyBase {
+    static constexpr bool LISTS = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int MIN_WAVES = 3;
     struct Acc { float s, rinv; };
