@@ -176,6 +176,17 @@ int sd_mean_shift_forward(const float* input, int B, int C, int HW, float* mean,
 int sd_channel_shift(const float* input, const float* shift, int B, int C, int HW, float sign,
                      float* output, sd_stream_t stream);
 
+/* Training-mode mean shift when every 32-sample sub-batch keeps its own channel subset
+ * (core/models/bound_basic_module.py:125-137,146-153, done there with torch ops).  input / output are
+ * (B, G * cnt, HW), already compacted; index is (S, G, cnt), S = ceil(B / 32), ascending channel numbers below
+ * Cg for every (sub-batch, group).  mean (G * Cg) receives, for every full channel, the mean over the samples
+ * and positions of the sub-batches that kept it (0 for a channel nobody kept); running_mean (G * Cg, may be
+ * NULL) is updated as above; output = input - mean[index].  Partial sums are added in sub-batch order, so
+ * the result is deterministic.  With running_mean = NULL it is also the backward of itself. */
+int sd_mean_shift_index_forward(const float* input, const int* index, int B, int G, int cnt, int Cg, int HW,
+                                float* mean, float* running_mean, float momentum, float* output,
+                                sd_stream_t stream);
+
 /* ---- device-side mask sampling for the index-list form (replaces sample_mask,
  * core/models/norm_dist.py:14-17, which draws on the host with a device synchronisation) ---- */
 

@@ -172,6 +172,17 @@ def mean_shift_forward(input, mean, running_mean, momentum, output):
          None if running_mean is None else _chk(running_mean, "running_mean"), momentum, _chk(output, "output"))
 
 
+def mean_shift_index_forward(input, index, channels_per_group, mean, running_mean, momentum, output):
+    """Not in the reference extension (done there with torch ops): training-mode mean shift of a
+    (B, G * cnt, HW) tensor that holds, per 32-sample sub-batch, the channels index[s, g, :] of
+    `channels_per_group` channels per group."""
+    B, HW = input.size(0), input.size(2)
+    G, cnt = index.size(-2), index.size(-1)
+    _run("sd_mean_shift_index_forward", input, _chk(input, "input"), _chk(index, "index", torch.int32), B, G, cnt,
+         channels_per_group, HW, _chk(mean, "mean"),
+         None if running_mean is None else _chk(running_mean, "running_mean"), momentum, _chk(output, "output"))
+
+
 def channel_shift(input, shift, sign, output):
     """output = input + sign * shift[c] (evaluation-mode mean shift, bias add)."""
     B, C, HW = input.size(0), input.size(1), input.size(2)

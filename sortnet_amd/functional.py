@@ -17,7 +17,7 @@ from . import ext as _C
 __all__ = [
     "NormDistF", "NormDistDropoutF", "SortNeuronF", "BoundInfDistF", "MaskedInfDistF",
     "norm_dist", "norm_dist_dropout", "sort_neuron", "bound_sort_neuron", "bound_inf_dist", "masked_inf_dist",
-    "MeanShiftF", "mean_shift",
+    "MeanShiftF", "mean_shift", "MeanShiftIndexF", "mean_shift_index",
 ]
 
 
@@ -257,6 +257,38 @@ class MeanShiftF(torch.autograd.Function):
         scratch = torch.empty(grad_y.size(1), device=grad_y.device, dtype=torch.float32)
         _C.mean_shift_forward(grad_y, scratch, None, 0.0, grad_x)
         return grad_x, None, None
+
+
+class MeanShiftIndexF(torch.autograd.Function):
+    """MeanShiftF when every 32-sample sub-batch keeps its own channels (`index`, shape (S, G, cnt)):
+    the mean of a channel runs over the sub-batches that kept it
+    (core/models/bound_basic_module.py:125-137,146-153).  The backward is the same centring of the gradient."""
+
+    @staticmethod
+    def forward(ctx, x, index, channels, running_mean, momentum):
+        x = x.contiguous()
+        y = torch.empty_like(x)
+        mean = torch.empty(channels, device=x.device, dtype=torch.float32)
+        _C.mean_shift_index_forward(x, index, channels // index.size(-2), mean, running_mean, momentum, y)
+        ctx.save_for_backward(index)
+        ctx.channels = channels
+        ctx.mark_non_differentiable(mean)
+        return y, mean
+
+    @staticmethod
+    def backward(ctx, grad_y, _grad_mean):
+        index, = ctx.saved_tensors
+        grad_y = grad_y.contiguous()
+        grad_x = torch.empty_like(grad_y)
+        scratch = torch.empty(ctx.channels, device=grad_y.device, dtype=torch.float32)
+        _C.mean_shift_index_forward(grad_y, index, ctx.channels // index.size(-2), scratch, None, 0.0, grad_x)
+        return grad_x, None, None, None, None
+
+
+def mean_shift_index(x, index, channels, running_mean=None, momentum=0.1):
+    """Training-mode mean shift of a compacted (B, G * cnt, HW) tensor; `channels` counts all channels of all
+    groups.  Returns (x - mean[index], mean) and updates `running_mean` in place when given."""
+    return MeanShiftIndexF.apply(x, index, channels, running_mean, momentum)
 
 
 def mean_shift(x, running_mean=None, momentum=0.1):

@@ -76,11 +76,16 @@ class MeanShiftDropout(nn.Module):
     def forward(self, x=None, lower=None, upper=None, index=None):
         if self.training:
             assert x is not None, "Currently not supported"
-            if index is None and self.bias is None:
+            if self.bias is None:
                 # fused kernels: mean, running-mean update and subtraction
-                x, _ = F.mean_shift(x.contiguous(), self.running_mean, self.momentum)
+                if index is None:
+                    x, _ = F.mean_shift(x.contiguous(), self.running_mean, self.momentum)
+                else:
+                    x, _ = F.mean_shift_index(x, index.to(torch.int32).contiguous(), self.out_channels,
+                                              self.running_mean, self.momentum)
                 mean = None
             else:
+                index = None if index is None else index.long()
                 mean = self._batch_mean(x, index)
                 with torch.no_grad():
                     self.running_mean.mul_(1 - self.momentum).add_(mean, alpha=self.momentum)
@@ -91,6 +96,7 @@ class MeanShiftDropout(nn.Module):
         if self.bias is not None:
             mean = mean - self.bias
         if index is not None:
+            index = index.long()
             rows = torch.div(torch.arange(x.size(0), device=x.device), SUB_BATCH, rounding_mode="trunc")
             per_row = mean.view(1, index.size(-2), -1).expand(x.size(0), -1, -1)
             mean_b = torch.gather(per_row, -1, index[rows]).reshape(x.size(0), -1).unsqueeze(-1)
@@ -160,7 +166,7 @@ class NormDistBase(nn.Module):
                 assert math.isinf(self.p)
                 lower, upper = F.bound_inf_dist(lower, upper, self.weight, self.groups, tag=self.tag)
         if self.mean_shift is not None:
-            x, lower, upper = self.mean_shift(x, lower, upper, index=None if index_out is None else index_out.long())
+            x, lower, upper = self.mean_shift(x, lower, upper, index=index_out)
         if bias is not None:
             x, lower, upper = apply_if_not_none((x, lower, upper), lambda z: z + bias.unsqueeze(-1))
         return x, lower, upper

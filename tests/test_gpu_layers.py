@@ -181,3 +181,49 @@ def test_model_zoo_modes(kind):
             s = net.scalar if not isinstance(net.scalar, (int, float)) else torch.tensor(float(net.scalar), device=dev)
             assert bool((m <= certified * scale * s + 1e-4).all())
         assert bool((certified.gather(1, targets.view(-1, 1)).abs() < 1e-6).all())
+
+
+@pytest.mark.parametrize("B,G,Cg,cnt,HW", [(70, 1, 96, 29, 1), (64, 2, 40, 17, 4), (5, 1, 12, 12, 1), (512, 1, 5120, 1530, 1)])
+def test_index_mean_shift_matches_float64_and_torch_ops(B, G, Cg, cnt, HW):
+    """Fused index-list mean shift: forward against a float64 restatement of
+    core/models/bound_basic_module.py:125-153, and forward + backward against the same computation written
+    with differentiable torch ops (the layer's path when it has a bias)."""
+    from sortnet_amd import functional as F
+    from sortnet_amd.layers import MeanShiftDropout
+    dev = _dev()
+    g = torch.Generator().manual_seed(B + cnt)
+    S = (B + 31) // 32
+    index = torch.stack([torch.stack([torch.randperm(Cg, generator=g)[:cnt].sort().values for _ in range(G)])
+                         for _ in range(S)]).to(torch.int32)
+    x = torch.randn(B, G * cnt, HW, generator=g)
+    running0 = torch.randn(G * Cg, generator=g)
+    # float64 restatement
+    xn, idx = x.double().numpy(), index.numpy()
+    tot, seen = np.zeros((G, Cg)), np.full((G, Cg), 1e-10)
+    for b in range(B):
+        for gi in range(G):
+            tot[gi, idx[b // 32, gi]] += xn[b, gi * cnt:(gi + 1) * cnt].sum(-1)
+            seen[gi, idx[b // 32, gi]] += 1
+    mean = tot / (seen * HW)
+    ref = xn.copy()
+    for b in range(B):
+        for gi in range(G):
+            ref[b, gi * cnt:(gi + 1) * cnt] -= mean[gi, idx[b // 32, gi]][:, None]
+    xd = x.to(dev).requires_grad_(True)
+    running = running0.to(dev).clone()
+    y, m = F.mean_shift_index(xd, index.to(dev), G * Cg, running, 0.1)
+    np.testing.assert_allclose(m.cpu().numpy(), mean.reshape(-1), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(y.detach().cpu().numpy(), ref, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(running.cpu().numpy(), 0.9 * running0.numpy() + 0.1 * mean.reshape(-1), rtol=1e-5, atol=1e-6)
+    # the torch-op formulation, forward and backward
+    layer = MeanShiftDropout(G * Cg, affine=True).to(dev).train()
+    x2 = x.to(dev).requires_grad_(True)
+    y2 = layer(x2, None, None, index=index.to(dev))[0]
+    torch.testing.assert_close(y.detach(), y2.detach(), rtol=1e-5, atol=1e-5)
+    gy = torch.randn(y.shape, generator=g).to(dev)
+    y.backward(gy)
+    y2.backward(gy)
+    torch.testing.assert_close(xd.grad, x2.grad, rtol=1e-5, atol=1e-5)
+    # deterministic: a second call gives the same bits
+    y3, _ = F.mean_shift_index(x.to(dev), index.to(dev), G * Cg, None, 0.1)
+    assert torch.equal(y3, y.detach())
