@@ -80,9 +80,16 @@ __global__ void __launch_bounds__(256) index_colsum_kernel(const float* __restri
     if (j >= cnt) return;
     const int b0 = s * kSubBatch, b1 = b0 + kSubBatch < B ? b0 + kSubBatch : B;
     float t = 0.f;
-    for (int b = b0; b < b1; b++) {
-        const float* src = x + ((size_t)(b * G + g) * cnt + j) * HW;
-        for (int hw = 0; hw < HW; hw++) t += src[hw];
+    if (HW == 1) {
+        const float* src = x + (size_t)g * cnt + j;
+        const size_t stride = (size_t)G * cnt;
+        #pragma unroll 8
+        for (int b = b0; b < b1; b++) t += src[b * stride];      // independent loads, added in sample order
+    } else {
+        for (int b = b0; b < b1; b++) {
+            const float* src = x + ((size_t)(b * G + g) * cnt + j) * HW;
+            for (int hw = 0; hw < HW; hw++) t += src[hw];
+        }
     }
     const size_t slot = (size_t)s * G * Cg + (size_t)g * Cg + index[(size_t)sg * cnt + j];
     part[slot] = t;

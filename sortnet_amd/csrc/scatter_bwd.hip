@@ -81,18 +81,18 @@ __global__ void __launch_bounds__(256) bound_bwd_kernel(BwdArgs a) {
 constexpr int kMaxRowLds = 12288;   // floats of LDS one row histogram may take
 
 template <bool SORT, bool HAS_W>
-__global__ void __launch_bounds__(256) scatter_bwd_rows_kernel(BwdArgs a) {
+__global__ void __launch_bounds__(1024) scatter_bwd_rows_kernel(BwdArgs a) {
     extern __shared__ float hist[];
     const int row = blockIdx.x;                 // ((b * G) + g) * HW + hw
     const int hw = row % a.HW;
     const int bg = row / a.HW;
     const int g = bg % a.G, b = bg / a.G;
     const int s = b / kSubBatch;
-    for (int n = threadIdx.x; n < a.CIg; n += 256) hist[n] = 0.f;
+    for (int n = threadIdx.x; n < a.CIg; n += blockDim.x) hist[n] = 0.f;
     __syncthreads();
     const size_t obase = ((size_t)(b * a.G + g) * a.COg) * a.HW + hw;
     const int K = SORT ? a.K : 1;
-    for (int m = threadIdx.x; m < a.COg; m += 256) {
+    for (int m = threadIdx.x; m < a.COg; m += blockDim.x) {
         size_t o = obase + (size_t)m * a.HW;
         float grad = a.g0[o];
         float coef = a.coef0;
@@ -115,7 +115,7 @@ __global__ void __launch_bounds__(256) scatter_bwd_rows_kernel(BwdArgs a) {
     }
     __syncthreads();
     const size_t xbase = ((size_t)(b * a.G + g) * a.CIg) * a.HW + hw;
-    for (int n = threadIdx.x; n < a.CIg; n += 256) a.gx0[xbase + (size_t)n * a.HW] = hist[n];
+    for (int n = threadIdx.x; n < a.CIg; n += blockDim.x) a.gx0[xbase + (size_t)n * a.HW] = hist[n];
 }
 
 template <bool HAS_W>
@@ -241,8 +241,10 @@ static int run_scatter(BwdArgs& a, hipStream_t st) {
     if (a.CIg <= kMaxRowLds) {
         dim3 rows((unsigned)(a.B * a.G * a.HW));
         size_t lds = (size_t)a.CIg * sizeof(float);
-        if (x.gw) hipLaunchKernelGGL((scatter_bwd_rows_kernel<SORT, true>), rows, dim3(256), lds, st, x);
-        else hipLaunchKernelGGL((scatter_bwd_rows_kernel<SORT, false>), rows, dim3(256), lds, st, x);
+        // few rows: more work-items per row, so that enough position / index loads are in flight
+        const dim3 block(rows.x < 4u * (unsigned)num_cus() ? 1024 : 256);
+        if (x.gw) hipLaunchKernelGGL((scatter_bwd_rows_kernel<SORT, true>), rows, block, lds, st, x);
+        else hipLaunchKernelGGL((scatter_bwd_rows_kernel<SORT, false>), rows, block, lds, st, x);
         return check_launch("scatter_bwd_rows_kernel");
     }
     if ((rc = fill_zero(a.gx0, (size_t)a.B * a.G * a.CIg * a.HW, st))) return rc;
