@@ -125,6 +125,12 @@ def main():
           lambda: ext.norm_dist_backward_input(gyc, xc, w, yc, gxc, 1, 8.0, ci, co), 4.5 / scale)
         t("  norm_dist_backward_input_weight p=8 (lists)",
           lambda: ext.norm_dist_backward_input_weight(gyc, xc, w, yc, gxc, gw, 1, 8.0, ci, co), 9 / scale)
+        t("  norm_dist_forward p=64 (lists)", lambda: ext.norm_dist_forward(xc, w, yc, 1, 64.0, ci, co), 5 / scale)
+        t("  norm_dist_backward_input_weight p=64 (lists)",
+          lambda: ext.norm_dist_backward_input_weight(gyc, xc, w, yc, gxc, gw, 1, 64.0, ci, co), 7 / scale)
+        meanc = torch.empty(M, device=dev)
+        t("  mean_shift_index_forward (lists)", lambda: ext.mean_shift_index_forward(yc, co, M, meanc, None, 0.1, gyc),
+          None, 4 * (3 * B * cm))
     if "shift" in on:
         t("mean_shift_forward", lambda: ext.mean_shift_forward(y, mean, None, 0.1, y2), None, 4 * (3 * B * M))
     if args.json:

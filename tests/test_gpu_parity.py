@@ -120,7 +120,8 @@ def test_inf_dist_ties_and_floor(oracle):
     assert pos.cpu().numpy().view(np.uint32)[0, 0, 0] == (1 | 0x80000000) and pos[0, 1, 0].item() == 0
 
 
-@pytest.mark.parametrize("B,CI,CO,G,ci_n,co_n", [(70, 96, 64, 1, 29, 21), (40, 64, 48, 2, 12, 8), (64, 128, 160, 1, 128, 37)])
+@pytest.mark.parametrize("B,CI,CO,G,ci_n,co_n", [(70, 96, 64, 1, 29, 21), (40, 64, 48, 2, 12, 8), (64, 128, 160, 1, 128, 37),
+                                                  (96, 1024, 300, 1, 701, 150)])
 def test_inf_dist_index_lists(oracle, B, CI, CO, G, ci_n, co_n):
     from sortnet_amd import ext
     dev = _dev()
@@ -355,18 +356,18 @@ def test_norm_dist(oracle, p, B, CI, CO, G, HW):
     np.testing.assert_allclose(y3.cpu().numpy(), ry, rtol=RTOL)
 
 
-@pytest.mark.parametrize("p", [8.0, 20.0])
-def test_norm_dist_index_lists(oracle, p):
+@pytest.mark.parametrize("p", [8.0, 20.0, 300.0])
+@pytest.mark.parametrize("B,CI,CO,G,ci_n,co_n", [(70, 96, 64, 1, 29, 21), (40, 64, 48, 2, 12, 8), (96, 1024, 300, 1, 701, 150)])
+def test_norm_dist_index_lists(oracle, p, B, CI, CO, G, ci_n, co_n):
     from sortnet_amd import ext
     dev = _dev()
-    B, CI, CO, G, ci_n, co_n = 70, 96, 64, 1, 29, 21
     ci, co = _index_lists(B, CI, CO, ci_n, co_n, G, 15)
-    w = _gen((CO, CI), 46, scale=0.3)
-    x, gy = _gen((B, ci_n, 1), 47), _gen((B, co_n, 1), 48)
+    w = _gen((CO, CI // G), 46, scale=0.3)
+    x, gy = _gen((B, ci_n * G, 1), 47), _gen((B, co_n * G, 1), 48)
     ry = oracle.norm_dist_forward(x.numpy(), w.numpy(), p, G, ci, co)
     xd, wd, gd = x.to(dev), w.to(dev), gy.to(dev)
     cid, cod = torch.from_numpy(ci).to(dev), torch.from_numpy(co).to(dev)
-    y = torch.empty(B, co_n, 1, device=dev)
+    y = torch.empty(B, co_n * G, 1, device=dev)
     ext.norm_dist_forward(xd, wd, y, G, p, cid, cod)
     np.testing.assert_allclose(y.cpu().numpy(), ry, rtol=RTOL)
     rgx, rgw = oracle.norm_dist_backward(gy.numpy(), x.numpy(), w.numpy(), ry, p, G, True, ci, co)
@@ -374,6 +375,14 @@ def test_norm_dist_index_lists(oracle, p):
     ext.norm_dist_backward_input_weight(gd, xd, wd, torch.from_numpy(ry).to(dev), gx, gw, G, p, cid, cod)
     _close(gx, rgx)
     _close(gw, rgw)
+    # only output channels dropped / only input channels dropped
+    xfull = _gen((B, CI, 1), 49)
+    y3 = torch.empty(B, co_n * G, 1, device=dev)
+    ext.norm_dist_forward(xfull.to(dev), wd, y3, G, p, None, cod)
+    np.testing.assert_allclose(y3.cpu().numpy(), oracle.norm_dist_forward(xfull.numpy(), w.numpy(), p, G, None, co), rtol=RTOL)
+    y4 = torch.empty(B, CO, 1, device=dev)
+    ext.norm_dist_forward(xd, wd, y4, G, p, cid, None)
+    np.testing.assert_allclose(y4.cpu().numpy(), oracle.norm_dist_forward(x.numpy(), w.numpy(), p, G, ci, None), rtol=RTOL)
 
 
 def test_config1_full_size(oracle):
