@@ -209,3 +209,51 @@ def test_wide_layers_256x12288x10240():
         assert torch.equal(du, y)
         x = (y - y.mean(dim=0, keepdim=True)).contiguous()
         del w, gw, tgw
+
+
+def test_index_lists_512x5120x5120():
+    """Index-list form at the benchmark size (keep probability 0.3 on both sides).  Every 32-sample sub-batch is
+    an ordinary dense problem on the gathered operands x[:, kept inputs] and W[kept outputs][:, kept inputs]:
+    the dense entry points (other kernels: vector loads, wide tiles) must give the same l-inf values and
+    positions bit for bit, the same l-p values to rel 1e-5, and the scatter backward must match index_put_."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, N, M = 512, 5120, 5120
+    S = B // 32
+    _, w, _ = _inputs(B, N, M, "rand")
+    wd = w.to(dev)
+    cn, cm = ext.mask_count(1, N, 0.3), ext.mask_count(2, M, 0.3)
+    ci = ext.sample_index_lists(1, S, 1, N, cn, dev)
+    co = ext.sample_index_lists(2, S, 1, M, cm, dev)
+    g = torch.Generator().manual_seed(3)
+    xc = torch.rand(B, cn, 1, generator=g).to(dev)
+    gy = torch.randn(B, cm, 1, generator=g).to(dev)
+    y = torch.empty(B, cm, 1, device=dev)
+    pos = torch.empty(B, cm, 1, device=dev, dtype=torch.int32)
+    ext.inf_dist_forward(xc, wd, y, pos, 1, ci, co)
+    yp = torch.empty_like(y)
+    ext.norm_dist_forward(xc, wd, yp, 1, 8.0, ci, co)
+    for s in (0, 7, S - 1):
+        rows = slice(32 * s, 32 * s + 32)
+        wsub = wd[co[s, 0].long()][:, ci[s, 0].long()].contiguous()        # (cm, cn)
+        xs = xc[rows].contiguous()
+        ys = torch.empty(32, cm, 1, device=dev)
+        ps = torch.empty(32, cm, 1, device=dev, dtype=torch.int32)
+        ext.inf_dist_forward(xs, wsub, ys, ps, 1)
+        assert torch.equal(ys, y[rows]) and torch.equal(ps, pos[rows])
+        ext.norm_dist_forward(xs, wsub, ys, 1, 8.0)
+        _close(yp[rows], ys)
+    assert float(y.min()) > 1e-10
+    # backward: grad_x[b, n'] += s g, grad_w[co[m'], ci[n']] -= s g through the compact positions
+    gx, gw = torch.empty_like(xc), torch.empty_like(wd)
+    ext.inf_dist_backward_input_weight(gy, pos, gx, gw, 1, ci, co)
+    npos = (pos & 0x7fffffff).long().squeeze(-1)                          # (B, cm) compact input index
+    sg = torch.where(pos.squeeze(-1) < 0, -gy.squeeze(-1), gy.squeeze(-1))
+    ref_gx = torch.zeros(B, cn, device=dev).index_put_((torch.arange(B, device=dev).unsqueeze(1).expand_as(npos), npos),
+                                                       sg, accumulate=True)
+    _close(gx.squeeze(-1), ref_gx)
+    sub = torch.arange(B, device=dev) // 32
+    wrow = co[sub, 0].long()                                              # (B, cm) full output channel
+    wcol = torch.gather(ci[sub, 0].long(), 1, npos)                       # (B, cm) full input channel
+    ref_gw = torch.zeros(M, N, device=dev).index_put_((wrow, wcol), -sg, accumulate=True)
+    _close(gw, ref_gw)
