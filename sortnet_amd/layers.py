@@ -44,17 +44,33 @@ class DropoutRegistry:
         self.next_tag = 0
         self.seed = seed
         self.draws = 0
+        self.overlap_sampler = True
+        self._side_streams = {}
 
     def new_tag(self):
         self.next_tag += 1
         return self.next_tag
 
     def sample(self, sub_batches, groups, channels, q, device):
-        """Ascending kept-channel lists (sub_batches, groups, count), count ~ Binomial(channels, q)."""
+        """Ascending kept-channel lists (sub_batches, groups, count), count ~ Binomial(channels, q).
+        The lists depend on nothing but the seed, and the sampler keeps only a few compute units busy, so it
+        is queued on a second stream (default priority) and overlaps the kernels already queued on the
+        caller's stream; the caller's stream waits for it before going on."""
         self.draws += 1
         seed = (self.seed * 1000003 + self.draws) & 0xFFFFFFFF
         count = ext.mask_count(seed, channels, q)
-        return ext.sample_index_lists(seed, sub_batches, groups, channels, count, device)
+        device = torch.device(device)
+        if device.type != "cuda" or not self.overlap_sampler:
+            return ext.sample_index_lists(seed, sub_batches, groups, channels, count, device)
+        main = torch.cuda.current_stream(device)
+        side = self._side_streams.get(device)
+        if side is None:
+            side = self._side_streams[device] = torch.cuda.Stream(device=device)
+        with torch.cuda.stream(side):
+            lists = ext.sample_index_lists(seed, sub_batches, groups, channels, count, device)
+        main.wait_stream(side)
+        lists.record_stream(main)
+        return lists
 
 
 DEFAULT_REGISTRY = DropoutRegistry()
