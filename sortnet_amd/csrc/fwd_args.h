@@ -43,11 +43,13 @@ inline int make_fwd_args(FwdArgs& a, const char* who, const float* x0, const flo
 // how many slices to cut the reduction range in.  A compute unit holds two to four of these
 // workgroups at a time and a workgroup runs about as long alone as with neighbours, so the last,
 // partly filled round of workgroups costs a full round: eight workgroups per compute unit keep that
-// tail below a fifth of the run.  A slice keeps at least four LDS chunks (128 inputs).
-inline int pick_nsplit(const FwdArgs& a, int BB, int BM) {
+// tail below a fifth of the run.  A slice keeps at least four LDS chunks (128 inputs).  The index-list
+// kernels are bound by their gather loads, not by the tail, and pay for every slice with merge traffic: they
+// ask for one workgroup per compute unit (per_cu).
+inline int pick_nsplit(const FwdArgs& a, int BB, int BM, int per_cu = 8) {
     long long tiles = (long long)((a.R + BB - 1) / BB) * ((a.COg + BM - 1) / BM) * a.G;
     int chunks = (a.CIg + 31) / 32;
-    long long want = 8ll * num_cus();
+    long long want = (long long)per_cu * num_cus();
     int max_ns = chunks / 4;
     if (max_ns > 16) max_ns = 16;
     int ns = 1;

@@ -29,7 +29,8 @@ static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st) {
     // with index lists a batch tile must stay inside one 32-sample sub-batch
     static const int kTb42[] = {4, 2};
     const int TB = index_lists ? 2 : pick_tb(a, kTb42, 2, 128);
-    a.nsplit = TB == 2 ? pick_nsplit(a, 32, 128) : pick_nsplit(a, 16 * P::WIDE_TB, 16 * P::WIDE_TM);
+    const bool gather = index_lists && !(a.fast_x && a.fast_w);      // served by the scalar-load kernel
+    a.nsplit = TB == 2 ? pick_nsplit(a, 32, 128, gather ? 1 : 8) : pick_nsplit(a, 16 * P::WIDE_TB, 16 * P::WIDE_TM);
     int rc;
     if (a.nsplit > 1) {
         // the merge buffer sits at the start of the workspace; a factored-mask call has already sized
