@@ -219,11 +219,12 @@ __global__ void __launch_bounds__(256, P::MIN_WAVES) fwd_kernel(FwdArgs a) {
 // (one 32-bit word per row and chunk).
 // -------------------------------------------------------------------------------------------
 // waves per SIMD the pipelined kernels are compiled for and the unroll factor of their inner loop: a policy may
-// name other values for register tiles of at most 16 outputs per work-item (PIPE_WAVES_16, UNROLL4_16; 0 = same)
+// name other values for register tiles of at most four channels per work-item (PIPE_WAVES_TM4, UNROLL4_TM4;
+// 0 = same)
 template <class P, int TB, int TM>
-constexpr int pipe_waves() { return (TB * TM <= 16 && P::PIPE_WAVES_16) ? P::PIPE_WAVES_16 : P::PIPE_WAVES; }
+constexpr int pipe_waves() { return (TM <= 4 && P::PIPE_WAVES_TM4) ? P::PIPE_WAVES_TM4 : P::PIPE_WAVES; }
 template <class P, int TB, int TM>
-constexpr int pipe_unroll() { return (TB * TM <= 16 && P::UNROLL4_16) ? P::UNROLL4_16 : P::UNROLL4; }
+constexpr int pipe_unroll() { return (TM <= 4 && P::UNROLL4_TM4) ? P::UNROLL4_TM4 : P::UNROLL4; }
 
 template <class P, int TB, int TM>
 __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_pipe(FwdArgs a) {
@@ -388,7 +389,7 @@ __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_pip
 // chunk k+1 (index, then the gathered weights) are in flight while chunk k is consumed.
 // -------------------------------------------------------------------------------------------
 template <class P, int TB, int TM>
-__global__ void __launch_bounds__(256, P::PIPE_WAVES) fwd_kernel_lists(FwdArgs a) {
+__global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_lists(FwdArgs a) {
     static_assert(P::NX == 1 && KT == 32, "one input tile, 32 columns per chunk");
     constexpr int BB = 16 * TB, BM = 16 * TM;
     constexpr int NXR = BB / 8, NWR = BM / 8;
@@ -462,7 +463,7 @@ __global__ void __launch_bounds__(256, P::PIPE_WAVES) fwd_kernel_lists(FwdArgs a
         if (k0 + KT < n_end) gload(k0 + KT);
         #pragma unroll
         for (int pass = 0; pass < P::PASSES; pass++) {
-            #pragma unroll P::UNROLL4
+            #pragma unroll (pipe_unroll<P, TB, TM>())
             for (int n4 = 0; n4 < KT; n4 += 4) {
                 float4 wv[TM];
                 #pragma unroll
@@ -520,7 +521,7 @@ struct PolicyBase {
     static constexpr int MIN_WAVES = 1;   // waves per SIMD the register budget must allow
     static constexpr int PIPE_WAVES = 2;  // same for the pipelined kernel
     static constexpr int UNROLL4 = 2;     // unroll factor of the loop over groups of four inputs
-    static constexpr int PIPE_WAVES_16 = 0, UNROLL4_16 = 0;   // overrides for tiles of <= 16 outputs (0: none)
+    static constexpr int PIPE_WAVES_TM4 = 0, UNROLL4_TM4 = 0;   // overrides for tiles of <= 4 channels (0: none)
     static constexpr int WIDE_TB = 4, WIDE_TM = 8;   // register tile of the large-batch launch of position kernels
     static constexpr bool LISTS = false;  // also built as fwd_kernel_lists (ops that accept kept-channel index lists)
     template <class A> static __device__ __forceinline__ void chunk_end(A&, const FwdArgs&, int, int) {}
@@ -571,10 +572,11 @@ struct LinfChunk : PolicyBase {
     static constexpr int PIPE_WAVES = 2;   // three accumulator registers per output: 2 x 8 outputs leave no room for more
     static constexpr int MIN_WAVES = 2;
     static constexpr int UNROLL4 = 2;
-    // large batches: 4 x 4 outputs in 114 registers, four waves per SIMD; measured 7 % faster than 4 x 8 outputs
-    // at two waves although it reads a third more LDS per term
+    // vector-load path: 4 x 4 (large batches) or 2 x 4 outputs per work-item in at most 128 registers, four
+    // waves per SIMD; measured 7 % faster than 4 x 8 / 2 x 8 outputs at two waves although it reads a third more
+    // LDS per term.  The gather kernel of the index lists keeps 2 x 8 at two waves (5 % faster there).
     static constexpr int WIDE_TB = 4, WIDE_TM = 4;
-    static constexpr int PIPE_WAVES_16 = 4, UNROLL4_16 = 1;
+    static constexpr int PIPE_WAVES_TM4 = 4, UNROLL4_TM4 = 1;
     struct Acc { float best, cm; int cid; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) { A.best = kEps; A.cm = 0.f; A.cid = -1; }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,

@@ -28,9 +28,9 @@ template <class P>
 static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st) {
     // with index lists a batch tile must stay inside one 32-sample sub-batch
     static const int kTb42[] = {4, 2};
-    const int TB = index_lists ? 2 : pick_tb(a, kTb42, 2, 128);
+    const int TB = index_lists ? 2 : pick_tb(a, kTb42, 2, 16 * P::WIDE_TM);
     const bool gather = index_lists && !(a.fast_x && a.fast_w);      // served by the scalar-load kernel
-    a.nsplit = TB == 2 ? pick_nsplit(a, 32, 128, gather ? 1 : 8) : pick_nsplit(a, 16 * P::WIDE_TB, 16 * P::WIDE_TM);
+    a.nsplit = TB == 2 ? pick_nsplit(a, 32, gather ? 128 : 16 * P::WIDE_TM, gather ? 1 : 8) : pick_nsplit(a, 16 * P::WIDE_TB, 16 * P::WIDE_TM);
     int rc;
     if (a.nsplit > 1) {
         // the merge buffer sits at the start of the workspace; a factored-mask call has already sized
@@ -40,7 +40,7 @@ static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st) {
         if (!a.packed0) return SD_ERR_HIP;
         if ((rc = fill_zero(a.packed0, n * 2, st))) return rc;
     }
-    if (TB == 2) rc = launch_fwd<P, 2, 8>(a, st);
+    if (TB == 2) rc = gather ? launch_fwd<P, 2, 8>(a, st) : launch_fwd<P, 2, P::WIDE_TM>(a, st);
     else rc = launch_fwd<P, P::WIDE_TB, P::WIDE_TM>(a, st);
     if (rc) return rc;
     return launch_resolve(a, st);
