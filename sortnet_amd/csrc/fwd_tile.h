@@ -382,10 +382,10 @@ __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_pip
 }
 
 // -------------------------------------------------------------------------------------------
-// Pipelined variant for scalar loads with HW == 1: kept-channel index lists on either side (the weight
-// element of input n is w[co_idx[m]][ci_idx[n]]), reduction lengths that are not a multiple of 4, unaligned
-// rows.  Work-item t stages column t % 32 of the chunk for the rows t / 32 + 8 k, so a row of the input tile
-// is one 128-byte segment and the index of the column is looked up once.  As in fwd_kernel_pipe the loads of
+// Pipelined variant for scalar loads: kept-channel index lists on either side (the weight element of input n
+// is w[co_idx[m]][ci_idx[n]]), reduction lengths that are not a multiple of 4, unaligned rows, spatial
+// positions (a row of the tile is one (sample, position) pair and its inputs lie HW floats apart).  Work-item t stages column t % 32 of the chunk for the rows t / 32 + 8 k, so a row of the input tile
+// is one 128-byte segment when HW == 1 and the index of the column is looked up once.  As in fwd_kernel_pipe the loads of
 // chunk k+1 (index, then the gathered weights) are in flight while chunk k is consumed.
 // -------------------------------------------------------------------------------------------
 template <class P, int TB, int TM>
@@ -399,7 +399,7 @@ __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_lis
     const int tid = threadIdx.x, tm = tid & 15, tb = tid >> 4;
     const int g = blockIdx.z % a.G, split = blockIdx.z / a.G;
     const int r0 = blockIdx.y * BB, m0 = blockIdx.x * BM;
-    const int s = r0 / kSubBatch;
+    const int s = (r0 / a.HW) / kSubBatch;
 
     const int nchunks = (a.CIg + KT - 1) / KT;
     const int n_begin = (int)((long long)split * nchunks / a.nsplit) * KT;
@@ -414,7 +414,8 @@ __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_lis
         const int r = r0 + lrow + 8 * k;
         const bool ok = r < a.R;
         okx |= ok ? 1u << k : 0u;
-        xoff[k] = ((ok ? r : r0) * a.G + g) * a.CIg;
+        const int rr = ok ? r : r0, b = rr / a.HW, hw = rr - b * a.HW;
+        xoff[k] = (b * a.G + g) * a.CIg * a.HW + hw;
     }
     #pragma unroll
     for (int k = 0; k < NWR; k++) {
@@ -433,7 +434,7 @@ __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_lis
         if (n >= n_end) n = n_begin;                  // a legal column; zeroed in sstore()
         const int wcol = cidx ? cidx[n] : n;
         #pragma unroll
-        for (int k = 0; k < NXR; k++) px[k] = a.x0[xoff[k] + n];
+        for (int k = 0; k < NXR; k++) px[k] = a.x0[xoff[k] + n * a.HW];
         #pragma unroll
         for (int k = 0; k < NWR; k++) pw[k] = a.w[woff[k] + wcol];
     };
@@ -451,7 +452,8 @@ __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_lis
         #pragma unroll
         for (int j = 0; j < TM; j++) {
             int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
-            size_t o = (size_t)(r * a.G + g) * a.COg + m;
+            int b = r / a.HW, hw = r - b * a.HW;
+            size_t o = ((size_t)(b * a.G + g) * a.COg + m) * a.HW + hw;
             P::init(acc[i][j], a, o, r < a.R && m < a.COg, split);
         }
     }
@@ -489,7 +491,10 @@ __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_lis
         #pragma unroll
         for (int j = 0; j < TM; j++) {
             int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
-            if (r < a.R && m < a.COg) P::store(acc[i][j], a, (size_t)(r * a.G + g) * a.COg + m, split);
+            if (r < a.R && m < a.COg) {
+                int b = r / a.HW, hw = r - b * a.HW;
+                P::store(acc[i][j], a, ((size_t)(b * a.G + g) * a.COg + m) * a.HW + hw, split);
+            }
         }
     }
 }
@@ -503,7 +508,7 @@ int launch_fwd(const FwdArgs& a, hipStream_t stream) {
         return check_launch("fwd_kernel");
     }
     if constexpr (P::LISTS && TB == 2) {
-        if (a.HW == 1 && a.mask_mode != SD_MASK_FACTORED) {
+        if (a.mask_mode != SD_MASK_FACTORED) {
             hipLaunchKernelGGL((fwd_kernel_lists<P, TB, TM>), grid, dim3(256), 0, stream, a);
             return check_launch("fwd_kernel");
         }
