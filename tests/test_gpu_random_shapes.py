@@ -28,6 +28,7 @@ def test_index_list_paths_on_random_shapes(oracle, seed):
     rng = np.random.default_rng(seed)
     for trial in range(25):
         G = int(rng.choice([1, 1, 2, 3]))
+        HW = int(rng.choice([1, 1, 2, 3]))
         B = int(rng.integers(1, 100)); CIg = int(rng.integers(1, 400)); COg = int(rng.integers(1, 150))
         cn = int(rng.integers(1, CIg + 1)); cm = int(rng.integers(1, COg + 1))
         S = (B + 31) // 32
@@ -35,15 +36,15 @@ def test_index_list_paths_on_random_shapes(oracle, seed):
         ci = np.stack([[np.sort(rng.choice(CIg, cn, replace=False)) for _ in range(G)] for _ in range(S)]).astype(np.int32) if use_ci else None
         co = np.stack([[np.sort(rng.choice(COg, cm, replace=False)) for _ in range(G)] for _ in range(S)]).astype(np.int32) if use_co else None
         nin, nout = (cn if use_ci else CIg), (cm if use_co else COg)
-        x = torch.from_numpy(rng.random((B, nin * G, 1), dtype=np.float32))
+        x = torch.from_numpy(rng.random((B, nin * G, HW), dtype=np.float32))
         w = torch.from_numpy((rng.standard_normal((COg * G, CIg)) * 0.3).astype(np.float32))
         if trial % 3 == 0:   # ties
             x, w = torch.round(x * 4) / 4, torch.round(w * 2) / 2
-        gy = torch.from_numpy(rng.standard_normal((B, nout * G, 1)).astype(np.float32))
+        gy = torch.from_numpy(rng.standard_normal((B, nout * G, HW)).astype(np.float32))
         ry, rpos = oracle.inf_dist_forward(x.numpy(), w.numpy(), G, True, ci, co)
         xd, wd, gd = x.to(dev), w.to(dev), gy.to(dev)
         cid = None if ci is None else torch.from_numpy(ci).to(dev); cod = None if co is None else torch.from_numpy(co).to(dev)
-        y = torch.empty(B, nout * G, 1, device=dev); pos = torch.empty(B, nout * G, 1, device=dev, dtype=torch.int32)
+        y = torch.empty(B, nout * G, HW, device=dev); pos = torch.empty(B, nout * G, HW, device=dev, dtype=torch.int32)
         ext.inf_dist_forward(xd, wd, y, pos, G, cid, cod)
         assert np.array_equal(y.cpu().numpy(), ry), "linf value"
         assert np.array_equal(pos.cpu().numpy(), rpos), "linf pos"
@@ -60,14 +61,14 @@ def test_index_list_paths_on_random_shapes(oracle, seed):
             close(gx, rgx, "lp gx"); close(gw, rgw, "lp gw")
         # index-list mean shift against float64
         if use_co:
-            yv = torch.from_numpy(rng.standard_normal((B, cm * G, 1)).astype(np.float32))
+            yv = torch.from_numpy(rng.standard_normal((B, cm * G, HW)).astype(np.float32))
             out, mean = F.mean_shift_index(yv.to(dev), cod, G * COg, None, 0.1)
             tot, seen = np.zeros((G, COg)), np.full((G, COg), 1e-10)
             yn = yv.double().numpy()
             for b in range(B):
                 for gi in range(G):
-                    tot[gi, co[b // 32, gi]] += yn[b, gi * cm:(gi + 1) * cm, 0]; seen[gi, co[b // 32, gi]] += 1
-            np.testing.assert_allclose(mean.cpu().numpy(), (tot / seen).reshape(-1), rtol=1e-5, atol=1e-6)
+                    tot[gi, co[b // 32, gi]] += yn[b, gi * cm:(gi + 1) * cm].sum(-1); seen[gi, co[b // 32, gi]] += 1
+            np.testing.assert_allclose(mean.cpu().numpy(), (tot / (seen * HW)).reshape(-1), rtol=1e-5, atol=1e-6)
 
 
 @pytest.mark.parametrize("seed", [3, 4])
