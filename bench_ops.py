@@ -23,6 +23,7 @@ def main():
     ap.add_argument("--shape", type=int, nargs=3, default=[512, 5120, 5120], metavar=("B", "N", "M"))
     ap.add_argument("--ops", default="linf,mask,bwd,bound,sort,lp,shift,idx")
     ap.add_argument("--reps", type=int, default=5)
+    ap.add_argument("--keep", type=float, default=0.3, help="keep probability of the index-list rows")
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
     import torch
@@ -101,7 +102,7 @@ def main():
             t("norm_dist_backward_input p=%g" % p, lambda: ext.norm_dist_backward_input(gy, xn, w, y, gx, 1, p), fb / 2)
     if "idx" in on:
         # index-list ("dropout") form: every 32-sample sub-batch keeps its own ~q share of the inputs and outputs
-        qk = 0.3
+        qk = args.keep
         S = (B + 31) // 32
         cn, cm = ext.mask_count(1, N, qk), ext.mask_count(2, M, qk)
         ci = ext.sample_index_lists(1, S, 1, N, cn, dev)

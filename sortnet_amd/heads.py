@@ -5,10 +5,9 @@ layer that returns worst-case margins against the target class.  Same constructo
 `(x, lower, upper)` protocol as the reference, so its checkpoints load.
 
 These layers are matrix products, so they run on the library GEMMs behind torch.  The one difference in
-formulation: the reference builds the (batch, classes, features) tensor `weight - weight[target]` for the
-margin radius; here samples are grouped by target class (one `(classes, features)` difference matrix and one
-GEMM per class present) or, with many classes, processed in bounded chunks, so memory stays O(classes x
-features) instead of O(batch x classes x features).
+formulation: the reference builds the whole (batch, classes, features) tensor `weight - weight[target]` for
+the margin radius; here it is built for a bounded number of samples at a time (all of them for ten classes,
+32 at a time for 1000 classes x 2048 features), so memory stays bounded for the many-class configurations.
 """
 import math
 
@@ -102,7 +101,7 @@ class BoundFinalLinear(_ScaledLinear):
     """core/models/bound_basic_module.py:79-103.  Without bounds or targets: the logits.  With both:
     `(logits, res)`, `res[b, j]` = upper bound over the box of `logit_j - logit_target(b)` (0 at j = target)."""
 
-    group_by_class_upto = 32     # classes up to which samples are grouped by target class
+    max_diff_elements = 1 << 26  # largest (samples, classes, features) difference tensor formed at once (256 MiB)
 
     def forward(self, x=None, lower=None, upper=None, targets=None):
         if x is not None:
@@ -117,18 +116,13 @@ class BoundFinalLinear(_ScaledLinear):
         return x, res
 
     def _margin_radius(self, radius, targets):
-        """sum_i |W[j, i] - W[target_b, i]| radius[b, i] for every sample b and class j."""
+        """sum_i |W[j, i] - W[target_b, i]| radius[b, i] for every sample b and class j, in chunks of samples
+        sized by `max_diff_elements`; no data-dependent shapes, hence no host synchronisation."""
         w = self.weight
-        out = radius.new_zeros(radius.size(0), w.size(0))
-        if w.size(0) <= self.group_by_class_upto:
-            for y in torch.unique(targets).tolist():
-                rows = (targets == y).nonzero(as_tuple=True)[0]
-                diff = (w - w[y]).abs()
-                out = out.index_add(0, rows, torch.mm(radius.index_select(0, rows), diff.t()))
-            return out
+        chunk = max(1, self.max_diff_elements // (w.size(0) * w.size(1)))
         pieces = []
-        for start in range(0, radius.size(0), 64):
-            t = targets[start:start + 64]
+        for start in range(0, radius.size(0), chunk):
+            t = targets[start:start + chunk]
             diff = (w.unsqueeze(0) - w.index_select(0, t).unsqueeze(1)).abs()      # (chunk, classes, features)
-            pieces.append(torch.bmm(diff, radius[start:start + 64].unsqueeze(-1)).squeeze(-1))
-        return torch.cat(pieces)
+            pieces.append(torch.bmm(diff, radius[start:start + chunk].unsqueeze(-1)).squeeze(-1))
+        return pieces[0] if len(pieces) == 1 else torch.cat(pieces)
