@@ -95,7 +95,7 @@ def main():
           lambda: ext.sort_neuron_backward_input_weight(gy, posK, gx, gw, 1, 0.3, 10), None,
           4 * (11 * B * M + B * N + M * N))
     if "lp" in on:
-        for p, ff, fb in ((8.0, 5, 9), (64.0, 3, 5)):
+        for p, ff, fb in ((8.0, 5, 9), (24.0, 3, 5), (64.0, 3, 5), (256.0, 3, 5)):
             t("norm_dist_forward p=%g" % p, lambda: ext.norm_dist_forward(xn, w, y, 1, p), ff)
             t("norm_dist_backward_input_weight p=%g" % p,
               lambda: ext.norm_dist_backward_input_weight(gy, xn, w, y, gx, gw, 1, p), fb)
@@ -126,9 +126,10 @@ def main():
           lambda: ext.norm_dist_backward_input(gyc, xc, w, yc, gxc, 1, 8.0, ci, co), 4.5 / scale)
         t("  norm_dist_backward_input_weight p=8 (lists)",
           lambda: ext.norm_dist_backward_input_weight(gyc, xc, w, yc, gxc, gw, 1, 8.0, ci, co), 9 / scale)
-        t("  norm_dist_forward p=64 (lists)", lambda: ext.norm_dist_forward(xc, w, yc, 1, 64.0, ci, co), 5 / scale)
-        t("  norm_dist_backward_input_weight p=64 (lists)",
-          lambda: ext.norm_dist_backward_input_weight(gyc, xc, w, yc, gxc, gw, 1, 64.0, ci, co), 7 / scale)
+        for p in (24.0, 256.0):
+            t("  norm_dist_forward p=%g (lists)" % p, lambda: ext.norm_dist_forward(xc, w, yc, 1, p, ci, co), 3 / scale)
+            t("  norm_dist_backward_input_weight p=%g (lists)" % p,
+              lambda: ext.norm_dist_backward_input_weight(gyc, xc, w, yc, gxc, gw, 1, p, ci, co), 5 / scale)
         meanc = torch.empty(M, device=dev)
         t("  mean_shift_index_forward (lists)", lambda: ext.mean_shift_index_forward(yc, co, M, meanc, None, 0.1, gyc),
           None, 4 * (3 * B * cm))

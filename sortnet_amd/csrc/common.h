@@ -54,6 +54,7 @@ struct FwdArgs {
     int nsplit;           // number of slices the reduction range is cut in (grid.z = G * nsplit)
     int fast_x, fast_w;   // 128-bit loads allowed for the x / w tiles
     float p, inv_p, q;
+    float skip_thr;       // l-p, large p: ratios to the running scale below this cannot change the fp32 result (0 = unused)
     uint32_t seed, t8, t16;
     int mask_mode;        // -1 none, SD_MASK_TERM, SD_MASK_FACTORED
 };

@@ -976,6 +976,35 @@ struct LpWithMax : PolicyBase {
     }
 };
 
+// Large p: a term whose ratio r to the scale is below skip_thr = (1e-6 / CI)^(1/p) contributes less than
+// 1e-6 / CI to a sum that is at least 1, so all such terms together move the result by less than 1e-6 / p
+// relative.  Nearly every term is of that kind once p reaches ~100, and the two transcendentals of r^p are
+// the whole cost of the kernel: they are evaluated only when some lane of the wavefront holds a significant
+// term (wave-uniform branches, first for the group of four inputs, then for each of them).
+__device__ __forceinline__ void lp_add_significant(float& s, float r0, float r1, float r2, float r3, float p, float thr) {
+    if (__builtin_amdgcn_ballot_w64(fmaxf(fmaxf(r0, r1), fmaxf(r2, r3)) > thr) == 0ull) return;
+    if (__builtin_amdgcn_ballot_w64(r0 > thr) != 0ull) s += pow_pos<-1>(r0, p);
+    if (__builtin_amdgcn_ballot_w64(r1 > thr) != 0ull) s += pow_pos<-1>(r1, p);
+    if (__builtin_amdgcn_ballot_w64(r2 > thr) != 0ull) s += pow_pos<-1>(r2, p);
+    if (__builtin_amdgcn_ballot_w64(r3 > thr) != 0ull) s += pow_pos<-1>(r3, p);
+}
+
+struct LpWithMaxSkip : LpWithMax<-1> {
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
+                                                 const float4& w, int, int) {
+        lp_add_significant(A.s, fabsf(x.x - w.x) * A.rinv, fabsf(x.y - w.y) * A.rinv, fabsf(x.z - w.z) * A.rinv,
+                           fabsf(x.w - w.w) * A.rinv, a.p, a.skip_thr);
+    }
+};
+
+struct LpOnlineSkip : LpOnline<-1> {
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4& xu,
+                                                 const float4& w, int n, int pass) {
+        if (pass == 0) LpOnline<-1>::step4(A, a, x, xu, w, n, pass);
+        else lp_add_significant(A.s, fabsf(x.x - w.x) * A.rinv, fabsf(x.y - w.y) * A.rinv, fabsf(x.z - w.z) * A.rinv,
+                                fabsf(x.w - w.w) * A.rinv, a.p, a.skip_thr);
+    }
+};
 
 // -------------------------------------------------------------------------------------------
 // resolve_pos_kernel: a wavefront owns 64 consecutive outputs.  Each lane first reads the winning

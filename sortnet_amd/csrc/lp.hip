@@ -6,9 +6,20 @@ namespace sd {
 
 // integral 0 <= p <= 8 selects a multiply chain, anything else the transcendental path
 // (core/cuda/norm_dist.cpp:17-38)
+// smallest thresholds from which the significance tests paid at B = 512, M = N = 5120 (p of about 32 for the
+// vector-load forward and both backward kernels, about 52 for the two-pass forward of the index lists)
+constexpr float kLpSkipFrom = 0.5f, kLpSkipFromOnline = 0.66f;
+
 static inline int int_power(float p) {
     if (p == (float)(int)p && p >= 0.f && p <= 8.f) return (int)p;
     return -1;
+}
+
+// ratio below which a term of r^p is dropped (see lp_add_significant); 0 when it is below `from`, i.e. when too
+// many terms would pass for the wavefront-level tests to pay
+static inline float lp_skip_threshold(float drop, float p, float from) {
+    const float thr = powf(drop, 1.f / p);
+    return thr >= from ? thr : 0.f;
 }
 
 template <template <int> class Pol, int TB, int TM>
@@ -89,7 +100,8 @@ static int lp_forward_max_first(FwdArgs& a, bool small, hipStream_t st) {
     a.part_stride = total;
     a.part0 = a.nsplit > 1 ? base + total : nullptr;
     a.part1 = nullptr;
-    rc = small ? launch_fwd<LpWithMax<-1>, 2, 8>(a, st) : launch_fwd<LpWithMax<-1>, 4, 8>(a, st);
+    if (a.skip_thr > 0.f) rc = small ? launch_fwd<LpWithMaxSkip, 2, 8>(a, st) : launch_fwd<LpWithMaxSkip, 4, 8>(a, st);
+    else rc = small ? launch_fwd<LpWithMax<-1>, 2, 8>(a, st) : launch_fwd<LpWithMax<-1>, 4, 8>(a, st);
     if (rc) return rc;
     return lp_split_finish(a, st);
 }
@@ -113,6 +125,7 @@ struct LpBwdArgs {
     const int* ci_idx; const int* co_idx;
     int B, R, HW, G, COg, CIg, W_COg, W_CIg;
     float pm1;   // p - 1
+    float skip_thr;  // general p: |d| / y below this cannot change the sums (0 = every term is evaluated)
     int zsplit;  // slices of the output-channel range (grad_input then merges with atomic adds)
 };
 
@@ -137,7 +150,13 @@ __device__ __forceinline__ float signed_pow(float d, float ry, float pm1) {
     }
 }
 
-template <int IP, bool WGRAD>
+// general p from the signed ratio sr = d / y
+__device__ __forceinline__ float signed_pow_ratio(float sr, float pm1) {
+    float pw = __builtin_amdgcn_exp2f(pm1 * __builtin_amdgcn_logf(fabsf(sr)));
+    return sr >= 0.f ? pw : -pw;
+}
+
+template <int IP, bool WGRAD, bool SKIP = false>
 __global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
     __shared__ float2 gr[MC][RB];   // (g, 1/y) of output channel m0+k, row r0+i
 
@@ -200,7 +219,26 @@ __global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
         const int mcount = m_hi - m0 < MC ? m_hi - m0 : MC;
         for (int k = 0; k < mcount; k++) {
             float wsum = 0.f;
-            if (rows == RB) {
+            if (SKIP) {
+                // large p: the two transcendentals only where some lane of the wavefront has a term that counts,
+                // tested for eight batch rows together first (padded rows have x = 0 and g = 0: whatever they
+                // add is multiplied by zero)
+                #pragma unroll
+                for (int i0 = 0; i0 < RB; i0 += 8) {
+                    float sr[8], big = 0.f;
+                    #pragma unroll
+                    for (int e = 0; e < 8; e++) { sr[e] = (xr[i0 + e] - wv[k]) * gr[k][i0 + e].y; big = fmaxf(big, fabsf(sr[e])); }
+                    if (__builtin_amdgcn_ballot_w64(big > a.skip_thr) == 0ull) continue;
+                    #pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        if (__builtin_amdgcn_ballot_w64(fabsf(sr[e]) > a.skip_thr) != 0ull) {
+                            float u = gr[k][i0 + e].x * signed_pow_ratio(sr[e], a.pm1);
+                            acc[i0 + e] += u;
+                            wsum += u;
+                        }
+                    }
+                }
+            } else if (rows == RB) {
                 #pragma unroll
                 for (int i = 0; i < RB; i++) {
                     float2 t = gr[k][i];
@@ -404,10 +442,10 @@ __global__ void __launch_bounds__(256) lp_recip_kernel(const float* __restrict__
     if (i < n) ry[i] = 1.f / y[i];
 }
 
-template <int IP>
+template <int IP, bool SKIP>
 __global__ void __launch_bounds__(256, 3) lp_bwd_fused_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                               const float* __restrict__ g, const float* __restrict__ ry,
-                                                              int B, int M, int N, int mr, float pm1,
+                                                              int B, int M, int N, int mr, float pm1, float skip_thr,
                                                               float* __restrict__ gx, float* __restrict__ gw) {
     constexpr int TI = 4, TJ = 2;                 // batch rows / weight rows per work-item
     constexpr int PSTRIDE = FN * 16 * TJ + 16;    // plane of one batch-row group, skewed by 16 banks
@@ -449,6 +487,8 @@ __global__ void __launch_bounds__(256, 3) lp_bwd_fused_kernel(const float* __res
                 #pragma unroll
                 for (int t = 0; t < FN; t++) gwp[j][t] = 0.f;
             }
+            // (g, 1/y) of the TI x TJ pairs first, so that the branches below do not serialise their loads
+            float gvs[TI][TJ], rvs[TI][TJ];
             #pragma unroll
             for (int i = 0; i < TI; i++) {
                 #pragma unroll
@@ -456,7 +496,33 @@ __global__ void __launch_bounds__(256, 3) lp_bwd_fused_kernel(const float* __res
                     const bool ok = bi[i] >= 0 && mj[j] >= 0;
                     // padded rows reuse the last valid row of x / w and its own 1/y, so the ratio stays <= 1
                     const size_t o = (size_t)(bi[i] >= 0 ? bi[i] : B - 1) * M + (mj[j] >= 0 ? mj[j] : m_hi - 1);
-                    const float gv = ok ? g[o] : 0.f, rv = ry[o];
+                    gvs[i][j] = ok ? g[o] : 0.f;
+                    rvs[i][j] = ry[o];
+                }
+            }
+            #pragma unroll
+            for (int i = 0; i < TI; i++) {
+                #pragma unroll
+                for (int j = 0; j < TJ; j++) {
+                    const float gv = gvs[i][j], rv = rvs[i][j];
+                    if (SKIP) {
+                        // large p: transcendentals only where some lane of the wavefront has a term that counts,
+                        // tested for the eight channels together first
+                        float sr[FN], big = 0.f;
+                        #pragma unroll
+                        for (int t = 0; t < FN; t++) { sr[t] = (xr[i][t] - wr[j][t]) * rv; big = fmaxf(big, fabsf(sr[t])); }
+                        if (__builtin_amdgcn_ballot_w64(big > skip_thr) != 0ull) {
+                            #pragma unroll
+                            for (int t = 0; t < FN; t++) {
+                                if (__builtin_amdgcn_ballot_w64(fabsf(sr[t]) > skip_thr) != 0ull) {
+                                    float pw = signed_pow_ratio(sr[t], pm1);
+                                    gxp[i][t] = fmaf(gv, pw, gxp[i][t]);
+                                    gwp[j][t] = fmaf(gv, pw, gwp[j][t]);
+                                }
+                            }
+                        }
+                        continue;
+                    }
                     #pragma unroll
                     for (int t = 0; t < FN; t++) {
                         float pw = signed_pow<IP>(xr[i][t] - wr[j][t], rv, pm1);
@@ -524,7 +590,10 @@ static int launch_lp_bwd_fused(int ip, const LpBwdArgs& a, hipStream_t st) {
     const int mr = (((M + ranges - 1) / ranges) + 31) / 32 * 32;   // equal ranges, whole weight tiles
     dim3 grid(N / FN, (M + mr - 1) / mr);
     (void)ip;
-    hipLaunchKernelGGL((lp_bwd_fused_kernel<-1>), grid, dim3(256), 0, st, a.x, a.w, a.gy, ry, B, M, N, mr, a.pm1, a.gx, a.gw);
+    if (a.skip_thr > 0.f)
+        hipLaunchKernelGGL((lp_bwd_fused_kernel<-1, true>), grid, dim3(256), 0, st, a.x, a.w, a.gy, ry, B, M, N, mr, a.pm1, a.skip_thr, a.gx, a.gw);
+    else
+        hipLaunchKernelGGL((lp_bwd_fused_kernel<-1, false>), grid, dim3(256), 0, st, a.x, a.w, a.gy, ry, B, M, N, mr, a.pm1, 0.f, a.gx, a.gw);
     return check_launch("lp_bwd_fused_kernel");
 }
 
@@ -577,7 +646,10 @@ static int launch_lp_bwd(int ip, const LpBwdArgs& a_in, hipStream_t st) {
 #define SD_CASE(k) case k: hipLaunchKernelGGL((lp_bwd_kernel<k, WGRAD>), grid, dim3(256), 0, st, a); break;
     switch (ip) {
         SD_CASE(0) SD_CASE(1) SD_CASE(2) SD_CASE(3) SD_CASE(4) SD_CASE(5) SD_CASE(6) SD_CASE(7) SD_CASE(8)
-        default: hipLaunchKernelGGL((lp_bwd_kernel<-1, WGRAD>), grid, dim3(256), 0, st, a); break;
+        default:
+            if (a.skip_thr > 0.f) hipLaunchKernelGGL((lp_bwd_kernel<-1, WGRAD, true>), grid, dim3(256), 0, st, a);
+            else hipLaunchKernelGGL((lp_bwd_kernel<-1, WGRAD>), grid, dim3(256), 0, st, a);
+            break;
     }
 #undef SD_CASE
     return check_launch("lp_bwd_kernel");
@@ -597,6 +669,8 @@ static int lp_backward(const char* who, const float* grad_output, const float* i
     a.ci_idx = ci_idx; a.co_idx = co_idx;
     a.B = B; a.R = f.R; a.HW = HW; a.G = G; a.COg = f.COg; a.CIg = f.CIg; a.W_COg = f.W_COg; a.W_CIg = f.W_CIg;
     a.pm1 = p - 1.f;
+    // a dropped term is below 1e-7 / (terms per sum) of a ratio that is at most 1
+    a.skip_thr = int_power(p - 1.f) < 0 ? lp_skip_threshold(1e-7f / (float)(f.COg > f.R ? f.COg : f.R), p - 1.f, kLpSkipFrom) : 0.f;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int ip = int_power(p - 1.f);
     const bool dense = G == 1 && HW == 1 && !ci_idx && !co_idx && f.CIg % TNB == 0 && aligned16(input) &&
@@ -631,13 +705,15 @@ extern "C" int sd_norm_dist_forward(const float* input, const float* weight,
     static const int kTb42[] = {4, 2};
     const bool small = w_index_ci || w_index_co || pick_tb(a, kTb42, 2, 128) == 2;
     const bool online = p > 10.f;   // core/cuda/norm_dist.cpp:4,51-55
+    a.skip_thr = lp_skip_threshold(1e-6f / (float)a.CIg, p, (a.fast_x && a.fast_w && !w_index_co) ? kLpSkipFrom : kLpSkipFromOnline);
     if (online && a.fast_x && a.fast_w && !w_index_co) return lp_forward_max_first(a, small, st);
     if ((rc = lp_split_setup(a, small ? 32 : 64, 128, online))) return rc;
     if (!online) {
         int ip = int_power(p);
         rc = small ? launch_lp<LpPlain, 2, 8>(ip, a, st) : launch_lp<LpPlain, 4, 8>(ip, a, st);
     } else {
-        rc = small ? launch_fwd<LpOnline<-1>, 2, 8>(a, st) : launch_fwd<LpOnline<-1>, 4, 8>(a, st);
+        if (a.skip_thr > 0.f) rc = small ? launch_fwd<LpOnlineSkip, 2, 8>(a, st) : launch_fwd<LpOnlineSkip, 4, 8>(a, st);
+        else rc = small ? launch_fwd<LpOnline<-1>, 2, 8>(a, st) : launch_fwd<LpOnline<-1>, 4, 8>(a, st);
     }
     if (rc) return rc;
     return lp_split_finish(a, st);

@@ -385,6 +385,40 @@ def test_norm_dist_index_lists(oracle, p, B, CI, CO, G, ci_n, co_n):
     np.testing.assert_allclose(y4.cpu().numpy(), oracle.norm_dist_forward(x.numpy(), w.numpy(), p, G, ci, None), rtol=RTOL)
 
 
+@pytest.mark.parametrize("p", [40.0, 100.0, 400.0, 1000.0])
+@pytest.mark.parametrize("kind", ["grid", "continuous"])
+def test_norm_dist_large_p(oracle, p, kind):
+    """Large p, where the kernels evaluate r^p only for terms that can matter: rows with many terms at or near
+    the maximum (coarse grid: hundreds of exact ties at the top and at fixed ratios below it) and continuous data,
+    dense and with index lists, forward and backward against the double-precision oracle.  The values keep
+    rel 1e-5.  The gradients are (d / y)^(p-1): the ratio is rounded to fp32 once before the power, so any fp32
+    evaluation of all terms is off by about (p - 1) * 6e-8 relative (measured on these inputs: 2.8e-5 at p = 400,
+    5e-4 at p = 1000, bit for bit the same as the kernels); their tolerance is max(1e-5, 1e-6 p)."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, CI, CO = 70, 2048, 96
+    x, w, gy = _gen((B, CI, 1), 71), _gen((CO, CI), 72, scale=0.3), _gen((B, CO, 1), 73)
+    if kind == "grid":
+        x, w = torch.round(x * 2) / 2, torch.round(w * 2) / 2
+    ci, co = _index_lists(B, CI, CO, 1500, 70, 1, 74)
+    for lists in (False, True):
+        a, b = (ci, co) if lists else (None, None)
+        xs = x[:, :1500].contiguous() if lists else x
+        gs = gy[:, :70].contiguous() if lists else gy
+        ry = oracle.norm_dist_forward(xs.numpy(), w.numpy(), p, 1, a, b)
+        xd, wd, gd = xs.to(dev), w.to(dev), gs.to(dev)
+        ad = None if a is None else torch.from_numpy(a).to(dev)
+        bd = None if b is None else torch.from_numpy(b).to(dev)
+        y = torch.empty(B, ry.shape[1], 1, device=dev)
+        ext.norm_dist_forward(xd, wd, y, 1, p, ad, bd)
+        np.testing.assert_allclose(y.cpu().numpy(), ry, rtol=RTOL)
+        rgx, rgw = oracle.norm_dist_backward(gs.numpy(), xs.numpy(), w.numpy(), ry, p, 1, True, a, b)
+        gx, gw = torch.empty_like(xd), torch.empty_like(wd)
+        ext.norm_dist_backward_input_weight(gd, xd, wd, torch.from_numpy(ry).to(dev), gx, gw, 1, p, ad, bd)
+        _close(gx, rgx, rtol=max(RTOL, 1e-6 * p))
+        _close(gw, rgw, rtol=max(RTOL, 1e-6 * p))
+
+
 def test_config1_full_size(oracle):
     """Single l-inf layer at B=128, N=3072, M=1024: x ~ U[0,1], w ~ N(0, 1/N), grad ~ N(0,1), seed 0."""
     from sortnet_amd import ext
