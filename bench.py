@@ -43,6 +43,8 @@ def parse():
                     help="masked: the headline step (fused masked neuron).  index-lists: the reference's own training "
                          "form (kept-channel lists per 32-sample sub-batch, SortMLPModel) plus its certification pass "
                          "(sort neuron and interval sort neuron); a secondary figure, without roofline / cpu_baseline")
+    ap.add_argument("--p", type=float, default=float("inf"),
+                    help="index-lists workload: norm of the distance layers during training (the reference anneals it from 8 to 1000, then inf)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain device copy of a width x width fp32 matrix after the timed steps "
@@ -107,6 +109,13 @@ def index_list_workload(args):
     net = SortMLPModel(args.depth, args.width, (3, side, side), num_classes=args.classes, dropout=args.q,
                        registry=reg).to(dev)
     opt = torch.optim.AdamW(net.parameters(), lr=1e-4, fused=True)
+    from sortnet_amd.layers import NormDistBase
+    dist_layers = [m for m in net.modules() if isinstance(m, NormDistBase)]
+
+    def set_p(p):
+        for m in dist_layers:
+            m.p = p
+
     g = torch.Generator().manual_seed(0)
     x = torch.rand(args.batch, 3, side, side, generator=g).to(dev)
     t = torch.randint(0, args.classes, (args.batch,), generator=g).to(dev)
@@ -115,6 +124,7 @@ def index_list_workload(args):
 
     def train_step():
         net.train()
+        set_p(args.p)
         loss = torch.nn.functional.cross_entropy(net(x), t)
         opt.zero_grad(set_to_none=True)
         loss.backward()
@@ -122,6 +132,7 @@ def index_list_workload(args):
 
     def certify():
         net.eval()
+        set_p(float("inf"))
         with torch.no_grad():
             return net(x, targets=t, eps=args.eps, up=up, down=down)
 
@@ -142,8 +153,8 @@ def index_list_workload(args):
         "metric": "train samples/s, SortMLPModel in the reference's index-list form", "value": args.batch / step_s,
         "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": step_s * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "SortMLPModel depth %d width %d, B=%d, keep probability %.2f: forward + cross entropy + "
-                               "backward + AdamW through kept-channel index lists" % (args.depth, args.width, args.batch, args.q)},
+        "config": {"workload": "SortMLPModel depth %d width %d, B=%d, keep probability %.2f, p=%g: forward + cross entropy + "
+                               "backward + AdamW through kept-channel index lists" % (args.depth, args.width, args.batch, args.q, args.p)},
         "certification_ms": cert_s * 1e3,
     }))
 
