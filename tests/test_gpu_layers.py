@@ -227,3 +227,31 @@ def test_index_mean_shift_matches_float64_and_torch_ops(B, G, Cg, cnt, HW):
     # deterministic: a second call gives the same bits
     y3, _ = F.mean_shift_index(x.to(dev), index.to(dev), G * Cg, None, 0.1)
     assert torch.equal(y3, y.detach())
+
+
+def test_running_mean_refresh_protocol():
+    """The reference refreshes the running means after training (main.py:184-202): training mode, no_grad, p = inf,
+    momentum 1 / (batch index + 1), so that the running mean ends as the average of the batch means of the
+    evaluation-form (sort neuron) outputs."""
+    from sortnet_amd import functional as F
+    from sortnet_amd.layers import NormDist, BoundSequential, DropoutRegistry
+    dev = _dev()
+    reg = DropoutRegistry()
+    torch.manual_seed(4)
+    net = BoundSequential(NormDist(40, 64, bias=False, std=0.3, registry=reg),
+                          NormDist(64, 48, bias=False, std=0.3, dropout=0.7, registry=reg),
+                          NormDist(48, 10, bias=True, mean_shift=False, std=0.3, dropout=0.7, registry=reg)).to(dev)
+    net.train()
+    batches = [torch.rand(50, 40, device=dev) for _ in range(3)]
+    layers = list(net)
+    expect0 = []
+    with torch.no_grad():
+        for i, xb in enumerate(batches):
+            for m in net.modules():
+                if hasattr(m, "momentum"):
+                    m.momentum = 1 / (i + 1)
+            net((xb, None, None))
+            h0 = F.sort_neuron(xb.unsqueeze(-1), layers[0].weight, 1, q=None)
+            expect0.append(h0.mean(dim=(0, 2)))
+    torch.testing.assert_close(layers[0].mean_shift.running_mean, torch.stack(expect0).mean(0), rtol=1e-5, atol=1e-6)
+    assert torch.isfinite(layers[1].mean_shift.running_mean).all() and layers[1].mean_shift.running_mean.abs().sum() > 0
