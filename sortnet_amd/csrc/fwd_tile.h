@@ -748,7 +748,8 @@ struct SortNograd : PolicyBase {
     }
     static __device__ __forceinline__ void term(Acc& A, float x, float w) {
         float v = fabsf(x - w);
-        if (v > A.res[0]) topk_insert_values<K>(A.res, v);
+        // wave-uniform test: inserting a value that does not exceed the smallest kept one changes nothing
+        if (__builtin_amdgcn_ballot_w64(v > A.res[0]) != 0ull) topk_insert_values<K>(A.res, v);
     }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
                                                  const float4& w, int, int) {
@@ -851,8 +852,12 @@ struct BoundSort : PolicyBase {
     static __device__ __forceinline__ void term(Acc& A, float l, float u, float w) {
         float t1 = w - l, t2 = u - w;
         float nl = -fminf(t1, t2), hu = fmaxf(t1, t2);
-        if (nl > A.lo[0]) topk_insert_values<K>(A.lo, nl);
-        if (hu > A.hi[0]) topk_insert_values<K>(A.hi, hu);
+        // one wave-uniform test for both lists: inserting a value that does not exceed the smallest kept one
+        // leaves a list unchanged, so the insertions themselves need no lane mask
+        if (__builtin_amdgcn_ballot_w64(nl > A.lo[0] || hu > A.hi[0]) != 0ull) {
+            topk_insert_values<K>(A.lo, nl);
+            topk_insert_values<K>(A.hi, hu);
+        }
     }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& l, const float4& u,
                                                  const float4& w, int, int) {
