@@ -10,6 +10,8 @@ namespace sd {
 // smallest thresholds from which the significance tests paid at B = 512, M = N = 5120 (p of about 32 for the
 // vector-load forward and both backward kernels, about 52 for the two-pass forward of the index lists)
 constexpr float kLpSkipFrom = 0.5f, kLpSkipFromOnline = 0.66f;
+// backward: the dense both-gradient kernel (p of about 50) and the general kernel (p of about 140)
+constexpr float kLpSkipFromFused = 0.6f, kLpSkipFromGeneral = 0.84f;
 
 static inline int int_power(float p) {
     if (p == (float)(int)p && p >= 0.f && p <= 8.f) return (int)p;
@@ -116,12 +118,16 @@ static int lp_forward_max_first(FwdArgs& a, bool small, hipStream_t st) {
 //
 // A workgroup owns 256 consecutive input channels (one per work-item) and RB = 32 batch rows.
 // Each work-item keeps its 32 inputs and 32 grad_x partial sums in registers and walks all
-// output channels; per output channel it needs its own w[m,n] (coalesced global load) and the
-// 32 wave-uniform pairs (g, 1/y), which are staged in LDS in chunks of MC channels and read as
-// broadcasts.  The sum over the 32 rows of grad_w is formed in registers and added to memory
-// with one coalesced atomic per work-item and output channel.
+// output channels in chunks of MC; per output channel it needs its own w[m,n] and the 32 wave-uniform
+// pairs (g, 1/y), which are staged in LDS and read as broadcasts.  Everything a chunk needs is
+// requested one chunk ahead, so that no load latency sits between two chunks: the weight rows of the
+// next chunk (index lists: the row numbers of the chunk after it, one per lane, handed out with
+// v_readlane), its weights (MC independent loads into registers) and its (g, 1/y) pairs (into the other
+// half of the LDS buffer, one barrier per chunk).  The sum over the 32 rows of grad_w is formed in
+// registers and added to memory with one coalesced atomic per work-item and output channel.
 constexpr int RB = 32;   // batch rows per workgroup (= one index-list sub-batch)
-constexpr int MC = 16;   // output channels per LDS chunk
+constexpr int MC = 8;    // output channels per chunk (the chunk body is unrolled: weights sit in named registers)
+static_assert(MC * RB == 256, "one (g, 1/y) pair per work-item and chunk");
 
 struct LpBwdArgs {
     const float* gy; const float* x; const float* w; const float* y;
@@ -160,15 +166,77 @@ __device__ __forceinline__ float signed_pow_ratio(float sr, float pm1) {
     return sr >= 0.f ? pw : -pw;
 }
 
+// terms of output channel k of a chunk: FULL = all RB rows present
+template <int IP, bool WGRAD, bool SKIP, bool FULL>
+__device__ __forceinline__ void lp_bwd_channel(const LpBwdArgs& a, const float2 (&gr)[RB], const float (&xr)[RB],
+                                               float (&acc)[RB], float wk, int rows, int row, bool n_ok,
+                                               float* __restrict__ gwcol) {
+    float wsum = 0.f;
+    if (SKIP) {
+        // large p: the two transcendentals only where some lane of the wavefront has a term that counts,
+        // tested for eight batch rows together first (padded rows have x = 0, g = 0 and 1/y = 0)
+        #pragma unroll
+        for (int i0 = 0; i0 < RB; i0 += 8) {
+            float sr[8], big = 0.f;
+            #pragma unroll
+            for (int e = 0; e < 8; e++) { sr[e] = (xr[i0 + e] - wk) * gr[i0 + e].y; big = fmaxf(big, fabsf(sr[e])); }
+            if (__builtin_amdgcn_ballot_w64(big > a.skip_thr) == 0ull) continue;
+            #pragma unroll
+            for (int e = 0; e < 8; e++) {
+                if (__builtin_amdgcn_ballot_w64(fabsf(sr[e]) > a.skip_thr) != 0ull) {
+                    float u = gr[i0 + e].x * signed_pow_ratio(sr[e], a.pm1);
+                    acc[i0 + e] += u;
+                    wsum += u;
+                }
+            }
+        }
+    } else {
+        #pragma unroll
+        for (int i = 0; i < RB; i++) {
+            if (FULL || i < rows) {
+                float2 t = gr[i];
+                float pw = signed_pow<IP>(xr[i] - wk, t.y, a.pm1);
+                acc[i] = fmaf(t.x, pw, acc[i]);
+                wsum = fmaf(t.x, pw, wsum);
+            }
+        }
+    }
+    if (WGRAD && n_ok) unsafeAtomicAdd(gwcol + (size_t)row * a.W_CIg, -wsum);
+}
+
+// one chunk.  The multiply-chain and plain general-p forms unroll the channels (weights in named registers); the
+// significance-test form is branchy and large, so it loops and picks its weight with selects.
+template <int IP, bool WGRAD, bool SKIP, bool FULL>
+__device__ __forceinline__ void lp_bwd_chunk(const LpBwdArgs& a, const float2 (&gr)[MC][RB], const float (&xr)[RB],
+                                             float (&acc)[RB], const float (&wv)[MC], int rows, int mcount,
+                                             int rowv, bool n_ok, float* __restrict__ gwcol) {
+    if (SKIP) {
+        #pragma unroll 1
+        for (int k = 0; k < mcount; k++) {
+            float wk = wv[0];
+            #pragma unroll
+            for (int j = 1; j < MC; j++) wk = k == j ? wv[j] : wk;
+            lp_bwd_channel<IP, WGRAD, SKIP, FULL>(a, gr[k], xr, acc, wk, rows, __builtin_amdgcn_readlane(rowv, k), n_ok, gwcol);
+        }
+    } else {
+        #pragma unroll
+        for (int k = 0; k < MC; k++) {
+            if (k < mcount)
+                lp_bwd_channel<IP, WGRAD, SKIP, FULL>(a, gr[k], xr, acc, wv[k], rows, __builtin_amdgcn_readlane(rowv, k), n_ok, gwcol);
+        }
+    }
+}
+
 template <int IP, bool WGRAD, bool SKIP = false>
-__global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
-    __shared__ float2 gr[MC][RB];   // (g, 1/y) of output channel m0+k, row r0+i
+__global__ void __launch_bounds__(256, (SKIP ? 4 : 1)) lp_bwd_kernel(LpBwdArgs a) {
+    __shared__ float2 gr[2][MC][RB];   // (g, 1/y) of output channel m0+k, row r0+i; two chunks
 
     const int tid = threadIdx.x;
     const int g = blockIdx.z % a.G, slice = blockIdx.z / a.G;
-    // output channels of this slice, whole LDS chunks
+    // output channels of this slice, whole chunks
     const int per = ((a.COg + a.zsplit - 1) / a.zsplit + MC - 1) / MC * MC;
     const int m_lo = slice * per, m_hi = m_lo + per < a.COg ? m_lo + per : a.COg;
+    if (m_lo >= m_hi) return;   // whole workgroup; grad_input of a sliced launch is zero-filled beforehand
     const int r0 = blockIdx.y * RB;
     const int n = blockIdx.x * 256 + tid;
     const bool n_ok = n < a.CIg;
@@ -177,6 +245,31 @@ __global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
     if (rows > RB) rows = RB;
 
     const int wcol = n_ok ? (a.ci_idx ? a.ci_idx[(s * a.G + g) * a.CIg + n] : n) : 0;
+    const int* __restrict__ co = a.co_idx ? a.co_idx + (size_t)(s * a.G + g) * a.COg : nullptr;
+    const float* __restrict__ wcolp = a.w + (size_t)g * a.W_COg * a.W_CIg + wcol;
+    float* __restrict__ gwcol = WGRAD ? a.gw + (size_t)g * a.W_COg * a.W_CIg + wcol : nullptr;
+    // weight row of output channel m0 + (lane mod MC), clamped into the slice so that every load stays inside W
+    const int kl = tid & (MC - 1);
+    auto row_of = [&](int m0) {
+        int m = m0 + kl;
+        m = m < m_hi ? m : m_hi - 1;
+        return co ? co[m] : m;
+    };
+    // (g, 1/y) pair number tid of the chunk at m0: consecutive work-items take consecutive channels of one row
+    const int sk = tid % MC, si = tid / MC;
+    // returns (g, y); the reciprocal is taken when the pair is written to LDS, after the chunk's arithmetic, so
+    // that nothing waits for these loads early (padding: g = 0, y = inf, i.e. 1/y = 0)
+    auto pair_of = [&](int m0) {
+        float2 v = make_float2(0.f, __builtin_inff());
+        const int m = m0 + sk, r = r0 + si;
+        if (m < m_hi && si < rows) {
+            int b = r / a.HW, hw = r - b * a.HW;
+            size_t o = ((size_t)(b * a.G + g) * a.COg + m) * a.HW + hw;
+            v.x = a.gy[o];
+            v.y = a.y[o];
+        }
+        return v;
+    };
 
     float xr[RB], acc[RB];
     #pragma unroll
@@ -191,82 +284,35 @@ __global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
         acc[i] = 0.f;
     }
 
-    for (int m0 = m_lo; m0 < m_hi; m0 += MC) {
-        __syncthreads();
-        // stage (g, 1/y): MC * RB = 512 pairs, two per work-item; consecutive work-items take
-        // consecutive channels of one row when HW == 1
+    int rowv = row_of(m_lo), rown = row_of(m_lo + MC);
+    float wv[MC];
+    #pragma unroll
+    for (int k = 0; k < MC; k++) wv[k] = wcolp[(size_t)__builtin_amdgcn_readlane(rowv, k) * a.W_CIg];
+    {
+        const float2 p0 = pair_of(m_lo);
+        gr[0][sk][si] = make_float2(p0.x, 1.f / p0.y);
+    }
+    __syncthreads();
+
+    int buf = 0;
+    for (int m0 = m_lo; m0 < m_hi; m0 += MC, buf ^= 1) {
+        // requests for the next chunk (clamped rows: always inside W) and the row numbers of the one after it
+        float wn[MC];
         #pragma unroll
-        for (int e = tid; e < MC * RB; e += 256) {
-            int k = e % MC, i = e / MC;
-            int m = m0 + k, r = r0 + i;
-            float2 v = make_float2(0.f, 0.f);
-            if (m < m_hi && i < rows) {
-                int b = r / a.HW, hw = r - b * a.HW;
-                size_t o = ((size_t)(b * a.G + g) * a.COg + m) * a.HW + hw;
-                v.x = a.gy[o];
-                v.y = 1.f / a.y[o];
-            }
-            gr[k][i] = v;
-        }
-        float wv[MC];
-        #pragma unroll
-        for (int k = 0; k < MC; k++) {
-            int m = m0 + k;
-            float v = 0.f;
-            if (n_ok && m < m_hi) {
-                int wrow = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + m] : m;
-                v = a.w[(size_t)(g * a.W_COg + wrow) * a.W_CIg + wcol];
-            }
-            wv[k] = v;
-        }
-        __syncthreads();
+        for (int k = 0; k < MC; k++) wn[k] = wcolp[(size_t)__builtin_amdgcn_readlane(rown, k) * a.W_CIg];
+        const int rownn = row_of(m0 + 2 * MC);
+        const float2 pn = pair_of(m0 + MC);
+
         const int mcount = m_hi - m0 < MC ? m_hi - m0 : MC;
-        for (int k = 0; k < mcount; k++) {
-            float wsum = 0.f;
-            if (SKIP) {
-                // large p: the two transcendentals only where some lane of the wavefront has a term that counts,
-                // tested for eight batch rows together first (padded rows have x = 0 and g = 0: whatever they
-                // add is multiplied by zero)
-                #pragma unroll
-                for (int i0 = 0; i0 < RB; i0 += 8) {
-                    float sr[8], big = 0.f;
-                    #pragma unroll
-                    for (int e = 0; e < 8; e++) { sr[e] = (xr[i0 + e] - wv[k]) * gr[k][i0 + e].y; big = fmaxf(big, fabsf(sr[e])); }
-                    if (__builtin_amdgcn_ballot_w64(big > a.skip_thr) == 0ull) continue;
-                    #pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        if (__builtin_amdgcn_ballot_w64(fabsf(sr[e]) > a.skip_thr) != 0ull) {
-                            float u = gr[k][i0 + e].x * signed_pow_ratio(sr[e], a.pm1);
-                            acc[i0 + e] += u;
-                            wsum += u;
-                        }
-                    }
-                }
-            } else if (rows == RB) {
-                #pragma unroll
-                for (int i = 0; i < RB; i++) {
-                    float2 t = gr[k][i];
-                    float u = t.x * signed_pow<IP>(xr[i] - wv[k], t.y, a.pm1);
-                    acc[i] += u;
-                    wsum += u;
-                }
-            } else {
-                #pragma unroll
-                for (int i = 0; i < RB; i++) {
-                    if (i < rows) {
-                        float2 t = gr[k][i];
-                        float u = t.x * signed_pow<IP>(xr[i] - wv[k], t.y, a.pm1);
-                        acc[i] += u;
-                        wsum += u;
-                    }
-                }
-            }
-            if (WGRAD && n_ok) {
-                int m = m0 + k;
-                int wrow = a.co_idx ? a.co_idx[(s * a.G + g) * a.COg + m] : m;
-                unsafeAtomicAdd(a.gw + (size_t)(g * a.W_COg + wrow) * a.W_CIg + wcol, -wsum);
-            }
-        }
+        if (rows == RB) lp_bwd_chunk<IP, WGRAD, SKIP, true>(a, gr[buf], xr, acc, wv, rows, mcount, rowv, n_ok, gwcol);
+        else lp_bwd_chunk<IP, WGRAD, SKIP, false>(a, gr[buf], xr, acc, wv, rows, mcount, rowv, n_ok, gwcol);
+
+        gr[buf ^ 1][sk][si] = make_float2(pn.x, 1.f / pn.y);   // last read in the previous iteration, before its barrier
+        __syncthreads();
+        #pragma unroll
+        for (int k = 0; k < MC; k++) wv[k] = wn[k];
+        rowv = rown;
+        rown = rownn;
     }
     if (n_ok) {
         #pragma unroll
@@ -282,153 +328,7 @@ __global__ void __launch_bounds__(256) lp_bwd_kernel(LpBwdArgs a) {
     }
 }
 
-// ---- backward, dense single-group case (G == 1, HW == 1, no index lists, CI % 16 == 0) -------------
-// Two reduction-free kernels instead of the fused one: every work-item owns TN = 16 consecutive input
-// channels of ONE batch row (grad_input) or of ONE weight row (grad_weight) and walks the other
-// axis; the operand that is shared by the whole wavefront (the weight row, resp. the input row) comes in
-// through scalar loads, the per-item (g, 1/y) pair through coalesced vector loads of pre-transposed
-// copies.  No LDS, no atomics, fixed summation order (deterministic gradients).
-typedef float sfloat16 __attribute__((ext_vector_type(16)));
-constexpr int TNB = 16;
-
-__device__ __forceinline__ void sload16(sfloat16& dst, const float* base, int byte_off) {
-    asm volatile("s_load_dwordx16 %0, %1, %2" : "=s"(dst) : "s"(base), "s"(byte_off));
-}
-__device__ __forceinline__ void swait(sfloat16& v) {   // ties the wait to the value so its uses stay behind it
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(v) :: "memory");
-}
-
-// ry = 1/y in (B, M) layout and the (M, B) transposes of g and 1/y
-__global__ void __launch_bounds__(256) lp_prep_kernel(const float* __restrict__ g, const float* __restrict__ y,
-                                                      int B, int M, float* __restrict__ ry,
-                                                      float* __restrict__ gT, float* __restrict__ ryT) {
-    __shared__ float tg[32][33], tr[32][33];
-    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
-    const int m0 = blockIdx.x * 32, b0 = blockIdx.y * 32;
-    #pragma unroll
-    for (int k = 0; k < 32; k += 8) {
-        int b = b0 + ty + k, m = m0 + tx;
-        float gv = 0.f, rv = 0.f;
-        if (b < B && m < M) {
-            gv = g[(size_t)b * M + m];
-            rv = 1.f / y[(size_t)b * M + m];
-            if (ry) ry[(size_t)b * M + m] = rv;
-        }
-        tg[ty + k][tx] = gv; tr[ty + k][tx] = rv;
-    }
-    __syncthreads();
-    #pragma unroll
-    for (int k = 0; k < 32; k += 8) {
-        int m = m0 + ty + k, b = b0 + tx;
-        if (b < B && m < M) {
-            gT[(size_t)m * B + b] = tg[tx][ty + k];
-            ryT[(size_t)m * B + b] = tr[tx][ty + k];
-        }
-    }
-}
-
-template <int IP>
-__device__ __forceinline__ void lp_bwd_accumulate(float (&acc)[TNB], const float (&own)[TNB], const sfloat16& shared,
-                                                  bool own_is_x, float gv, float rv, float pm1) {
-    #pragma unroll
-    for (int t = 0; t < TNB; t++) {
-        float d = own_is_x ? own[t] - shared[t] : shared[t] - own[t];   // always x - w
-        acc[t] = fmaf(gv, signed_pow<IP>(d, rv, pm1), acc[t]);
-    }
-}
-
-// grad_x[b, n0..n0+15] = sum_m u(b, m, n): work-item = batch row, scalar operand = weight row m
-template <int IP>
-__global__ void __launch_bounds__(256) lp_bwd_x_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                       const float* __restrict__ gT, const float* __restrict__ ryT,
-                                                       int B, int M, int N, float pm1, float* __restrict__ gx) {
-    const int n0 = blockIdx.x * TNB;
-    const int b = blockIdx.y * 256 + threadIdx.x;
-    const bool ok = b < B;
-    const int bb = ok ? b : B - 1;
-    float xr[TNB], acc[TNB];
-    #pragma unroll
-    for (int q = 0; q < TNB / 4; q++) {
-        float4 v = *reinterpret_cast<const float4*>(x + (size_t)bb * N + n0 + 4 * q);
-        xr[4 * q] = v.x; xr[4 * q + 1] = v.y; xr[4 * q + 2] = v.z; xr[4 * q + 3] = v.w;
-    }
-    #pragma unroll
-    for (int t = 0; t < TNB; t++) acc[t] = 0.f;
-    const float* wp = w + n0;
-    const int stride = N * 4;
-    // gridDim.z slices of the channel range keep enough wavefronts in flight for small batches
-    const int per = (M + gridDim.z - 1) / gridDim.z;
-    const int m_lo = blockIdx.z * per, m_hi = m_lo + per < M ? m_lo + per : M;
-    sfloat16 wa, wb;
-    sload16(wa, wp, (m_lo < M ? m_lo : 0) * stride);
-    for (int m = m_lo; m < m_hi; m += 2) {
-        float g0 = gT[(size_t)m * B + bb], r0 = ryT[(size_t)m * B + bb];
-        const bool two = m + 1 < m_hi;
-        const int m1 = two ? m + 1 : m;
-        float g1 = gT[(size_t)m1 * B + bb], r1 = ryT[(size_t)m1 * B + bb];
-        swait(wa);
-        sload16(wb, wp, m1 * stride);
-        lp_bwd_accumulate<IP>(acc, xr, wa, true, g0, r0, pm1);
-        swait(wb);
-        sload16(wa, wp, (m + 2 < m_hi ? m + 2 : m) * stride);
-        if (two) lp_bwd_accumulate<IP>(acc, xr, wb, true, g1, r1, pm1);
-    }
-    swait(wa);
-    if (ok) {
-        if (gridDim.z == 1) {
-            #pragma unroll
-            for (int q = 0; q < TNB / 4; q++)
-                *reinterpret_cast<float4*>(gx + (size_t)b * N + n0 + 4 * q) =
-                    make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
-        } else {
-            #pragma unroll
-            for (int t = 0; t < TNB; t++) unsafeAtomicAdd(gx + (size_t)b * N + n0 + t, acc[t]);
-        }
-    }
-}
-
-// grad_w[m, n0..n0+15] = - sum_b u(b, m, n): work-item = weight row, scalar operand = input row b
-template <int IP>
-__global__ void __launch_bounds__(256) lp_bwd_w_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                       const float* __restrict__ g, const float* __restrict__ ry,
-                                                       int B, int M, int N, float pm1, float* __restrict__ gw) {
-    const int n0 = blockIdx.x * TNB;
-    const int m = blockIdx.y * 256 + threadIdx.x;
-    const bool ok = m < M;
-    const int mm = ok ? m : M - 1;
-    float wr[TNB], acc[TNB];
-    #pragma unroll
-    for (int q = 0; q < TNB / 4; q++) {
-        float4 v = *reinterpret_cast<const float4*>(w + (size_t)mm * N + n0 + 4 * q);
-        wr[4 * q] = v.x; wr[4 * q + 1] = v.y; wr[4 * q + 2] = v.z; wr[4 * q + 3] = v.w;
-    }
-    #pragma unroll
-    for (int t = 0; t < TNB; t++) acc[t] = 0.f;
-    const float* xp = x + n0;
-    const int stride = N * 4;
-    sfloat16 xa, xb;
-    sload16(xa, xp, 0);
-    for (int b = 0; b < B; b += 2) {
-        float g0 = g[(size_t)b * M + mm], r0 = ry[(size_t)b * M + mm];
-        const bool two = b + 1 < B;
-        const int b1 = two ? b + 1 : b;
-        float g1 = g[(size_t)b1 * M + mm], r1 = ry[(size_t)b1 * M + mm];
-        swait(xa);
-        sload16(xb, xp, b1 * stride);
-        lp_bwd_accumulate<IP>(acc, wr, xa, false, g0, r0, pm1);
-        swait(xb);
-        sload16(xa, xp, (b + 2 < B ? b + 2 : b) * stride);
-        if (two) lp_bwd_accumulate<IP>(acc, wr, xb, false, g1, r1, pm1);
-    }
-    swait(xa);
-    if (ok) {
-        #pragma unroll
-        for (int q = 0; q < TNB / 4; q++)
-            *reinterpret_cast<float4*>(gw + (size_t)m * N + n0 + 4 * q) =
-                make_float4(-acc[4 * q], -acc[4 * q + 1], -acc[4 * q + 2], -acc[4 * q + 3]);
-    }
-}
-
+// ---- backward, dense single-group case with grad_weight and large p ------------------------------
 // Fused dense backward for grad_input AND grad_weight: u(b, m, n) is formed once and feeds both sums.
 // A workgroup owns FN = 8 consecutive input channels and a range of at most FMR weight rows; its 256
 // work-items are 16 (row of W: m = tm + 16 j) x 16 (batch row: b = tb + 16 i) with a 4 x 2 x 8 block of terms
@@ -594,45 +494,8 @@ static int launch_lp_bwd_fused(int ip, const LpBwdArgs& a, hipStream_t st) {
     const int mr = (((M + ranges - 1) / ranges) + 31) / 32 * 32;   // equal ranges, whole weight tiles
     dim3 grid(N / FN, (M + mr - 1) / mr);
     (void)ip;
-    if (a.skip_thr > 0.f)
-        hipLaunchKernelGGL((lp_bwd_fused_kernel<-1, true>), grid, dim3(256), 0, st, a.x, a.w, a.gy, ry, B, M, N, mr, a.pm1, a.skip_thr, a.gx, a.gw);
-    else
-        hipLaunchKernelGGL((lp_bwd_fused_kernel<-1, false>), grid, dim3(256), 0, st, a.x, a.w, a.gy, ry, B, M, N, mr, a.pm1, 0.f, a.gx, a.gw);
+    hipLaunchKernelGGL((lp_bwd_fused_kernel<-1, true>), grid, dim3(256), 0, st, a.x, a.w, a.gy, ry, B, M, N, mr, a.pm1, a.skip_thr, a.gx, a.gw);
     return check_launch("lp_bwd_fused_kernel");
-}
-
-template <int IP>
-static void launch_lp_bwd_dense_ip(const LpBwdArgs& a, const float* ry, const float* gT, const float* ryT, hipStream_t st) {
-    const int B = a.R, M = a.COg, N = a.CIg;
-    hipLaunchKernelGGL((lp_bwd_x_kernel<IP>), dim3(N / TNB, (B + 255) / 256, a.zsplit), dim3(256), 0, st,
-                       a.x, a.w, gT, ryT, B, M, N, a.pm1, a.gx);
-    if (a.gw)
-        hipLaunchKernelGGL((lp_bwd_w_kernel<IP>), dim3(N / TNB, (M + 255) / 256), dim3(256), 0, st,
-                           a.x, a.w, a.gy, ry, B, M, N, a.pm1, a.gw);
-}
-
-static int launch_lp_bwd_dense(int ip, const LpBwdArgs& a_in, hipStream_t st) {
-    const size_t n = (size_t)a_in.R * a_in.COg;
-    float* ws = static_cast<float*>(workspace(3 * n * sizeof(float)));
-    if (!ws) return SD_ERR_HIP;
-    float *ry = ws, *gT = ws + n, *ryT = ws + 2 * n;
-    hipLaunchKernelGGL(lp_prep_kernel, dim3((a_in.COg + 31) / 32, (a_in.R + 31) / 32), dim3(256), 0, st,
-                       a_in.gy, a_in.y, a_in.R, a_in.COg, a_in.gw ? ry : nullptr, gT, ryT);
-    int rc = check_launch("lp_prep_kernel");
-    if (rc) return rc;
-    // aim at >= 8 wavefronts per SIMD for the grad_input kernel; its slices merge with atomic adds
-    LpBwdArgs a = a_in;
-    long long waves = (long long)(a.CIg / TNB) * ((a.R + 255) / 256) * 4;
-    a.zsplit = 1;
-    while (a.zsplit < 8 && waves * a.zsplit < 8ll * 4 * num_cus() && a.COg / (a.zsplit * 2) >= 64) a.zsplit *= 2;
-    if (a.zsplit > 1 && (rc = fill_zero(a.gx, (size_t)a.R * a.CIg, st))) return rc;
-#define SD_CASE(k) case k: launch_lp_bwd_dense_ip<k>(a, ry, gT, ryT, st); break;
-    switch (ip) {
-        SD_CASE(0) SD_CASE(1) SD_CASE(2) SD_CASE(3) SD_CASE(4) SD_CASE(5) SD_CASE(6) SD_CASE(7) SD_CASE(8)
-        default: launch_lp_bwd_dense_ip<-1>(a, ry, gT, ryT, st); break;
-    }
-#undef SD_CASE
-    return check_launch("lp_bwd_x/w_kernel");
 }
 
 template <bool WGRAD>
@@ -643,7 +506,7 @@ static int launch_lp_bwd(int ip, const LpBwdArgs& a_in, hipStream_t st) {
     LpBwdArgs a = a_in;
     const long long blocks = (long long)((a.CIg + 255) / 256) * ((a.R + RB - 1) / RB) * a.G;
     a.zsplit = 1;
-    while (a.zsplit < 16 && blocks * a.zsplit < 4ll * num_cus() && a.COg / (a.zsplit * 2) >= 4 * MC) a.zsplit *= 2;
+    while (a.zsplit < 16 && blocks * a.zsplit < 4ll * num_cus() && a.COg / (a.zsplit * 2) >= 64) a.zsplit *= 2;
     int rc;
     if (a.zsplit > 1 && (rc = fill_zero(a.gx, (size_t)a.R * a.G * a.CIg, st))) return rc;
     dim3 grid((a.CIg + 255) / 256, (a.R + RB - 1) / RB, a.G * a.zsplit);
@@ -677,12 +540,13 @@ static int lp_backward(const char* who, const float* grad_output, const float* i
     a.skip_thr = int_power(p - 1.f) < 0 ? lp_skip_threshold(1e-7f / (float)(f.COg > f.R ? f.COg : f.R), p - 1.f, kLpSkipFrom) : 0.f;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int ip = int_power(p - 1.f);
-    const bool dense = G == 1 && HW == 1 && !ci_idx && !co_idx && f.CIg % TNB == 0 && aligned16(input) &&
-                       aligned16(weight) && aligned16(grad_input) && (!grad_weight || aligned16(grad_weight));
-    // general p: the two transcendentals per term are worth sharing between both gradients; integral
-    // p - 1 <= 8 (multiply chains) is faster through the two reduction-free kernels
-    if (dense && grad_weight && ip < 0) return launch_lp_bwd_fused(ip, a, st);
-    if (dense) return launch_lp_bwd_dense(ip, a, st);
+    // large p with both gradients in the dense single-group case: the kernel that forms every term once for both
+    // sums and owns its grad_weight block tests significance more cheaply than the general kernel, whose
+    // test only pays from a higher threshold; everything else goes through the general kernel
+    const bool dense = G == 1 && HW == 1 && !ci_idx && !co_idx && f.CIg % FN == 0 && aligned16(input) &&
+                       aligned16(weight) && aligned16(grad_weight);
+    if (dense && grad_weight && a.skip_thr >= kLpSkipFromFused) return launch_lp_bwd_fused(ip, a, st);
+    if (a.skip_thr < kLpSkipFromGeneral) a.skip_thr = 0.f;
     if (grad_weight) {
         if ((rc = fill_zero(grad_weight, (size_t)G * f.W_COg * f.W_CIg, st))) return rc;
         return launch_lp_bwd<true>(ip, a, st);
