@@ -417,6 +417,9 @@ def test_norm_dist_large_p(oracle, p, kind):
         ext.norm_dist_backward_input_weight(gd, xd, wd, torch.from_numpy(ry).to(dev), gx, gw, 1, p, ad, bd)
         _close(gx, rgx, rtol=max(RTOL, 1e-6 * p))
         _close(gw, rgw, rtol=max(RTOL, 1e-6 * p))
+        gx.fill_(float("nan"))
+        ext.norm_dist_backward_input(gd, xd, wd, torch.from_numpy(ry).to(dev), gx, 1, p, ad, bd)
+        _close(gx, rgx, rtol=max(RTOL, 1e-6 * p))
 
 
 def test_config1_full_size(oracle):

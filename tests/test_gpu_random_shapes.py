@@ -59,6 +59,9 @@ def test_index_list_paths_on_random_shapes(oracle, seed):
             rgx, rgw = oracle.norm_dist_backward(gy.numpy(), x.numpy(), w.numpy(), ryp, p, G, True, ci, co)
             ext.norm_dist_backward_input_weight(gd, xd, wd, torch.from_numpy(ryp).to(dev), gx, gw, G, p, cid, cod)
             close(gx, rgx, "lp gx"); close(gw, rgw, "lp gw")
+            gx.fill_(float("nan"))
+            ext.norm_dist_backward_input(gd, xd, wd, torch.from_numpy(ryp).to(dev), gx, G, p, cid, cod)
+            close(gx, rgx, "lp gx (input only)")
         # index-list mean shift against float64
         if use_co:
             yv = torch.from_numpy(rng.standard_normal((B, cm * G, HW)).astype(np.float32))
