@@ -505,8 +505,15 @@ static int launch_lp_bwd(int ip, const LpBwdArgs& a_in, hipStream_t st) {
     // cut in slices that merge into grad_input with atomic adds
     LpBwdArgs a = a_in;
     const long long blocks = (long long)((a.CIg + 255) / 256) * ((a.R + RB - 1) / RB) * a.G;
+    // workgroups run in rounds of (resident workgroups per CU) x CUs: take the slice count whose last round
+    // is fullest, a smaller count unless a larger one gains 3 %, slices of at least 64 channels
+    const double slots = (double)((a.skip_thr > 0.f ? 4 : 3) * num_cus());
+    double best = 0.0;
     a.zsplit = 1;
-    while (a.zsplit < 16 && blocks * a.zsplit < 4ll * num_cus() && a.COg / (a.zsplit * 2) >= 64) a.zsplit *= 2;
+    for (int z = 1; z <= 16 && (z == 1 || a.COg / z >= 64); z++) {
+        const double rounds = (double)blocks * z / slots, eff = rounds / std::ceil(rounds);
+        if (eff > best * 1.03) { best = eff; a.zsplit = z; }
+    }
     int rc;
     if (a.zsplit > 1 && (rc = fill_zero(a.gx, (size_t)a.R * a.G * a.CIg, st))) return rc;
     dim3 grid((a.CIg + 255) / 256, (a.R + RB - 1) / RB, a.G * a.zsplit);
