@@ -22,11 +22,13 @@
  * caller-visible memory.  pos packs the arg-max input index in bits 0..30 and a branch/sign
  * flag in bit 31.
  *
- * Scratch memory: the library keeps one device buffer per GPU for partial results (split
- * reductions, mask bits, candidate lists, per-slice sums) and grows it on demand with
- * hipMalloc; growing waits for the device to go idle first.  Calls are asynchronous on
- * `stream`, but two calls that use the buffer must not overlap on different streams of one
- * GPU.  Outputs that are zero-filled or merged with 128-bit stores must be 16-byte aligned.
+ * Scratch memory: the library keeps one device buffer per (GPU, stream) for partial results
+ * (split reductions, mask bits, candidate lists, per-slice sums) and grows it on demand with
+ * hipMalloc; growing waits for that stream first.  Calls are asynchronous on `stream`; calls
+ * on different streams never share a buffer and may overlap, calls on one stream use it in
+ * queue order.  A call that would have to grow the buffer while its stream is being captured
+ * into a graph fails with SD_ERR_HIP: run it once on that stream before the capture.
+ * Outputs that are zero-filled or merged with 128-bit stores must be 16-byte aligned.
  */
 #ifndef SORTDIST_H
 #define SORTDIST_H

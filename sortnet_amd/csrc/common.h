@@ -71,9 +71,10 @@ int check_launch(const char* what);
 // number of compute units of the current device (cached)
 int num_cus();
 
-// grow-only per-device scratch buffer owned by the library (split-N merge of position kernels).
-// Calls that use it must be ordered on one stream per device.
-void* workspace(size_t bytes);
+// grow-only scratch buffer owned by the library, one per (device, stream): split-N merges, bit masks, partial
+// sums.  Work queued on different streams never shares one; calls on ONE stream use it in queue order.
+// Growing waits for that stream and re-allocates (bytes == 0 returns the current buffer).
+void* workspace(size_t bytes, hipStream_t stream);
 
 // zero-fill n floats on `stream` with a kernel (graph-capture friendly, no memset node)
 int fill_zero(void* ptr, size_t n_words, hipStream_t stream);

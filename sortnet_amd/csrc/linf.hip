@@ -36,7 +36,7 @@ static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st) {
         // the merge buffer sits at the start of the workspace; a factored-mask call has already sized
         // the workspace for it and placed its bit masks behind it
         size_t n = (size_t)a.R * a.G * a.COg;
-        a.packed0 = static_cast<unsigned long long*>(a.xmask ? workspace(0) : workspace(n * 8));
+        a.packed0 = static_cast<unsigned long long*>(a.xmask ? workspace(0, st) : workspace(n * 8, st));
         if (!a.packed0) return SD_ERR_HIP;
         if ((rc = fill_zero(a.packed0, n * 2, st))) return rc;
     }
@@ -104,7 +104,7 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
         const int nchunks = (a.CIg + KT - 1) / KT;
         const long long xrows = (long long)a.R * G, wrows = (long long)CO;
         packed_bytes = pos ? (((size_t)a.R * CO * 8 + 255) / 256) * 256 : 0;
-        char* base = static_cast<char*>(workspace(packed_bytes + (size_t)(xrows + wrows) * nchunks * 4));
+        char* base = static_cast<char*>(workspace(packed_bytes + (size_t)(xrows + wrows) * nchunks * 4, st));
         if (!base) return SD_ERR_HIP;
         uint32_t* xm = reinterpret_cast<uint32_t*>(base + packed_bytes);
         uint32_t* wm = xm + xrows * nchunks;
@@ -162,7 +162,7 @@ extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* input
     a.nsplit = pick_nsplit(a, 16 * TB, 64);
     if (a.nsplit > 1) {
         size_t n = (size_t)a.R * a.G * a.COg;
-        a.packed0 = static_cast<unsigned long long*>(workspace(n * 16));
+        a.packed0 = static_cast<unsigned long long*>(workspace(n * 16, st));
         if (!a.packed0) return SD_ERR_HIP;
         a.packed1 = a.packed0 + n;
         if ((rc = fill_zero(a.packed0, n * 4, st))) return rc;

@@ -69,11 +69,11 @@ __global__ void __launch_bounds__(256) lp_finalize_kernel(const float* __restric
 
 // cuts the reduction range when the output tiles alone cannot fill the device; partial sums go to the
 // library workspace and are merged by lp_finalize_kernel
-static int lp_split_setup(FwdArgs& a, int BB, int BM, bool online) {
+static int lp_split_setup(FwdArgs& a, int BB, int BM, bool online, hipStream_t st) {
     a.nsplit = pick_nsplit(a, BB, BM);
     if (a.nsplit > 1) {
         a.part_stride = (size_t)a.R * a.G * a.COg;
-        a.part0 = static_cast<float*>(workspace(a.part_stride * a.nsplit * (online ? 2 : 1) * sizeof(float)));
+        a.part0 = static_cast<float*>(workspace(a.part_stride * a.nsplit * (online ? 2 : 1) * sizeof(float), st));
         if (!a.part0) return SD_ERR_HIP;
         a.part1 = online ? a.part0 + a.part_stride * a.nsplit : nullptr;
     }
@@ -95,7 +95,7 @@ static int lp_forward_max_first(FwdArgs& a, bool small, hipStream_t st) {
     FwdArgs m = a;
     m.nsplit = pick_nsplit(m, small ? 32 : 64, 128);
     a.nsplit = m.nsplit;
-    float* base = static_cast<float*>(workspace(total * (size_t)(1 + (a.nsplit > 1 ? a.nsplit : 0)) * sizeof(float)));
+    float* base = static_cast<float*>(workspace(total * (size_t)(1 + (a.nsplit > 1 ? a.nsplit : 0)) * sizeof(float), st));
     if (!base) return SD_ERR_HIP;
     m.y0 = base;
     int rc;
@@ -484,7 +484,7 @@ __global__ void __launch_bounds__(256, 3) lp_bwd_fused_kernel(const float* __res
 static int launch_lp_bwd_fused(int ip, const LpBwdArgs& a, hipStream_t st) {
     const int B = a.R, M = a.COg, N = a.CIg;
     const size_t n = (size_t)B * M;
-    float* ry = static_cast<float*>(workspace(n * sizeof(float)));
+    float* ry = static_cast<float*>(workspace(n * sizeof(float), st));
     if (!ry) return SD_ERR_HIP;
     hipLaunchKernelGGL(lp_recip_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a.y, n, ry);
     int rc = check_launch("lp_recip_kernel");
@@ -582,7 +582,7 @@ extern "C" int sd_norm_dist_forward(const float* input, const float* weight,
     const bool online = p > 10.f;   // core/cuda/norm_dist.cpp:4,51-55
     a.skip_thr = lp_skip_threshold(1e-6f / (float)a.CIg, p, (a.fast_x && a.fast_w && !w_index_co) ? kLpSkipFrom : kLpSkipFromOnline);
     if (online && a.fast_x && a.fast_w && !w_index_co) return lp_forward_max_first(a, small, st);
-    if ((rc = lp_split_setup(a, small ? 32 : 64, 128, online))) return rc;
+    if ((rc = lp_split_setup(a, small ? 32 : 64, 128, online, st))) return rc;
     if (!online) {
         int ip = int_power(p);
         rc = small ? launch_lp<LpPlain, 2, 8>(ip, a, st) : launch_lp<LpPlain, 4, 8>(ip, a, st);

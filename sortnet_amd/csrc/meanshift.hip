@@ -172,7 +172,7 @@ extern "C" int sd_mean_shift_index_forward(const float* input, const int* index,
     SD_REQUIRE(input && index && mean && output, "mean_shift_index_forward: null pointer");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int S = (B + kSubBatch - 1) / kSubBatch, C = G * Cg;
-    float* part = static_cast<float*>(workspace((size_t)2 * S * C * sizeof(float)));
+    float* part = static_cast<float*>(workspace((size_t)2 * S * C * sizeof(float), st));
     if (!part) return SD_ERR_HIP;
     float* rows = part + (size_t)S * C;
     if ((rc = fill_zero(part, (size_t)2 * S * C, st))) return rc;

@@ -1,5 +1,7 @@
 // Library runtime: error reporting, device queries, fill kernel and the verification exports.
 #include <cmath>
+#include <mutex>
+#include <vector>
 #include "common.h"
 
 namespace sd {
@@ -34,20 +36,33 @@ int num_cus() {
     return cached[dev];
 }
 
-void* workspace(size_t bytes) {
-    static void* buf[64] = {nullptr};
-    static size_t cap[64] = {0};
+void* workspace(size_t bytes, hipStream_t stream) {
+    struct Slot { int dev; hipStream_t stream; void* buf; size_t cap; };
+    static std::mutex mu;
+    static std::vector<Slot> slots;
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { set_error("workspace: no current device"); return nullptr; }
-    if (cap[dev] < bytes) {
-        // the old buffer may still be in use by queued kernels: release it only after the device is idle
-        if (buf[dev]) { (void)hipDeviceSynchronize(); (void)hipFree(buf[dev]); buf[dev] = nullptr; cap[dev] = 0; }
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0) { set_error("workspace: no current device"); return nullptr; }
+    std::lock_guard<std::mutex> lock(mu);
+    Slot* slot = nullptr;
+    for (Slot& c : slots) if (c.dev == dev && c.stream == stream) { slot = &c; break; }
+    if (!slot) { slots.push_back(Slot{dev, stream, nullptr, 0}); slot = &slots.back(); }
+    if (slot->cap < bytes) {
+        // nothing may be allocated or waited for while the stream records a graph: the caller runs the same
+        // call once on this stream beforehand, which sizes the buffer
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cap) != hipSuccess) (void)hipGetLastError();
+        if (cap != hipStreamCaptureStatusNone) {
+            set_error("workspace: %zu bytes needed while the stream is capturing; run the call once on this stream before the capture", bytes);
+            return nullptr;
+        }
+        // kernels queued on this stream may still use the old buffer: release it only after they are done
+        if (slot->buf) { (void)hipStreamSynchronize(stream); (void)hipFree(slot->buf); slot->buf = nullptr; slot->cap = 0; }
         size_t want = bytes + bytes / 4;
         void* p = nullptr;
         if (hipMalloc(&p, want) != hipSuccess) { (void)hipGetLastError(); set_error("workspace: hipMalloc of %zu bytes failed", want); return nullptr; }
-        buf[dev] = p; cap[dev] = want;
+        slot->buf = p; slot->cap = want;
     }
-    return buf[dev];
+    return slot->buf;
 }
 
 __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t* __restrict__ p, size_t n) {

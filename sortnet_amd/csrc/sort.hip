@@ -113,7 +113,7 @@ template <int K, bool VALUES>
 static int run_two_level(FwdArgs& a, bool small, hipStream_t st) {
     constexpr int KP = K + kKeySlack;
     const size_t total = (size_t)a.R * a.G * a.COg;
-    int* keys = static_cast<int*>(workspace((size_t)KP * total * sizeof(int)));
+    int* keys = static_cast<int*>(workspace((size_t)KP * total * sizeof(int), st));
     if (!keys) return SD_ERR_HIP;
     FwdArgs t = a;
     t.p0 = keys;

@@ -1,8 +1,11 @@
-"""HIP graph capture of the library's entry points: a sequence of forward and backward calls is captured once
-(after an eager warm-up, so that the library workspace already has its size and nothing allocates under capture)
-and replayed several times on new input contents, with eager work between the replays; every replay must
-reproduce the eager results (bit for bit for the l-inf values and positions, to the gradient tolerance for the
-atomically accumulated sums).  The library zero-fills with a kernel, never a memset node."""
+"""HIP graph capture of the library's entry points, and calls that overlap on two streams.
+
+A sequence of forward and backward calls is captured once (after an eager warm-up on the capture stream, so
+that this stream's library workspace already has its size and nothing allocates under capture) and replayed
+several times on new input contents, with eager work between the replays; every replay must reproduce the eager
+results (bit for bit for the l-inf values and positions, to the gradient tolerance for the atomically
+accumulated sums).  The library zero-fills with a kernel, never a memset node.  The workspace is kept per
+(device, stream), so calls queued on two streams may overlap: the second test checks that."""
 import numpy as np
 import pytest
 import torch
@@ -64,12 +67,16 @@ def test_graph_replays_match_eager():
 
     new_inputs(1.0)
     eager = outputs()
-    run(eager)                      # warm-up: workspace growth and one-time queries happen here
+    captured = outputs()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(captured)               # warm-up on the capture stream: its workspace grows here, not under capture
+    torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
 
-    captured = outputs()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    with torch.cuda.graph(graph, stream=side):
         run(captured)
 
     exact = ("y", "pos", "yl", "yu", "yc", "posc")
@@ -84,3 +91,41 @@ def test_graph_replays_match_eager():
                 assert torch.equal(eager[name], captured[name]), "%s, replay %d" % (name, replay)
             else:
                 _close(captured[name], eager[name], "%s, replay %d" % (name, replay))
+
+
+def test_calls_on_two_streams_overlap_safely(oracle):
+    """Two streams run workspace-using calls of different sizes at the same time (split-reduction merges of the
+    position kernels, the two-level sort neuron, l-p partial sums); each result must equal the one the same call
+    gives alone."""
+    from sortnet_amd import ext
+    dev = _dev()
+    g = torch.Generator().manual_seed(9)
+
+    def make(B, CI, CO):
+        x = torch.rand(B, CI, 1, generator=g).to(dev); w = (torch.randn(CO, CI, generator=g) * 0.2).to(dev)
+        return x, w, dict(y=torch.empty(B, CO, 1, device=dev), pos=torch.empty(B, CO, 1, device=dev, dtype=torch.int32),
+                          ys=torch.empty(B, CO, 1, device=dev), yp=torch.empty(B, CO, 1, device=dev))
+
+    def run(x, w, o):
+        ext.inf_dist_forward(x, w, o["y"], o["pos"], 1)
+        ext.sort_neuron_forward_nograd(x, w, o["ys"], 1, 0.4, 5)
+        ext.norm_dist_forward(x, w, o["yp"], 1, 24.0)
+
+    xa, wa, oa = make(64, 4096, 96)       # few output tiles: split reductions, partial sums in the workspace
+    xb, wb, ob = make(40, 2048, 200)
+    _, _, ra = make(64, 4096, 96); _, _, rb = make(40, 2048, 200)
+    run(xa, wa, ra); run(xb, wb, rb)
+    torch.cuda.synchronize()
+    ry, rpos = oracle.inf_dist_forward(xa.cpu().numpy(), wa.cpu().numpy())
+    assert np.array_equal(ra["y"].cpu().numpy(), ry) and np.array_equal(ra["pos"].cpu().numpy(), rpos)
+
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    for _ in range(20):
+        with torch.cuda.stream(sa):
+            run(xa, wa, oa)
+        with torch.cuda.stream(sb):
+            run(xb, wb, ob)
+    torch.cuda.synchronize()
+    for got, want in ((oa, ra), (ob, rb)):
+        assert torch.equal(got["y"], want["y"]) and torch.equal(got["pos"], want["pos"])
+        _close(got["ys"], want["ys"], "sort neuron"); _close(got["yp"], want["yp"], "l-p")
