@@ -155,7 +155,7 @@ __device__ __forceinline__ float signed_pow(float d, float ry, float pm1) {
         case 8: t1 = sr * sr; return fabsf(sr) * sr * t1 * (t1 * t1);
         default: {
             float pw = __builtin_amdgcn_exp2f(pm1 * __builtin_amdgcn_logf(fabsf(sr)));
-            return d >= 0.f ? pw : -pw;
+            return __builtin_copysignf(pw, sr);   // 1/y > 0: the ratio carries the sign of d (one v_bfi)
         }
     }
 }
@@ -163,7 +163,7 @@ __device__ __forceinline__ float signed_pow(float d, float ry, float pm1) {
 // general p from the signed ratio sr = d / y
 __device__ __forceinline__ float signed_pow_ratio(float sr, float pm1) {
     float pw = __builtin_amdgcn_exp2f(pm1 * __builtin_amdgcn_logf(fabsf(sr)));
-    return sr >= 0.f ? pw : -pw;
+    return __builtin_copysignf(pw, sr);
 }
 
 // terms of output channel k of a chunk: FULL = all RB rows present
