@@ -912,16 +912,23 @@ struct LpPlain : PolicyBase {
 
 // p > 10: running maximum M with rescaling, two passes over every LDS chunk
 // (core/cuda/norm_dist_cuda.cu:36-160): y = M (sum (|d|/M)^p + (1e-10/M)^p)^(1/p).
-template <int IP>
+template <int IP, bool FOLD = (IP < 0)>
 struct LpOnline : PolicyBase {
     static constexpr bool LISTS = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int MIN_WAVES = 3;
     static constexpr int PASSES = 2;
+    // rinv = 1 / M; FOLD (general p) keeps c = p log2(1 / M) there instead, a term is exp2(p log2|d| + c) and the
+    // rescaling factor of a new maximum is exp2(c_new - c_old) (see LpWithMax)
     struct Acc { float s, M, rinv, cm; };
-    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t, bool, int split = 0) {
         // the virtual term of size 1e-10 (res starts at 1 relative to M = 1e-10) belongs to slice 0 only
-        A.s = split == 0 ? 1.f : 0.f; A.M = kEps; A.rinv = 1.f / kEps; A.cm = 0.f;
+        A.s = split == 0 ? 1.f : 0.f; A.M = kEps; A.cm = 0.f;
+        A.rinv = FOLD ? -a.p * __builtin_amdgcn_logf(kEps) : 1.f / kEps;
+    }
+    static __device__ __forceinline__ float term(const Acc& A, const FwdArgs& a, float d) {
+        if (FOLD) return __builtin_amdgcn_exp2f(fmaf(a.p, __builtin_amdgcn_logf(fabsf(d)), A.rinv));
+        return pow_pos<IP>(fabsf(d) * A.rinv, a.p);
     }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
                                                  const float4& w, int, int pass) {
@@ -931,18 +938,24 @@ struct LpOnline : PolicyBase {
             v = fmaxf(fmaxf(v, fabsf(x.z - w.z)), fabsf(x.w - w.w));
             A.cm = v;
         } else {
-            A.s += pow_pos<IP>(fabsf(x.x - w.x) * A.rinv, a.p);
-            A.s += pow_pos<IP>(fabsf(x.y - w.y) * A.rinv, a.p);
-            A.s += pow_pos<IP>(fabsf(x.z - w.z) * A.rinv, a.p);
-            A.s += pow_pos<IP>(fabsf(x.w - w.w) * A.rinv, a.p);
+            A.s += term(A, a, x.x - w.x);
+            A.s += term(A, a, x.y - w.y);
+            A.s += term(A, a, x.z - w.z);
+            A.s += term(A, a, x.w - w.w);
         }
     }
     static __device__ __forceinline__ void chunk_end(Acc& A, const FwdArgs& a, int pass, int) {
         if (pass == 0) {
             if (A.cm > A.M) {
-                A.s *= __builtin_amdgcn_exp2f(a.p * __builtin_amdgcn_logf(A.M / A.cm));
+                if (FOLD) {
+                    const float cn = -a.p * __builtin_amdgcn_logf(A.cm);
+                    A.s *= __builtin_amdgcn_exp2f(cn - A.rinv);
+                    A.rinv = cn;
+                } else {
+                    A.s *= __builtin_amdgcn_exp2f(a.p * __builtin_amdgcn_logf(A.M / A.cm));
+                    A.rinv = 1.f / A.cm;
+                }
                 A.M = A.cm;
-                A.rinv = 1.f / A.cm;
             }
             A.cm = 0.f;
         }
@@ -957,27 +970,35 @@ struct LpOnline : PolicyBase {
 
 // caller-supplied maximum (core/cuda/norm_dist_cuda.cu:163-259 with has_max); also the second step of the
 // general-p forward, whose first step is the l-inf kernel
-template <int IP>
+template <int IP, bool FOLD = (IP < 0)>
 struct LpWithMax : PolicyBase {
     static constexpr bool LISTS = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int MIN_WAVES = 3;
+    // rinv = 1 / maximum; FOLD (general p) keeps c = p log2(1 / maximum) instead, so that a term is
+    // exp2(p log2|d| + c): one fused multiply-add in place of the scaling and the product (the rounding of
+    // log2|d|, about 2.5e-7 absolute, reaches y divided by p times p, i.e. unchanged: far inside the 1e-5 bar)
     struct Acc { float s, rinv; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs& a, size_t o, bool valid, int split = 0) {
-        A.rinv = valid ? 1.f / a.aux[o] : 1.f;
+        const float rinv = valid ? 1.f / a.aux[o] : 1.f;
         // the virtual term of size 1e-10 belongs to slice 0 only
-        A.s = split == 0 ? __builtin_amdgcn_exp2f(a.p * __builtin_amdgcn_logf(kEps * A.rinv)) : 0.f;
+        A.s = split == 0 ? __builtin_amdgcn_exp2f(a.p * __builtin_amdgcn_logf(kEps * rinv)) : 0.f;
+        A.rinv = FOLD ? a.p * __builtin_amdgcn_logf(rinv) : rinv;
+    }
+    static __device__ __forceinline__ float term(const Acc& A, const FwdArgs& a, float d) {
+        if (FOLD) return __builtin_amdgcn_exp2f(fmaf(a.p, __builtin_amdgcn_logf(fabsf(d)), A.rinv));
+        return pow_pos<IP>(fabsf(d) * A.rinv, a.p);
     }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
                                                  const float4& w, int, int) {
-        A.s += pow_pos<IP>(fabsf(x.x - w.x) * A.rinv, a.p);
-        A.s += pow_pos<IP>(fabsf(x.y - w.y) * A.rinv, a.p);
-        A.s += pow_pos<IP>(fabsf(x.z - w.z) * A.rinv, a.p);
-        A.s += pow_pos<IP>(fabsf(x.w - w.w) * A.rinv, a.p);
+        A.s += term(A, a, x.x - w.x);
+        A.s += term(A, a, x.y - w.y);
+        A.s += term(A, a, x.z - w.z);
+        A.s += term(A, a, x.w - w.w);
     }
     static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
         if (a.nsplit > 1) a.part0[(size_t)split * a.part_stride + o] = A.s;   // merged by lp_finalize_kernel
-        else a.y0[o] = powf(A.s, a.inv_p) / A.rinv;
+        else a.y0[o] = powf(A.s, a.inv_p) * a.aux[o];
     }
 };
 
@@ -994,7 +1015,7 @@ __device__ __forceinline__ void lp_add_significant(float& s, float r0, float r1,
     if (__builtin_amdgcn_ballot_w64(r3 > thr) != 0ull) s += pow_pos<-1>(r3, p);
 }
 
-struct LpWithMaxSkip : LpWithMax<-1> {
+struct LpWithMaxSkip : LpWithMax<-1, false> {   // the significance test needs the ratio itself
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
                                                  const float4& w, int, int) {
         lp_add_significant(A.s, fabsf(x.x - w.x) * A.rinv, fabsf(x.y - w.y) * A.rinv, fabsf(x.z - w.z) * A.rinv,
@@ -1002,10 +1023,10 @@ struct LpWithMaxSkip : LpWithMax<-1> {
     }
 };
 
-struct LpOnlineSkip : LpOnline<-1> {
+struct LpOnlineSkip : LpOnline<-1, false> {
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4& xu,
                                                  const float4& w, int n, int pass) {
-        if (pass == 0) LpOnline<-1>::step4(A, a, x, xu, w, n, pass);
+        if (pass == 0) LpOnline<-1, false>::step4(A, a, x, xu, w, n, pass);
         else lp_add_significant(A.s, fabsf(x.x - w.x) * A.rinv, fabsf(x.y - w.y) * A.rinv, fabsf(x.z - w.z) * A.rinv,
                                 fabsf(x.w - w.w) * A.rinv, a.p, a.skip_thr);
     }
