@@ -889,6 +889,24 @@ __device__ __forceinline__ float pow_pos(float a, float p) {
     }
 }
 
+// s + a^ip for a >= 0: the last product of the chain and the sum are one fused multiply-add
+template <int IP>
+__device__ __forceinline__ float add_pow(float s, float a, float p) {
+    float t1;
+    switch (IP) {
+        case 0: return s + 1.f;
+        case 1: return s + a;
+        case 2: return fmaf(a, a, s);
+        case 3: return fmaf(a * a, a, s);
+        case 4: t1 = a * a; return fmaf(t1, t1, s);
+        case 5: t1 = a * a; return fmaf(t1 * t1, a, s);
+        case 6: t1 = a * a; return fmaf(t1 * t1, t1, s);
+        case 7: t1 = a * a; return fmaf(t1 * t1, t1 * a, s);
+        case 8: t1 = a * a; t1 = t1 * t1; return fmaf(t1, t1, s);
+        default: return s + __builtin_amdgcn_exp2f(p * __builtin_amdgcn_logf(a));
+    }
+}
+
 // p <= 10: y = max(sum |d|^p, FLT_MIN)^(1/p)   (core/cuda/norm_dist_cuda.cu:163-259, no max)
 template <int IP>
 struct LpPlain : PolicyBase {
@@ -899,10 +917,10 @@ struct LpPlain : PolicyBase {
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) { A.s = 0.f; }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
                                                  const float4& w, int, int) {
-        A.s += pow_pos<IP>(fabsf(x.x - w.x), a.p);
-        A.s += pow_pos<IP>(fabsf(x.y - w.y), a.p);
-        A.s += pow_pos<IP>(fabsf(x.z - w.z), a.p);
-        A.s += pow_pos<IP>(fabsf(x.w - w.w), a.p);
+        A.s = add_pow<IP>(A.s, fabsf(x.x - w.x), a.p);
+        A.s = add_pow<IP>(A.s, fabsf(x.y - w.y), a.p);
+        A.s = add_pow<IP>(A.s, fabsf(x.z - w.z), a.p);
+        A.s = add_pow<IP>(A.s, fabsf(x.w - w.w), a.p);
     }
     static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {
         if (a.nsplit > 1) a.part0[(size_t)split * a.part_stride + o] = A.s;   // summed by lp_finalize_kernel
