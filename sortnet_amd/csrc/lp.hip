@@ -8,10 +8,10 @@ namespace sd {
 // integral 0 <= p <= 8 selects a multiply chain, anything else the transcendental path
 // (core/cuda/norm_dist.cpp:17-38)
 // smallest thresholds from which the significance tests paid at B = 512, M = N = 5120 (p of about 32 for the
-// vector-load forward and both backward kernels, about 52 for the two-pass forward of the index lists)
-constexpr float kLpSkipFrom = 0.5f, kLpSkipFromOnline = 0.66f;
-// backward: the dense both-gradient kernel (p of about 50) and the general kernel (p of about 140)
-constexpr float kLpSkipFromFused = 0.6f, kLpSkipFromGeneral = 0.84f;
+// vector-load forward, about 77 for the two-pass forward of the index lists)
+constexpr float kLpSkipFrom = 0.5f, kLpSkipFromOnline = 0.75f;
+// backward: the dense both-gradient kernel (p of about 65) and the general kernel (p of about 80)
+constexpr float kLpSkipFromFused = 0.68f, kLpSkipFromGeneral = 0.73f;
 
 static inline int int_power(float p) {
     if (p == (float)(int)p && p >= 0.f && p <= 8.f) return (int)p;
