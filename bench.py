@@ -6,11 +6,16 @@ inputs (3072 features in [0,1], 10 classes): forward through the distance layers
 first layer, masked order-statistic neuron with q = 0.3 on the others) with mean shift, hinge
 loss on the 1-Lipschitz margin, backward through every layer (grad_input and grad_weight),
 AdamW update, and the interval-bound (certification) pass with eps = 8/255 through all layers.
-Prints one JSON line; see --help for the knobs.
+
+Prints one JSON line.  `value` belongs to the mask named in config.workload (--mask); the same line carries,
+under "secondary", short runs of the other formulations of the same step: the other mask granularity, the pure
+l-inf net (q = 1), the reference's own index-list training form at its published keep probability (p = inf and
+p = 8) with its certification pass, and the wide 64x64-image configuration.  See --help for the knobs.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -19,10 +24,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 FP32_VECTOR_PEAK_TFLOPS = 157.3     # MI355X published fp32 vector peak
-# HBM bytes of one 512x5120x5120 interval-bound launch from the FETCH_SIZE / WRITE_SIZE counter runs
-# (2.00 * 171079 KiB + 163840 KiB); only reported when the benchmark runs at that shape
-IBP_LAUNCH_TRAFFIC_BYTES = 518.0e6
 VALU_LANE_RATE = 78.64e12           # 256 CUs x 4 SIMD x 16 lanes x 2 issue ports x 2.4 GHz lane-instructions/s
+# HBM bytes of one 512x5120x5120 interval-bound launch come from the committed counter summary (two rocprofv3
+# --pmc runs, FETCH_SIZE and WRITE_SIZE, scaled by a plain copy of known size): the line "traffic_bytes_per_launch"
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_headline_hbm_traffic.txt")
 
 
 def parse():
@@ -38,14 +43,16 @@ def parse():
     ap.add_argument("--q", type=float, default=0.3)
     ap.add_argument("--eps", type=float, default=8.0 / 255)
     ap.add_argument("--mask", choices=["term", "factored"], default="factored",
-                    help="granularity of the Bernoulli keep mask of the masked neuron")
+                    help="granularity of the Bernoulli keep mask of the masked neuron that `value` is measured with: "
+                         "term = an independent draw per (b, m, n) term; factored = keep_x(b, n) & keep_w(m, n)")
     ap.add_argument("--workload", choices=["masked", "index-lists"], default="masked",
-                    help="masked: the headline step (fused masked neuron).  index-lists: the reference's own training "
-                         "form (kept-channel lists per 32-sample sub-batch, SortMLPModel) plus its certification pass "
-                         "(sort neuron and interval sort neuron); a secondary figure, without roofline / cpu_baseline")
+                    help="masked: the headline step (fused masked neuron).  index-lists: only the reference's own "
+                         "training form (kept-channel lists per 32-sample sub-batch, SortMLPModel) and its certification "
+                         "pass (sort neuron and interval sort neuron), without roofline / cpu_baseline")
     ap.add_argument("--p", type=float, default=float("inf"),
                     help="index-lists workload: norm of the distance layers during training (the reference anneals it from 8 to 1000, then inf)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true", help="skip the short runs of the other formulations")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain device copy of a width x width fp32 matrix after the timed steps "
                          "(a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE counters with)")
@@ -94,27 +101,26 @@ def cpu_baseline(args, model_dims):
                       "bounds of all %d layers; no optimizer), %.1f s" % (nb, len(ws), t)}
 
 
-def index_list_workload(args):
-    """Training step of SortMLPModel in the reference's index-list form and the certification pass of the same
-    model in evaluation mode (sort neuron for the value, interval sort neuron for the bounds)."""
+def run_index_lists(args, q, p, steps, warmup, certify_runs=0):
+    """Training step of SortMLPModel in the reference's index-list form and, when asked for, the certification pass
+    of the same model in evaluation mode (sort neuron for the value, interval sort neuron for the bounds)."""
     import torch
     from sortnet_amd.ell_inf_models import SortMLPModel
-    from sortnet_amd.layers import DropoutRegistry, set_mask_seed
+    from sortnet_amd.layers import DropoutRegistry, NormDistBase, set_mask_seed
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     reg = DropoutRegistry()
     torch.manual_seed(0)
     side = int(round((args.in_features / 3) ** 0.5))
     assert 3 * side * side == args.in_features, "--in-features must be 3 x side x side for this workload"
-    net = SortMLPModel(args.depth, args.width, (3, side, side), num_classes=args.classes, dropout=args.q,
+    net = SortMLPModel(args.depth, args.width, (3, side, side), num_classes=args.classes, dropout=q,
                        registry=reg).to(dev)
     opt = torch.optim.AdamW(net.parameters(), lr=1e-4, fused=True)
-    from sortnet_amd.layers import NormDistBase
     dist_layers = [m for m in net.modules() if isinstance(m, NormDistBase)]
 
-    def set_p(p):
+    def set_p(v):
         for m in dist_layers:
-            m.p = p
+            m.p = v
 
     g = torch.Generator().manual_seed(0)
     x = torch.rand(args.batch, 3, side, side, generator=g).to(dev)
@@ -124,7 +130,7 @@ def index_list_workload(args):
 
     def train_step():
         net.train()
-        set_p(args.p)
+        set_p(p)
         loss = torch.nn.functional.cross_entropy(net(x), t)
         opt.zero_grad(set_to_none=True)
         loss.backward()
@@ -144,44 +150,43 @@ def index_list_workload(args):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / n
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         train_step()
-    step_s = timed(train_step, args.steps)
-    certify()
-    cert_s = timed(certify, max(2, args.steps // 4))
-    print(json.dumps({
-        "metric": "train samples/s, SortMLPModel in the reference's index-list form", "value": args.batch / step_s,
-        "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": step_s * 1e3,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "SortMLPModel depth %d width %d, B=%d, keep probability %.2f, p=%g: forward + cross entropy + "
-                               "backward + AdamW through kept-channel index lists" % (args.depth, args.width, args.batch, args.q, args.p)},
-        "certification_ms": cert_s * 1e3,
-    }))
+    step_s = timed(train_step, steps)
+    out = {"ms_per_step": step_s * 1e3, "samples_per_s": args.batch / step_s, "steps": steps,
+           "workload": "SortMLPModel depth %d width %d, B=%d, keep probability %.2f, p=%g: forward + cross entropy + "
+                       "backward + AdamW through kept-channel index lists (the reference's training form)"
+                       % (args.depth, args.width, args.batch, q, p)}
+    if certify_runs:
+        certify()
+        cert_s = timed(certify, certify_runs)
+        out["certification_ms"] = cert_s * 1e3
+    del net, opt
+    torch.cuda.empty_cache()
+    return out
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (no collective path exists); run with --gpus 1",
-              file=sys.stderr)
-        sys.exit(2)
-    if args.workload == "index-lists":
-        return index_list_workload(args)
+def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width=None, classes=None, eps=None,
+               time_ibp=False, calib_copy=False):
+    """K timed steps of the fused-mask formulation; returns timings, phase split and the per-launch events of the
+    interval-bound forward of the width x width layers."""
     import torch
     from sortnet_amd import ext
     from sortnet_amd.model import DistanceMLP, margins, hinge_loss
-
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    batch = batch or args.batch
+    in_features = in_features or args.in_features
+    width = width or args.width
+    classes = classes or args.classes
+    eps = args.eps if eps is None else eps
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    mode = ext.MASK_TERM if args.mask == "term" else ext.MASK_FACTORED
-    model = DistanceMLP(args.in_features, args.width, args.depth, args.classes, q=args.q, device=dev, seed=0,
-                        mask_mode=mode)
+    mode = ext.MASK_TERM if mask == "term" else ext.MASK_FACTORED
+    model = DistanceMLP(in_features, width, args.depth, classes, q=q, device=dev, seed=0, mask_mode=mode)
     opt = torch.optim.AdamW(model.parameters(), lr=1e-4, fused=True)
     g = torch.Generator().manual_seed(0)
-    x = torch.rand(args.batch, args.in_features, generator=g).to(dev)
-    targets = torch.randint(0, args.classes, (args.batch,), generator=g).to(dev)
-    lower, upper = (x - args.eps).clamp(min=0), (x + args.eps).clamp(max=1)
+    x = torch.rand(batch, in_features, generator=g).to(dev)
+    targets = torch.randint(0, classes, (batch,), generator=g).to(dev)
+    lower, upper = (x - eps).clamp(min=0), (x + eps).clamp(max=1)
 
     ev = lambda: torch.cuda.Event(enable_timing=True)
     phase_ms = {"forward": 0.0, "backward": 0.0, "optimizer": 0.0, "bounds": 0.0}
@@ -191,7 +196,7 @@ def main():
         marks = [ev() for _ in range(5)]
         marks[0].record()
         dist = model.forward(x, step_seed=i)
-        logits, worst = margins(dist, targets, args.eps)
+        logits, worst = margins(dist, targets, eps)
         loss = hinge_loss(worst)
         marks[1].record()
         opt.zero_grad(set_to_none=True)
@@ -199,8 +204,9 @@ def main():
         marks[2].record()
         opt.step()
         marks[3].record()
-        if timed:
-            # per-launch timing of the dominant kernel: the interval-bound forward of a width x width layer
+        if timed and time_ibp:
+            # same certification pass, spelled out to time every launch of the dominant kernel (the interval-bound
+            # forward of a width x width layer) with events on the stream it is queued on (torch's current stream)
             lo, up = lower.unsqueeze(-1).contiguous(), upper.unsqueeze(-1).contiguous()
             with torch.no_grad():
                 for li, w in enumerate(model.weights):
@@ -210,30 +216,30 @@ def main():
                     e0.record()
                     ext.bound_inf_dist_forward_nograd(lo, up, w, ylo, yup, 1)
                     e1.record()
-                    if w.size(0) == args.width and w.size(1) == args.width:
+                    if w.size(0) == width and w.size(1) == width:
                         ibp_events.append((e0, e1))
                     shift = (model.running_mean[li].view(1, -1, 1) if li < model.num_layers - 1
                              else -model.bias.view(1, -1, 1))
                     lo, up = ylo - shift, yup - shift
-                cert = margins(dist.detach(), targets, args.eps, lo.squeeze(-1), up.squeeze(-1))[1]
+                cert = margins(dist.detach(), targets, eps, lo.squeeze(-1), up.squeeze(-1))[1]
         else:
             lo, up = model.bounds(lower, upper)
-            cert = margins(dist.detach(), targets, args.eps, lo, up)[1]
+            cert = margins(dist.detach(), targets, eps, lo, up)[1]
         marks[4].record()
         return marks, loss, cert
 
-    for i in range(args.warmup):
+    for i in range(warmup):
         step(i, False)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     all_marks = []
-    for i in range(args.steps):
-        marks, loss, cert = step(args.warmup + i, True)
+    for i in range(steps):
+        marks, loss, cert = step(warmup + i, True)
         all_marks.append(marks)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
-    if args.calib_copy:
+    if calib_copy:
         src = model.weights[1]
         dst = torch.empty_like(src)
         dst.copy_(src)
@@ -241,42 +247,116 @@ def main():
 
     for marks in all_marks:
         for k, (a, b) in zip(phase_ms, zip(marks[:-1], marks[1:])):
-            phase_ms[k] += a.elapsed_time(b) / args.steps
-    ms_per_step = elapsed * 1e3 / args.steps
-    value = args.batch / (elapsed / args.steps)
+            phase_ms[k] += a.elapsed_time(b) / steps
+    res = {
+        "ms_per_step": elapsed * 1e3 / steps, "samples_per_s": batch / (elapsed / steps), "steps": steps,
+        "phase_ms": phase_ms, "terms_per_step": model.terms_per_sample() * batch,
+        "ibp_launch_ms": [a.elapsed_time(b) for a, b in ibp_events],
+        "loss": float(loss.detach()), "certified_frac": float((cert.max(dim=1)[0] < 0).float().mean()),
+    }
+    del model, opt
+    torch.cuda.empty_cache()
+    return res
 
-    terms = model.terms_per_sample() * args.batch
-    step_flops = terms * (2 + 6)                      # forward 2 flops/term, interval bounds 6 flops/term
+
+def committed_traffic():
+    """traffic_bytes_per_launch of the committed counter summary, or None."""
+    try:
+        m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(TRAFFIC_PROFILE).read(), re.M)
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def workload_text(args, mask, q):
+    return ("SortNet-MLP training step: %d->%s->%d distance layers, B=%d, q=%.2f (%s), "
+            "forward+hinge loss+backward+AdamW+interval bounds eps=%.4f"
+            % (args.in_features, "x".join([str(args.width)] * (args.depth - 1)), args.classes, args.batch, q,
+               "no mask: pure l-inf net" if q >= 1.0 else
+               ("independent Bernoulli draw per term" if mask == "term" else
+                "factored mask keep_x(b,n)&keep_w(m,n), each output a max over a Bernoulli(q) subset"), args.eps))
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (no collective path exists); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.workload == "index-lists":
+        r = run_index_lists(args, args.q, args.p, args.steps, args.warmup, certify_runs=max(2, args.steps // 4))
+        print(json.dumps({
+            "metric": "train samples/s, SortMLPModel in the reference's index-list form", "value": r["samples_per_s"],
+            "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": r["workload"]}, "certification_ms": r["certification_ms"]}))
+        return
+
+    head = run_masked(args, args.mask, args.q, args.steps, args.warmup, time_ibp=True, calib_copy=args.calib_copy)
+    step_s = head["ms_per_step"] * 1e-3
+    step_flops = head["terms_per_step"] * (2 + 6)         # forward 2 flops/term, interval bounds 6 flops/term
     layer_terms = args.batch * args.width * args.width
-    ibp_ms = sum(a.elapsed_time(b) for a, b in ibp_events) / max(len(ibp_events), 1)
-    achieved = 6.0 * layer_terms / (ibp_ms * 1e-3) / 1e12 if ibp_events else None
+    launches = head["ibp_launch_ms"]
+    ibp_ms = sum(launches) / max(len(launches), 1)
+    achieved = 6.0 * layer_terms / (ibp_ms * 1e-3) / 1e12 if launches else None
+    tb = 4 if args.batch > 32 else 2
     roofline = {
-        "bound": "valu", "kernel": "fwd_kernel<BoundNograd,4,8> (interval bounds, %dx%dx%d)" % (args.batch, args.width, args.width),
+        "bound": "valu",
+        "kernel": "sd::fwd_kernel_pipe<sd::BoundNograd, %d, 8> (interval-bound forward, %dx%dx%d)" % (tb, args.batch, args.width, args.width),
         "achieved": achieved, "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": achieved / FP32_VECTOR_PEAK_TFLOPS if achieved else None,
-        "traffic": IBP_LAUNCH_TRAFFIC_BYTES if (args.batch, args.width) == (512, 5120) else None,
+        "traffic": committed_traffic() if (args.batch, args.width) == (512, 5120) else None,
         "algorithmic_bytes": 4.0 * (args.width * args.width + 4 * args.batch * args.width),
-        "avg_launch_ms": ibp_ms, "launches_timed": len(ibp_events),
-        "valu_issue_frac": 4.0 * layer_terms / (ibp_ms * 1e-3) / VALU_LANE_RATE if ibp_events else None,
+        "avg_launch_ms": ibp_ms, "launches_timed": len(launches),
+        "valu_issue_frac": 4.0 * layer_terms / (ibp_ms * 1e-3) / VALU_LANE_RATE if launches else None,
         "note": "tropical (sub/min/max) contraction on the fp32 vector ALUs, not MFMA; 6 flops per term in 4 VALU "
                 "instructions; a register-only stream of this mix reaches 72 T lane-instructions/s on this part "
                 "(floor 56 fs/term = 69% of peak) and the part sustains ~2.0 of its 2.4 GHz under this kernel",
     }
     out = {
         "metric": "train samples/s (fwd+bwd+IBP) 5x5120 SortNet-MLP, B=512; % FP32 VALU peak",
-        "value": value, "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": head["samples_per_s"], "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "SortNet-MLP training step: %d->%s->%d distance layers, B=%d, q=%.2f (%s mask), "
-                               "forward+hinge loss+backward+AdamW+interval bounds eps=%.4f"
-                               % (args.in_features, "x".join([str(args.width)] * (args.depth - 1)), args.classes,
-                                  args.batch, args.q, args.mask, args.eps),
+        "config": {"workload": workload_text(args, args.mask, args.q),
                    "batch": args.batch, "width": args.width, "distance_layers": args.depth, "mask": args.mask},
-        "step_fp32_vector_frac": step_flops / (elapsed / args.steps) / (FP32_VECTOR_PEAK_TFLOPS * 1e12),
-        "phase_ms": phase_ms,
+        "step_fp32_vector_frac": step_flops / step_s / (FP32_VECTOR_PEAK_TFLOPS * 1e12),
+        "phase_ms": head["phase_ms"],
         "roofline": roofline,
-        "loss": float(loss.detach()), "certified_frac": float((cert.max(dim=1)[0] < 0).float().mean()),
+        "loss": head["loss"], "certified_frac": head["certified_frac"],
     }
+
+    if not args.no_secondary:
+        sec = {}
+        short, warm = max(3, args.steps // 4), 2
+
+        def masked_entry(mask, q, **kw):
+            r = run_masked(args, mask, q, short, warm, **kw)
+            return {"ms_per_step": r["ms_per_step"], "samples_per_s": r["samples_per_s"], "steps": short,
+                    "phase_ms": r["phase_ms"]}
+
+        other = "term" if args.mask == "factored" else "factored"
+        sec[other + "_mask"] = dict(masked_entry(other, args.q), workload=workload_text(args, other, args.q))
+        sec["q1"] = dict(masked_entry(args.mask, 1.0), workload=workload_text(args, args.mask, 1.0))
+        # the reference's own training form at the keep probability of its published commands (0.7-0.85)
+        r = run_index_lists(args, 0.75, float("inf"), short, warm, certify_runs=3)
+        sec["index_lists_q0.75_inf"] = {k: r[k] for k in ("ms_per_step", "samples_per_s", "steps", "workload")}
+        sec["certification"] = {"ms_per_pass": r["certification_ms"],
+                                "workload": "evaluation-mode pass of the same model: sort neuron (K=10) for the value, "
+                                            "interval sort neuron for the bounds, all layers, B=%d" % args.batch}
+        r = run_index_lists(args, 0.75, 8.0, short, warm)
+        sec["index_lists_q0.75_p8"] = {k: r[k] for k in ("ms_per_step", "samples_per_s", "steps", "workload")}
+        if (args.batch, args.width, args.in_features, args.classes) == (512, 5120, 3072, 10):
+            r = run_masked(args, args.mask, args.q, short, warm, batch=256, in_features=12288, width=10240, classes=200,
+                           eps=1.0 / 255)
+            sec["wide"] = {"ms_per_step": r["ms_per_step"], "samples_per_s": r["samples_per_s"], "steps": short,
+                           "phase_ms": r["phase_ms"],
+                           "workload": "same step, 64x64 images: 12288->4x10240->200, B=256, q=%.2f (%s mask), eps=1/255"
+                                       % (args.q, args.mask)}
+        out["secondary"] = sec
+
     dims = [args.in_features] + [args.width] * (args.depth - 1) + [args.classes]
     out["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args, dims)
     print(json.dumps(out))

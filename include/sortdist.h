@@ -22,6 +22,10 @@
  * caller-visible memory.  pos packs the arg-max input index in bits 0..30 and a branch/sign
  * flag in bit 31.
  *
+ * The backward entry points trust pos: bits 0..30 must be below CI / G (the forward entry points
+ * only write such values); an index outside that range is read or written out of bounds, as in
+ * the reference.
+ *
  * Scratch memory: the library keeps one device buffer per (GPU, stream) for partial results
  * (split reductions, mask bits, candidate lists, per-slice sums) and grows it on demand with
  * hipMalloc; growing waits for that stream first.  Calls are asynchronous on `stream`; calls

@@ -7,8 +7,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# SORTNET_AMD_LIB selects another build of the same library (e.g. an experimental one)
-LIB_PATH = os.environ.get("SORTNET_AMD_LIB") or os.path.join(_HERE, "libsortdist.so")
+LIB_PATH = os.path.join(_HERE, "libsortdist.so")
 
 _F = ctypes.c_void_p          # device pointer to float
 _I = ctypes.c_void_p          # device pointer to int32

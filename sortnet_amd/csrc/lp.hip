@@ -21,11 +21,12 @@ static inline int int_power(float p) {
 // ratio below which a term of r^p is dropped (see lp_add_significant); 0 when it is below `from`, i.e. when too
 // many terms would pass for the wavefront-level tests to pay
 static inline float lp_skip_threshold(float drop, float p, float from) {
-    // SORTDIST_LP_SKIP=0 turns the tests off: they cost 10-20 % when the terms of a row are spread evenly up
-    // to its maximum (uniformly distributed |x - w|) instead of thinning out towards it
-    static const bool enabled = [] { const char* e = getenv("SORTDIST_LP_SKIP"); return !(e && e[0] == '0'); }();
+    // the test only makes sense for an exponent above 1: then 0 < thr < 1 and ratios below it are small.  For
+    // an exponent of at most 1 (backward with p <= 2) drop^(1/p) is no threshold at all (it exceeds 1 for
+    // negative exponents) and every term is evaluated.
+    if (!(p > 1.f)) return 0.f;
     const float thr = powf(drop, 1.f / p);
-    return enabled && thr >= from ? thr : 0.f;
+    return (thr >= from && thr < 1.f) ? thr : 0.f;
 }
 
 template <template <int> class Pol, int TB, int TM>
@@ -543,8 +544,10 @@ static int lp_backward(const char* who, const float* grad_output, const float* i
     a.ci_idx = ci_idx; a.co_idx = co_idx;
     a.B = B; a.R = f.R; a.HW = HW; a.G = G; a.COg = f.COg; a.CIg = f.CIg; a.W_COg = f.W_COg; a.W_CIg = f.W_CIg;
     a.pm1 = p - 1.f;
-    // a dropped term is below 1e-7 / (terms per sum) of a ratio that is at most 1
-    a.skip_thr = int_power(p - 1.f) < 0 ? lp_skip_threshold(1e-7f / (float)(f.COg > f.R ? f.COg : f.R), p - 1.f, kLpSkipFrom) : 0.f;
+    // a dropped term has (|d| / y)^(p-1) < 1e-16: the reference trains with AdamW at eps = 1e-10 (main.py:38,432), which
+    // turns gradient entries far below the parity bar into full-size updates, so the cut sits where even the sum of
+    // all dropped terms of an entry (at most 1e-16 x terms x |grad_output|) cannot move such an update visibly
+    a.skip_thr = int_power(p - 1.f) < 0 ? lp_skip_threshold(1e-16f, p - 1.f, kLpSkipFrom) : 0.f;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int ip = int_power(p - 1.f);
     // large p with both gradients in the dense single-group case: the kernel that forms every term once for both

@@ -92,23 +92,22 @@ class MeanShiftDropout(nn.Module):
     def forward(self, x=None, lower=None, upper=None, index=None):
         if self.training:
             assert x is not None, "Currently not supported"
-            if self.bias is None:
-                # fused kernels: mean, running-mean update and subtraction
+            if self.bias is None and lower is None and upper is None:
+                # fused kernels: mean, running-mean update and subtraction (own backward)
                 if index is None:
                     x, _ = F.mean_shift(x.contiguous(), self.running_mean, self.momentum)
                 else:
                     x, _ = F.mean_shift_index(x, index.to(torch.int32).contiguous(), self.out_channels,
                                               self.running_mean, self.momentum)
-                mean = None
-            else:
-                index = None if index is None else index.long()
-                mean = self._batch_mean(x, index)
-                with torch.no_grad():
-                    self.running_mean.mul_(1 - self.momentum).add_(mean, alpha=self.momentum)
+                return x, lower, upper
+            # bounds alongside x, or an affine bias: the batch mean of x, inside the graph, is subtracted from
+            # all three (core/models/bound_basic_module.py:125-157)
+            index = None if index is None else index.long()
+            mean = self._batch_mean(x, index)
+            with torch.no_grad():
+                self.running_mean.mul_(1 - self.momentum).add_(mean, alpha=self.momentum)
         else:
             mean = self.running_mean
-        if mean is None:
-            return x, lower, upper
         if self.bias is not None:
             mean = mean - self.bias
         if index is not None:
@@ -117,8 +116,6 @@ class MeanShiftDropout(nn.Module):
             per_row = mean.view(1, index.size(-2), -1).expand(x.size(0), -1, -1)
             mean_b = torch.gather(per_row, -1, index[rows]).reshape(x.size(0), -1).unsqueeze(-1)
             return tuple(apply_if_not_none((x, lower, upper), lambda z: z - mean_b))
-        if self.training:
-            return tuple(apply_if_not_none((x, lower, upper), lambda z: z - mean.view(1, -1, 1)))
         return tuple(apply_if_not_none((x, lower, upper), lambda z: _shift(z, mean, -1.0)))
 
     def _batch_mean(self, x, index):
@@ -139,6 +136,10 @@ class MeanShiftDropout(nn.Module):
 
 
 def _shift(z, vec, sign):
+    """z + sign * vec[channel].  The kernel form has no backward, so it only serves tensors outside a graph
+    (the attack differentiates an evaluation-mode stack with respect to its input, attack.py:26-29)."""
+    if torch.is_grad_enabled() and (z.requires_grad or vec.requires_grad):
+        return z + sign * vec.view(1, -1, 1)
     out = torch.empty_like(z)
     ext.channel_shift(z.contiguous(), vec.contiguous(), sign, out)
     return out

@@ -1,4 +1,4 @@
-"""The distance-layer stack that the benchmark and the end-to-end tests drive: the `fc_dist`
+"""The distance-layer stack that the benchmark times and tests/test_gpu_bench_stack.py checks against the oracle: the `fc_dist`
 part of the reference's SortMLPModel (ell_inf_models.py:17-50) -- `depth - 1` distance layers of
 equal width with mean shift, then a distance layer onto the classes with a bias -- and the
 reference's hinge loss on the 1-Lipschitz margin (main.py:329-335, ell_inf_models.py:45-50).
@@ -12,6 +12,7 @@ import torch
 
 from . import functional as F
 from .ext import MASK_TERM
+from .losses import hinge_loss  # noqa: F401  (the benchmark's loss)
 
 
 class DistanceMLP:
@@ -34,18 +35,34 @@ class DistanceMLP:
     def terms_per_sample(self):
         return sum(w.numel() for w in self.weights)
 
-    def forward(self, x, step_seed):
-        """Training forward: x (B, in_features) -> distances to the class prototypes (B, classes)."""
+    def forward(self, x, step_seed, trace=None):
+        """Training forward: x (B, in_features) -> distances to the class prototypes (B, classes).
+        `trace`, a list, receives per layer (input, raw distances, batch mean or None) for inspection."""
         h = x.unsqueeze(-1)
         for i, w in enumerate(self.weights):
+            h_in = h
             if i == 0 or self.q is None or self.q == 1.0:
                 h = F.norm_dist(h, w, float("inf"))
             else:
                 h = F.masked_inf_dist(h, w, self.q, seed=step_seed * 64 + i, mode=self.mask_mode)
+            y, mean = h, None
             if i < self.num_layers - 1:
-                h, _ = F.mean_shift(h, self.running_mean[i], self.momentum)
+                h, mean = F.mean_shift(h, self.running_mean[i], self.momentum)
             else:
                 h = h + self.bias.view(1, -1, 1)
+            if trace is not None:
+                trace.append((h_in.detach(), y.detach(), mean))
+        return h.squeeze(-1)
+
+    @torch.no_grad()
+    def predict(self, x):
+        """Evaluation forward of the pure l-inf net (q = 1): every layer without a mask, mean shift taken from
+        the running means -- the value that `bounds()` brackets."""
+        h = x.unsqueeze(-1).contiguous()
+        for i, w in enumerate(self.weights):
+            h = F.norm_dist(h, w, float("inf"))
+            shift = self.running_mean[i].view(1, -1, 1) if i < self.num_layers - 1 else -self.bias.view(1, -1, 1)
+            h = h - shift
         return h.squeeze(-1)
 
     @torch.no_grad()
@@ -68,9 +85,3 @@ def margins(dist, targets, eps, lower=None, upper=None):
     margin = up - torch.gather(lo, 1, targets.view(-1, 1))
     margin = margin.scatter(1, targets.view(-1, 1), 0)
     return logits, margin / (2 * eps)
-
-
-def hinge_loss(worst_outputs, mix=0.25):
-    """main.py:329-335."""
-    res = worst_outputs.clamp(min=0)
-    return (1 - mix) * res.max(dim=1)[0].mean() + mix * res.mean()

@@ -188,7 +188,7 @@ def main():
 
     xn = rng_inputs(14, (B, N), "randn")
     out["lp"] = {"x": xn.tolist(), "w": w.tolist(), "g": g.tolist(), "cases": []}
-    for p in (3.0, 8.0, 20.0, 9.5):
+    for p in (3.0, 8.0, 20.0, 9.5, 4.0, 5.0, 6.0, 9.0, 1.5):
         y = lp_forward(xn, w, p)
         gx, gw = lp_backward(g.astype(np.float64), xn, w, y, p)
         out["lp"]["cases"].append({"p": p, "y": y.tolist(), "gx": gx.tolist(), "gw": gw.tolist()})

@@ -328,7 +328,8 @@ def test_sort_neuron_widest_rows(oracle):
         _close(y, ry)
 
 
-@pytest.mark.parametrize("p", [1.0, 2.0, 3.0, 7.0, 8.0, 9.5, 11.3, 64.0, 300.0])
+# every integer-power chain (forward p = 1..8, backward p - 1 = 0..8), exponents below 1 on either side, general p
+@pytest.mark.parametrize("p", [0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0, 8.0, 9.0, 9.5, 11.3, 64.0, 300.0])
 @pytest.mark.parametrize("B,CI,CO,G,HW", [SHAPES[1], SHAPES[3], SHAPES[4]])
 def test_norm_dist(oracle, p, B, CI, CO, G, HW):
     from sortnet_amd import ext
@@ -375,6 +376,11 @@ def test_norm_dist_index_lists(oracle, p, B, CI, CO, G, ci_n, co_n):
     ext.norm_dist_backward_input_weight(gd, xd, wd, torch.from_numpy(ry).to(dev), gx, gw, G, p, cid, cod)
     _close(gx, rgx)
     _close(gw, rgw)
+    # caller-supplied maximum with index lists (any scale at or above the true maximum gives the same norm)
+    mx = torch.from_numpy(oracle.inf_dist_forward(x.numpy(), w.numpy(), G, False, ci, co) * np.float32(1.25)).to(dev)
+    y2 = torch.empty_like(y)
+    ext.norm_dist_forward_with_max(xd, wd, mx, y2, G, p, cid, cod)
+    np.testing.assert_allclose(y2.cpu().numpy(), ry, rtol=RTOL)
     # only output channels dropped / only input channels dropped
     xfull = _gen((B, CI, 1), 49)
     y3 = torch.empty(B, co_n * G, 1, device=dev)
@@ -420,6 +426,32 @@ def test_norm_dist_large_p(oracle, p, kind):
         gx.fill_(float("nan"))
         ext.norm_dist_backward_input(gd, xd, wd, torch.from_numpy(ry).to(dev), gx, 1, p, ad, bd)
         _close(gx, rgx, rtol=max(RTOL, 1e-6 * p))
+
+
+@pytest.mark.parametrize("p", [128.0, 400.0])
+def test_norm_dist_large_p_adam_update(oracle, p):
+    """The reference trains with AdamW at eps = 1e-10 (main.py:38,432): a gradient entry of 1e-9 still produces a
+    full-size update.  The backward kernels leave out terms with (|d| / y)^(p-1) < 1e-16; the first Adam update
+    g / (|g| + eps) from their gradients must agree with the one from the oracle's gradients (which sum every
+    term in double precision), also where whole gradient entries consist of tiny terms only."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, CI, CO = 64, 1024, 96
+    x, w, gy = _gen((B, CI, 1), 81), _gen((CO, CI), 82, scale=0.3), _gen((B, CO, 1), 83)
+    ry = oracle.norm_dist_forward(x.numpy(), w.numpy(), p)
+    rgx, rgw = oracle.norm_dist_backward(gy.numpy(), x.numpy(), w.numpy(), ry, p)
+    xd, wd, gd, yd = x.to(dev), w.to(dev), gy.to(dev), torch.from_numpy(ry).to(dev)
+    gx, gw = torch.empty_like(xd), torch.empty_like(wd)
+    ext.norm_dist_backward_input_weight(gd, xd, wd, yd, gx, gw, 1, p)
+    gx2 = torch.empty_like(xd)
+    ext.norm_dist_backward_input(gd, xd, wd, yd, gx2, 1, p)
+    eps = 1e-10
+    for got, ref in ((gw, rgw), (gx, rgx), (gx2, rgx)):
+        got = got.cpu().numpy().astype(np.float64)
+        ref = ref.astype(np.float64)
+        upd_got, upd_ref = got / (np.abs(got) + eps), ref / (np.abs(ref) + eps)
+        assert np.abs(ref).min() < 1e-8 < np.abs(ref).max()       # the data does hold entries in Adam's eps range
+        assert np.abs(upd_got - upd_ref).max() < 2e-3, p
 
 
 def test_config1_full_size(oracle):
