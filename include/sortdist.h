@@ -69,6 +69,18 @@ int sd_inf_dist_forward(const float* input, const float* weight,
                         int B, int CO, int CI, int G, int HW, float* output, int* pos,
                         const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI, sd_stream_t stream);
 
+/* No counterpart in the reference.  sd_inf_dist_forward for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): same arguments and
+ * results, but the scratch of its split reduction lives in a 32 MiB device array built into the library
+ * instead of the grow-only workspace, and the call performs no hipMalloc / hipFree.  At most
+ * 4 194 304 outputs (B * CO * HW); larger calls return SD_ERR_ARG.  The first call on a GPU looks the
+ * array's address up (make it before any capture).  All calls on one GPU share the array: calls that
+ * overlap on one GPU (other streams or threads) race. */
+int sd_inf_dist_forward_noalloc(const float* input, const float* weight,
+                                int B, int CO, int CI, int G, int HW, float* output, int* pos,
+                                const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
+                                sd_stream_t stream);
+
 /* inf_dist::backward_input (norm_dist.h:26-27; inf_dist_cuda.cu:325-336). */
 int sd_inf_dist_backward_input(const float* grad_output, const int* pos,
                                int B, int CO, int CI, int G, int HW, float* grad_input, sd_stream_t stream);

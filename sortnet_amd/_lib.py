@@ -20,6 +20,7 @@ _u = ctypes.c_uint32
 SIGNATURES = {
     "sd_inf_dist_forward_nograd": [_F, _F, _i, _i, _i, _i, _i, _F, _S],
     "sd_inf_dist_forward": [_F, _F, _i, _i, _i, _i, _i, _F, _I, _I, _I, _i, _i, _S],
+    "sd_inf_dist_forward_noalloc": [_F, _F, _i, _i, _i, _i, _i, _F, _I, _I, _I, _i, _i, _S],
     "sd_inf_dist_backward_input": [_F, _I, _i, _i, _i, _i, _i, _F, _S],
     "sd_inf_dist_backward_input_weight": [_F, _I, _i, _i, _i, _i, _i, _F, _F, _I, _I, _i, _i, _S],
     "sd_bound_inf_dist_forward_nograd": [_F, _F, _F, _i, _i, _i, _i, _i, _F, _F, _S],

@@ -1,6 +1,7 @@
 // l-inf distance, masked order-statistic neuron and interval-bound forward entry points.
 #include "fwd_tile.h"
 #include "fwd_args.h"
+#include <mutex>
 
 using namespace sd;
 
@@ -24,8 +25,10 @@ static __global__ void __launch_bounds__(256) build_masks_kernel(uint32_t* __res
 
 // forward with positions: chunk-tracking kernel (split-N through the packed workspace when the
 // grid would otherwise be too small) followed by the position resolve pass
+// merge_buf / merge_cap: caller-supplied memory for the split-N merge instead of the library workspace (the entry
+// point that allocates nothing); a problem that needs more than merge_cap bytes is rejected
 template <class P>
-static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st) {
+static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st, void* merge_buf = nullptr, size_t merge_cap = 0) {
     // with index lists a batch tile must stay inside one 32-sample sub-batch
     static const int kTb42[] = {4, 2};
     const int TB = index_lists ? 2 : pick_tb(a, kTb42, 2, 16 * P::WIDE_TM);
@@ -36,7 +39,11 @@ static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st) {
         // the merge buffer sits at the start of the workspace; a factored-mask call has already sized
         // the workspace for it and placed its bit masks behind it
         size_t n = (size_t)a.R * a.G * a.COg;
-        a.packed0 = static_cast<unsigned long long*>(a.xmask ? workspace(0, st) : workspace(n * 8, st));
+        if (merge_buf) {
+            SD_REQUIRE(n * 8 <= merge_cap, "inf_dist_forward_noalloc: %zu outputs need %zu bytes of merge scratch, the "
+                       "built-in buffer holds %zu (at most %zu outputs)", n, n * 8, merge_cap, merge_cap / 8);
+            a.packed0 = static_cast<unsigned long long*>(merge_buf);
+        } else a.packed0 = static_cast<unsigned long long*>(a.xmask ? workspace(0, st) : workspace(n * 8, st));
         if (!a.packed0) return SD_ERR_HIP;
         if ((rc = fill_zero(a.packed0, n * 2, st))) return rc;
     }
@@ -74,6 +81,59 @@ extern "C" int sd_inf_dist_forward(const float* input, const float* weight,
     a.y0 = output; a.p0 = pos;
     hipStream_t st = static_cast<hipStream_t>(stream);
     return run_chunk_pos<LinfChunk>(a, w_index_ci || w_index_co, st);
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------------
+// Same operation as sd_inf_dist_forward for callers that cannot call hipMalloc (code under graph capture,
+// serving loops, harnesses that forbid allocation).  The split-N merge buffer, which sd_inf_dist_forward takes
+// from the grow-only library workspace, lives in a file-scope device array instead.  Every GPU holds its own
+// copy of the array at its own address: the address is looked up once per device with hipGetSymbolAddress and
+// only that pointer is ever handed to kernels.  All calls on one GPU share the array, so calls that overlap on
+// one GPU (different streams or threads) race; the part a call uses is cleared by a fill kernel first.
+constexpr size_t kScratchBytes = (size_t)32 << 20;   // 4 Mi outputs of 8 bytes: covers 512 x 5120 outputs
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+static int scratch_address(void** out) {
+    static std::mutex mu;
+    static void* ptrs[64] = {nullptr};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        (void)hipGetLastError();
+        set_error("inf_dist_forward_noalloc: no current device");
+        return SD_ERR_HIP;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            set_error("inf_dist_forward_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return SD_ERR_HIP;
+        }
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return SD_OK;
+}
+
+extern "C" int sd_inf_dist_forward_noalloc(const float* input, const float* weight,
+                                           int B, int CO, int CI, int G, int HW, float* output, int* pos,
+                                           const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
+                                           sd_stream_t stream) {
+    FwdArgs a;
+    int rc = make_fwd_args(a, "inf_dist_forward_noalloc", input, nullptr, weight, B, CO, CI, G, HW,
+                           w_index_ci, w_index_co, W_CO, W_CI);
+    if (rc) return rc;
+    SD_REQUIRE(output && pos, "inf_dist_forward_noalloc: null output or pos");
+    a.y0 = output; a.p0 = pos;
+    const size_t outputs = (size_t)B * CO * HW;
+    SD_REQUIRE(outputs * 8 <= kScratchBytes, "inf_dist_forward_noalloc: %zu outputs exceed the maximum of %zu "
+               "(8 bytes of built-in merge scratch per output, %zu bytes in all); use sd_inf_dist_forward",
+               outputs, kScratchBytes / 8, kScratchBytes);
+    void* buf = nullptr;
+    if ((rc = scratch_address(&buf))) return rc;
+    return run_chunk_pos<LinfChunk>(a, w_index_ci || w_index_co, static_cast<hipStream_t>(stream), buf, kScratchBytes);
 }
 
 extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weight,
