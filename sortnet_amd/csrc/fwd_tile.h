@@ -499,9 +499,17 @@ __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_lis
     }
 }
 
+}  // namespace sd
+#include "fwd_direct.h"
+namespace sd {
+
 // host-side launcher; the caller has validated shapes
 template <class P, int TB, int TM>
 int launch_fwd(const FwdArgs& a, hipStream_t stream) {
+    // exact dense tiles of the policies that opt in go through the LDS-direct kernel
+    if constexpr (P::DIRECT && TB % 4 == 0 && TM % 4 == 0) {
+        if (direct_ok<TB, TM>(a)) return launch_fwd_direct<P, TB, TM>(a, stream);
+    }
     dim3 grid((a.COg + 16 * TM - 1) / (16 * TM), (a.R + 16 * TB - 1) / (16 * TB), a.G * a.nsplit);
     if (a.fast_x && a.fast_w && (a.mask_mode != SD_MASK_FACTORED || a.xmask)) {
         hipLaunchKernelGGL((fwd_kernel_pipe<P, TB, TM>), grid, dim3(256), 0, stream, a);
@@ -529,12 +537,14 @@ struct PolicyBase {
     static constexpr int PIPE_WAVES_TM4 = 0, UNROLL4_TM4 = 0;   // overrides for tiles of <= 4 channels (0: none)
     static constexpr int WIDE_TB = 4, WIDE_TM = 8;   // register tile of the large-batch launch of position kernels
     static constexpr bool LISTS = false;  // also built as fwd_kernel_lists (ops that accept kept-channel index lists)
+    static constexpr bool DIRECT = false; // also built as fwd_kernel_direct (global -> LDS loads, exact dense tiles)
     template <class A> static __device__ __forceinline__ void chunk_end(A&, const FwdArgs&, int, int) {}
 };
 
 // l-inf forward without indices (core/cuda/inf_dist_cuda.cu:17-107)
 struct LinfNograd : PolicyBase {
     static constexpr bool LISTS = true;
+    static constexpr bool DIRECT = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int MIN_WAVES = 3;
     static constexpr int UNROLL4 = 1;
@@ -654,6 +664,7 @@ struct MaskedTermMax : PolicyBase {
 
 // interval bounds, values only (core/cuda/bound_inf_dist_cuda.cu:15-118)
 struct BoundNograd : PolicyBase {
+    static constexpr bool DIRECT = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int NX = 2;
     static constexpr int MIN_WAVES = 3;
@@ -911,6 +922,7 @@ __device__ __forceinline__ float add_pow(float s, float a, float p) {
 template <int IP>
 struct LpPlain : PolicyBase {
     static constexpr bool LISTS = true;
+    static constexpr bool DIRECT = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int MIN_WAVES = 3;
     struct Acc { float s; };
@@ -991,6 +1003,7 @@ struct LpOnline : PolicyBase {
 template <int IP, bool FOLD = (IP < 0)>
 struct LpWithMax : PolicyBase {
     static constexpr bool LISTS = true;
+    static constexpr bool DIRECT = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int MIN_WAVES = 3;
     // rinv = 1 / maximum; FOLD (general p) keeps c = p log2(1 / maximum) instead, so that a term is
