@@ -171,7 +171,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     """K timed steps of the fused-mask formulation; returns timings, phase split and the per-launch events of the
     interval-bound forward of the width x width layers."""
     import torch
-    from sortnet_amd import ext
+    from sortnet_amd import ext, _lib
     from sortnet_amd.model import DistanceMLP, margins, hinge_loss
     batch = batch or args.batch
     in_features = in_features or args.in_features
@@ -191,6 +191,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     ev = lambda: torch.cuda.Event(enable_timing=True)
     phase_ms = {"forward": 0.0, "backward": 0.0, "optimizer": 0.0, "bounds": 0.0}
     ibp_events = []
+    ibp_kernel = [None]          # the tile kernel the library dispatched for the width x width interval layers
 
     def step(i, timed):
         marks = [ev() for _ in range(5)]
@@ -218,6 +219,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
                     e1.record()
                     if w.size(0) == width and w.size(1) == width:
                         ibp_events.append((e0, e1))
+                        ibp_kernel[0] = _lib.last_forward_kernel()
                     shift = (model.running_mean[li].view(1, -1, 1) if li < model.num_layers - 1
                              else -model.bias.view(1, -1, 1))
                     lo, up = ylo - shift, yup - shift
@@ -251,7 +253,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     res = {
         "ms_per_step": elapsed * 1e3 / steps, "samples_per_s": batch / (elapsed / steps), "steps": steps,
         "phase_ms": phase_ms, "terms_per_step": model.terms_per_sample() * batch,
-        "ibp_launch_ms": [a.elapsed_time(b) for a, b in ibp_events],
+        "ibp_launch_ms": [a.elapsed_time(b) for a, b in ibp_events], "ibp_kernel": ibp_kernel[0],
         "loss": float(loss.detach()), "certified_frac": float((cert.max(dim=1)[0] < 0).float().mean()),
     }
     del model, opt
@@ -301,10 +303,9 @@ def main():
     launches = head["ibp_launch_ms"]
     ibp_ms = sum(launches) / max(len(launches), 1)
     achieved = 6.0 * layer_terms / (ibp_ms * 1e-3) / 1e12 if launches else None
-    tb = 4 if args.batch > 32 else 2
     roofline = {
         "bound": "valu",
-        "kernel": "sd::fwd_kernel_pipe<sd::BoundNograd, %d, 8> (interval-bound forward, %dx%dx%d)" % (tb, args.batch, args.width, args.width),
+        "kernel": "sd::%s, policy BoundNograd (interval-bound forward, %dx%dx%d)" % (head["ibp_kernel"], args.batch, args.width, args.width),
         "achieved": achieved, "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": achieved / FP32_VECTOR_PEAK_TFLOPS if achieved else None,
         "traffic": committed_traffic() if (args.batch, args.width) == (512, 5120) else None,

@@ -55,6 +55,10 @@ typedef void* sd_stream_t;
 /* library / error reporting (no reference counterpart) */
 int sd_version(void);
 const char* sd_last_error(void);
+/* Which forward tile kernel the calling thread's last forward call dispatched, with its register tile, e.g.
+ * "fwd_kernel_direct<4,8>" (global -> LDS loads), "fwd_kernel_pipe<4,8>" (register-staged), "fwd_kernel_lists<2,8>"
+ * (gather loads), "fwd_kernel<2,4>" (general): for tests and benchmarks that must know which path they measured. */
+const char* sd_last_forward_kernel(void);
 
 /* ---- l-inf distance: struct inf_dist, core/cuda/norm_dist.h:20-31 ---- */
 

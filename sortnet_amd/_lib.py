@@ -45,6 +45,7 @@ SIGNATURES = {
 _OTHER = {
     "sd_version": ([], _i),
     "sd_last_error": ([], ctypes.c_char_p),
+    "sd_last_forward_kernel": ([], ctypes.c_char_p),
     "sd_rng_word": ([_u, _u, _u, _u], _u),
     "sd_mask_threshold8": ([_f], _u),
     "sd_mask_threshold16": ([_f], _u),
@@ -83,3 +84,8 @@ def call(name, *args):
     if rc != 0:
         msg = lib.sd_last_error()
         raise RuntimeError("%s failed (status %d): %s" % (name, rc, msg.decode() if msg else "?"))
+
+
+def last_forward_kernel():
+    """Name and register tile of the forward tile kernel that this thread's last forward call dispatched."""
+    return load().sd_last_forward_kernel().decode()

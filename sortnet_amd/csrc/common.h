@@ -62,6 +62,8 @@ struct FwdArgs {
 // ---- error reporting ---------------------------------------------------------------------------
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);
+// records which forward tile kernel the calling thread dispatched last (sd_last_forward_kernel)
+void note_forward_kernel(const char* kind, int tb, int tm);
 
 #define SD_REQUIRE(cond, ...)                                   \
     do {                                                        \

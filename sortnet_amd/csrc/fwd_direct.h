@@ -46,13 +46,14 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
 // slot of input group c (0..3) in tile row r
 __device__ __forceinline__ int swz(int c, int r) { return c ^ ((r >> 2) & 3); }
 
-template <class P, int TB, int TM>
+template <class P, int TB, int TM, bool MASKED>
 __global__ void __launch_bounds__(256, 4) fwd_kernel_direct(FwdArgs a) {
     constexpr int BB = 16 * TB, BM = 16 * TM, NX = P::NX;
     constexpr int XG = BB / 16, WG = BM / 16;          // 16-row groups of one x tile / of the w tile
     constexpr int NG = NX * XG + WG;                    // wave-wide loads per chunk
     constexpr int GPW = NG / 4;                         // per wave
     static_assert(P::PASSES == 1, "single-pass policies only");
+    static_assert(!MASKED || P::NX == 1, "the factored mask applies to one-input policies");
     __shared__ __attribute__((aligned(1024))) float tiles[2][NG * 16 * KD];
 
     const int tid = threadIdx.x, tm = tid & 15, tb = tid >> 4;
@@ -102,6 +103,36 @@ __global__ void __launch_bounds__(256, 4) fwd_kernel_direct(FwdArgs a) {
                               __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)((buf * NG + lds_group(v)) * 16 * KD * 4)));
         }
     };
+    // Factored mask: dropped inputs / weights become NaN in LDS (NaN never wins a maximum), from the keep-bit words
+    // that build_masks_kernel left in the workspace (one 32-bit word per row and 32 inputs).  A lane patches the
+    // slots it loaded itself, after its loads have landed and before the barrier publishes them.
+    int moff[GPW];
+    #pragma unroll
+    for (int v = 0; v < GPW; v++) {
+        if (!MASKED) moff[v] = 0;
+        else if (v < XL) moff[v] = ((r0 + (wave + 4 * v) * 16 + lr) * a.G + g) * nchunks;
+        else moff[v] = (g * a.COg + m0 + (wave + 4 * (v - XL)) * 16 + lr) * nchunks;
+    }
+    uint32_t mword[GPW];
+    auto fetch_masks = [&](int k0) {       // words of the 32-input chunk that holds k0
+        if (!MASKED) return;
+        #pragma unroll
+        for (int v = 0; v < GPW; v++) mword[v] = (v < XL ? a.xmask : a.wmask)[moff[v] + k0 / KT];
+    };
+    auto apply_masks = [&](int buf, int k0) {
+        if (!MASKED) return;
+        const float qnan = __builtin_nanf("");
+        #pragma unroll
+        for (int v = 0; v < GPW; v++) {
+            float4* ps = reinterpret_cast<float4*>(&tiles[buf][lds_group(v) * 16 * KD + lane * 4]);
+            float4 t = *ps;
+            const uint32_t bits = mword[v] >> ((k0 & (KT - 1)) + col);
+            t.x = (bits & 1u) ? t.x : qnan; t.y = (bits & 2u) ? t.y : qnan;
+            t.z = (bits & 4u) ? t.z : qnan; t.w = (bits & 8u) ? t.w : qnan;
+            *ps = t;
+        }
+    };
+
     // inverted intervals (lower > upper) become their midpoint (core/cuda/bound_inf_dist_cuda.cu:63); this lane
     // checks the slots it loaded itself, after its loads have landed and before the barrier publishes them
     auto repair = [&](int buf) {
@@ -123,6 +154,8 @@ __global__ void __launch_bounds__(256, 4) fwd_kernel_direct(FwdArgs a) {
     };
 
     typename P::Acc acc[TB][TM];
+    typename P::template TState<TB * TM> tstate;
+    if constexpr (P::HAS_TSTATE) P::tinit(tstate);
     #pragma unroll
     for (int i = 0; i < TB; i++) {
         #pragma unroll
@@ -153,23 +186,35 @@ __global__ void __launch_bounds__(256, 4) fwd_kernel_direct(FwdArgs a) {
         }
     };
 
+    // waits until this wave's LDS-direct loads have landed; the empty statement keeps the compiler from moving the
+    // LDS reads of the patch-up code above the wait (it does not know that the loads write LDS)
+    auto landed = [&]() {
+        __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0)
+        asm volatile("" ::: "memory");
+    };
+
     // one iteration = one chunk of KT = 32 inputs = two LDS-direct sub-chunks (buffers 0 and 1)
-    if (n_begin < n_end) issue(n_begin, 0);
+    if (n_begin < n_end) { fetch_masks(n_begin); issue(n_begin, 0); }
     for (int k0 = n_begin; k0 < n_end; k0 += KT) {
-        __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's loads of buffer 0 have landed
+        landed();
         repair(0);
+        apply_masks(0, k0);
         __syncthreads();                          // buffer 0 complete; everyone is done reading buffer 1
         issue(k0 + KD, 1);
         compute(0, k0);
-        __builtin_amdgcn_s_waitcnt(0x0f70);
+        landed();
         repair(1);
+        apply_masks(1, k0 + KD);
         __syncthreads();                          // buffer 1 complete; everyone is done reading buffer 0
-        if (k0 + KT < n_end) issue(k0 + KT, 0);
+        if (k0 + KT < n_end) { fetch_masks(k0 + KT); issue(k0 + KT, 0); }
         compute(1, k0 + KD);
         #pragma unroll
         for (int i = 0; i < TB; i++) {
             #pragma unroll
-            for (int j = 0; j < TM; j++) P::chunk_end(acc[i][j], a, 0, k0);
+            for (int j = 0; j < TM; j++) {
+                if constexpr (P::HAS_TSTATE) P::chunk_end_t(acc[i][j], tstate, a, i * TM + j, k0, (k0 - n_begin) / KT);
+                else P::chunk_end(acc[i][j], a, 0, k0);
+            }
         }
     }
 
@@ -178,22 +223,32 @@ __global__ void __launch_bounds__(256, 4) fwd_kernel_direct(FwdArgs a) {
         #pragma unroll
         for (int j = 0; j < TM; j++) {
             const int r = r0 + tb + 16 * i, m = m0 + tm + 16 * j;
-            P::store(acc[i][j], a, (size_t)(r * a.G + g) * a.COg + m, split);
+            const size_t o = (size_t)(r * a.G + g) * a.COg + m;
+            if constexpr (P::HAS_TSTATE) P::store_t(acc[i][j], tstate, a, o, split, i * TM + j, n_begin / KT);
+            else P::store(acc[i][j], a, o, split);
         }
     }
 }
 
-// true when the LDS-direct kernel with this tile can serve the call
+// true when the LDS-direct kernel with this tile can serve the call (the factored mask needs its keep-bit words)
 template <int TB, int TM>
 inline bool direct_ok(const FwdArgs& a) {
-    return a.fast_x && a.fast_w && a.mask_mode < 0 && !a.co_idx && !a.ci_idx && a.HW == 1 &&
+    const bool mask_ok = a.mask_mode < 0 || (a.mask_mode == SD_MASK_FACTORED && a.xmask && a.wmask && !a.x1);
+    return a.fast_x && a.fast_w && mask_ok && !a.co_idx && !a.ci_idx && a.HW == 1 &&
            a.CIg % KT == 0 && a.R % (16 * TB) == 0 && a.COg % (16 * TM) == 0;
 }
 
 template <class P, int TB, int TM>
 int launch_fwd_direct(const FwdArgs& a, hipStream_t stream) {
     dim3 grid(a.COg / (16 * TM), a.R / (16 * TB), a.G * a.nsplit);
-    hipLaunchKernelGGL((fwd_kernel_direct<P, TB, TM>), grid, dim3(256), 0, stream, a);
+    note_forward_kernel("fwd_kernel_direct", TB, TM);
+    if constexpr (P::NX == 1) {
+        if (a.mask_mode == SD_MASK_FACTORED) {
+            hipLaunchKernelGGL((fwd_kernel_direct<P, TB, TM, true>), grid, dim3(256), 0, stream, a);
+            return check_launch("fwd_kernel_direct");
+        }
+    }
+    hipLaunchKernelGGL((fwd_kernel_direct<P, TB, TM, false>), grid, dim3(256), 0, stream, a);
     return check_launch("fwd_kernel_direct");
 }
 

@@ -512,15 +512,18 @@ int launch_fwd(const FwdArgs& a, hipStream_t stream) {
     }
     dim3 grid((a.COg + 16 * TM - 1) / (16 * TM), (a.R + 16 * TB - 1) / (16 * TB), a.G * a.nsplit);
     if (a.fast_x && a.fast_w && (a.mask_mode != SD_MASK_FACTORED || a.xmask)) {
+        note_forward_kernel("fwd_kernel_pipe", TB, TM);
         hipLaunchKernelGGL((fwd_kernel_pipe<P, TB, TM>), grid, dim3(256), 0, stream, a);
         return check_launch("fwd_kernel");
     }
     if constexpr (P::LISTS && TB == 2) {
         if (a.mask_mode != SD_MASK_FACTORED) {
+            note_forward_kernel("fwd_kernel_lists", TB, TM);
             hipLaunchKernelGGL((fwd_kernel_lists<P, TB, TM>), grid, dim3(256), 0, stream, a);
             return check_launch("fwd_kernel");
         }
     }
+    note_forward_kernel("fwd_kernel", TB, TM);
     hipLaunchKernelGGL((fwd_kernel<P, TB, TM>), grid, dim3(256), 0, stream, a);
     return check_launch("fwd_kernel");
 }
@@ -539,6 +542,12 @@ struct PolicyBase {
     static constexpr bool LISTS = false;  // also built as fwd_kernel_lists (ops that accept kept-channel index lists)
     static constexpr bool DIRECT = false; // also built as fwd_kernel_direct (global -> LDS loads, exact dense tiles)
     template <class A> static __device__ __forceinline__ void chunk_end(A&, const FwdArgs&, int, int) {}
+    // Per-work-item state next to the per-output accumulators (fwd_kernel_direct only).  A policy with
+    // HAS_TSTATE defines TState<N> (N = outputs per work-item), tinit, chunk_end_t and store_t, which then replace
+    // chunk_end and store: idx = number of the output inside the register tile, kl = chunk number inside the
+    // slice, c0 = first chunk of the slice.
+    static constexpr bool HAS_TSTATE = false;
+    template <int N> struct TState {};
 };
 
 // l-inf forward without indices (core/cuda/inf_dist_cuda.cu:17-107)
@@ -606,6 +615,45 @@ struct LinfChunk : PolicyBase {
         A.cm = 0.f;
     }
     static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) { store_chunk_winner(a, o, A.best, A.cid); }
+};
+
+// LinfChunk for fwd_kernel_direct with the chunk numbers packed four to a register: the number of the winning chunk
+// inside the slice needs 8 bits (at most 254 chunks per slice; 255 = none yet), so 4 x 8 outputs cost 64 + 8
+// registers instead of 96 and fit four waves per SIMD without staging registers.
+struct LinfChunkPacked : PolicyBase {
+    static constexpr bool DIRECT = true;
+    static constexpr bool HAS_TSTATE = true;
+    static constexpr int MAX_CHUNKS = 254;      // per slice
+    struct Acc { float best, cm; };
+    template <int N> struct TState { uint32_t cids[(N + 3) / 4]; };
+    template <int N> static __device__ __forceinline__ void tinit(TState<N>& S) {
+        #pragma unroll
+        for (int k = 0; k < (N + 3) / 4; k++) S.cids[k] = 0xffffffffu;
+    }
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) { A.best = kEps; A.cm = 0.f; }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& x, const float4&,
+                                                 const float4& w, int, int) {
+        float v = A.cm;
+        v = fmaxf(fmaxf(v, fabsf(x.x - w.x)), fabsf(x.y - w.y));
+        v = fmaxf(fmaxf(v, fabsf(x.z - w.z)), fabsf(x.w - w.w));
+        A.cm = v;
+    }
+    template <int N>
+    static __device__ __forceinline__ void chunk_end_t(Acc& A, TState<N>& S, const FwdArgs&, int idx, int, int kl) {
+        const bool win = A.cm > A.best;          // strictly larger: the lowest chunk attaining the value survives
+        const int sh = 8 * (idx & 3);
+        const uint32_t f = S.cids[idx >> 2];
+        A.best = win ? A.cm : A.best;
+        S.cids[idx >> 2] = win ? ((f & ~(0xffu << sh)) | ((uint32_t)kl << sh)) : f;
+        A.cm = 0.f;
+    }
+    template <int N>
+    static __device__ __forceinline__ void store_t(Acc& A, TState<N>& S, const FwdArgs& a, size_t o, int, int idx, int c0) {
+        const uint32_t kl = (S.cids[idx >> 2] >> (8 * (idx & 3))) & 0xffu;
+        store_chunk_winner(a, o, A.best, kl == 0xffu ? -1 : c0 + (int)kl);
+    }
+    static __device__ __forceinline__ void chunk_end(Acc&, const FwdArgs&, int, int) {}
+    static __device__ __forceinline__ void store(Acc&, const FwdArgs&, size_t, int split = 0) {}
 };
 
 // the per-term masked neuron with the same chunk tracking

@@ -2,6 +2,7 @@
 #include "fwd_tile.h"
 #include "fwd_args.h"
 #include <mutex>
+#include <type_traits>
 
 using namespace sd;
 
@@ -34,6 +35,15 @@ static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st, void* mer
     const int TB = index_lists ? 2 : pick_tb(a, kTb42, 2, 16 * P::WIDE_TM);
     const bool gather = index_lists && !(a.fast_x && a.fast_w);      // served by the scalar-load kernel
     a.nsplit = TB == 2 ? pick_nsplit(a, 32, gather ? 128 : 16 * P::WIDE_TM, gather ? 1 : 8) : pick_nsplit(a, 16 * P::WIDE_TB, 16 * P::WIDE_TM);
+    // dense exact tiles of the l-inf policy: LDS-direct kernel with 4 x 8 outputs per work-item and the chunk numbers
+    // packed four to a register (same (value, chunk) results, so the same resolve pass follows)
+    bool packed_direct = false;
+    if constexpr (std::is_same<P, LinfChunk>::value) {
+        if (TB == 4 && direct_ok<4, 8>(a)) {
+            const int ns = pick_nsplit(a, 64, 128);
+            if ((a.CIg / KT + ns - 1) / ns <= LinfChunkPacked::MAX_CHUNKS) { packed_direct = true; a.nsplit = ns; }
+        }
+    }
     int rc;
     if (a.nsplit > 1) {
         // the merge buffer sits at the start of the workspace; a factored-mask call has already sized
@@ -47,7 +57,8 @@ static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st, void* mer
         if (!a.packed0) return SD_ERR_HIP;
         if ((rc = fill_zero(a.packed0, n * 2, st))) return rc;
     }
-    if (TB == 2) rc = gather ? launch_fwd<P, 2, 8>(a, st) : launch_fwd<P, 2, P::WIDE_TM>(a, st);
+    if (packed_direct) rc = launch_fwd_direct<LinfChunkPacked, 4, 8>(a, st);
+    else if (TB == 2) rc = gather ? launch_fwd<P, 2, 8>(a, st) : launch_fwd<P, 2, P::WIDE_TM>(a, st);
     else rc = launch_fwd<P, P::WIDE_TB, P::WIDE_TM>(a, st);
     if (rc) return rc;
     return launch_resolve(a, st);

@@ -24,6 +24,12 @@ int check_launch(const char* what) {
     return SD_OK;
 }
 
+static thread_local char g_fwd_kernel[64] = "";
+
+void note_forward_kernel(const char* kind, int tb, int tm) {
+    snprintf(g_fwd_kernel, sizeof(g_fwd_kernel), "%s<%d,%d>", kind, tb, tm);
+}
+
 int num_cus() {
     static int cached[64] = {0};
     int dev = 0;
@@ -96,6 +102,8 @@ extern "C" {
 int sd_version(void) { return 100; }
 
 const char* sd_last_error(void) { return sd::g_err; }
+
+const char* sd_last_forward_kernel(void) { return sd::g_fwd_kernel; }
 
 uint32_t sd_rng_word(uint32_t seed, uint32_t stream_id, uint32_t row, uint32_t col) {
     return sd::rng_word(sd::rng_row_key(seed, stream_id, row), col);
