@@ -230,11 +230,14 @@ __global__ void __launch_bounds__(256, 4) fwd_kernel_direct(FwdArgs a) {
     }
 }
 
-// true when the LDS-direct kernel with this tile can serve the call (the factored mask needs its keep-bit words)
-template <int TB, int TM>
+// true when the LDS-direct kernel with this tile can serve the call (the factored mask needs its keep-bit words and
+// a policy that is built with the mask patch)
+template <int TB, int TM, bool MASKABLE = true>
 inline bool direct_ok(const FwdArgs& a) {
-    const bool mask_ok = a.mask_mode < 0 || (a.mask_mode == SD_MASK_FACTORED && a.xmask && a.wmask && !a.x1);
-    return a.fast_x && a.fast_w && mask_ok && !a.co_idx && !a.ci_idx && a.HW == 1 &&
+    const bool mask_ok = a.mask_mode < 0 || (MASKABLE && a.mask_mode == SD_MASK_FACTORED && a.xmask && a.wmask && !a.x1);
+    // per-lane byte offsets are 32-bit and relative to the first row of the tile: 128 rows must stay below 4 GiB
+    const bool offsets_ok = 128ll * a.G * a.CIg * 4 < (1ll << 32) && 128ll * a.W_CIg * 4 < (1ll << 32);
+    return a.fast_x && a.fast_w && mask_ok && offsets_ok && !a.co_idx && !a.ci_idx && a.HW == 1 &&
            a.CIg % KT == 0 && a.R % (16 * TB) == 0 && a.COg % (16 * TM) == 0;
 }
 
@@ -242,7 +245,7 @@ template <class P, int TB, int TM>
 int launch_fwd_direct(const FwdArgs& a, hipStream_t stream) {
     dim3 grid(a.COg / (16 * TM), a.R / (16 * TB), a.G * a.nsplit);
     note_forward_kernel("fwd_kernel_direct", TB, TM);
-    if constexpr (P::NX == 1) {
+    if constexpr (P::NX == 1 && P::MASKABLE) {
         if (a.mask_mode == SD_MASK_FACTORED) {
             hipLaunchKernelGGL((fwd_kernel_direct<P, TB, TM, true>), grid, dim3(256), 0, stream, a);
             return check_launch("fwd_kernel_direct");

@@ -508,7 +508,7 @@ template <class P, int TB, int TM>
 int launch_fwd(const FwdArgs& a, hipStream_t stream) {
     // exact dense tiles of the policies that opt in go through the LDS-direct kernel
     if constexpr (P::DIRECT && TB % 4 == 0 && TM % 4 == 0) {
-        if (direct_ok<TB, TM>(a)) return launch_fwd_direct<P, TB, TM>(a, stream);
+        if (direct_ok<TB, TM, P::MASKABLE>(a)) return launch_fwd_direct<P, TB, TM>(a, stream);
     }
     dim3 grid((a.COg + 16 * TM - 1) / (16 * TM), (a.R + 16 * TB - 1) / (16 * TB), a.G * a.nsplit);
     if (a.fast_x && a.fast_w && (a.mask_mode != SD_MASK_FACTORED || a.xmask)) {
@@ -541,6 +541,7 @@ struct PolicyBase {
     static constexpr int WIDE_TB = 4, WIDE_TM = 8;   // register tile of the large-batch launch of position kernels
     static constexpr bool LISTS = false;  // also built as fwd_kernel_lists (ops that accept kept-channel index lists)
     static constexpr bool DIRECT = false; // also built as fwd_kernel_direct (global -> LDS loads, exact dense tiles)
+    static constexpr bool MASKABLE = false;  // fwd_kernel_direct is also built with the factored mask patched into LDS
     template <class A> static __device__ __forceinline__ void chunk_end(A&, const FwdArgs&, int, int) {}
     // Per-work-item state next to the per-output accumulators (fwd_kernel_direct only).  A policy with
     // HAS_TSTATE defines TState<N> (N = outputs per work-item), tinit, chunk_end_t and store_t, which then replace
@@ -554,6 +555,7 @@ struct PolicyBase {
 struct LinfNograd : PolicyBase {
     static constexpr bool LISTS = true;
     static constexpr bool DIRECT = true;
+    static constexpr bool MASKABLE = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int MIN_WAVES = 3;
     static constexpr int UNROLL4 = 1;
@@ -622,6 +624,7 @@ struct LinfChunk : PolicyBase {
 // registers instead of 96 and fit four waves per SIMD without staging registers.
 struct LinfChunkPacked : PolicyBase {
     static constexpr bool DIRECT = true;
+    static constexpr bool MASKABLE = true;
     static constexpr bool HAS_TSTATE = true;
     static constexpr int MAX_CHUNKS = 254;      // per slice
     struct Acc { float best, cm; };

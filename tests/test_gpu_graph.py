@@ -129,3 +129,55 @@ def test_calls_on_two_streams_overlap_safely(oracle):
     for got, want in ((oa, ra), (ob, rb)):
         assert torch.equal(got["y"], want["y"]) and torch.equal(got["pos"], want["pos"])
         _close(got["ys"], want["ys"], "sort neuron"); _close(got["yp"], want["yp"], "l-p")
+
+
+def test_graph_replays_of_the_lds_direct_kernels():
+    """The same protocol at a shape that takes the LDS-direct kernels (exact 64 x 128 tiles, split reduction range):
+    l-inf with and without positions, the factored-mask neuron, the interval forward and the l-p forward, captured once
+    and replayed on new contents; all of them bit for bit against eager calls except the l-p sums (rel 1e-5)."""
+    from sortnet_amd import ext, _lib
+    dev = _dev()
+    B, CI, CO = 256, 2048, 2048
+    g = torch.Generator().manual_seed(15)
+    x = torch.empty(B, CI, 1, device=dev); w = torch.empty(CO, CI, device=dev)
+
+    def outputs():
+        f = lambda: torch.empty(B, CO, 1, device=dev)
+        i = lambda: torch.empty(B, CO, 1, device=dev, dtype=torch.int32)
+        return dict(y=f(), pos=i(), yn=f(), ym=f(), pm=i(), yl=f(), yu=f(), yp=f())
+
+    def run(o):
+        names = []
+        ext.inf_dist_forward(x, w, o["y"], o["pos"], 1); names.append(_lib.last_forward_kernel())
+        ext.inf_dist_forward_nograd(x, w, o["yn"], 1); names.append(_lib.last_forward_kernel())
+        ext.masked_inf_dist_forward(x, w, o["ym"], o["pm"], 1, 0.3, 21, ext.MASK_FACTORED); names.append(_lib.last_forward_kernel())
+        ext.bound_inf_dist_forward_nograd(x - 0.05, x + 0.05, w, o["yl"], o["yu"], 1); names.append(_lib.last_forward_kernel())
+        ext.norm_dist_forward(x, w, o["yp"], 1, 8.0); names.append(_lib.last_forward_kernel())
+        return names
+
+    def new_inputs(scale):
+        x.copy_(torch.rand(B, CI, 1, generator=g) * scale); w.copy_(torch.randn(CO, CI, generator=g) * 0.2)
+
+    new_inputs(1.0)
+    eager, captured = outputs(), outputs()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        names = run(captured)       # warm-up on the capture stream sizes its workspace
+    assert all(n == "fwd_kernel_direct<4,8>" for n in names), names
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run(captured)
+    for replay, scale in enumerate((1.0, 0.5, 2.0)):
+        new_inputs(scale)
+        run(eager)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name in eager:
+            if name == "yp":
+                _close(captured[name], eager[name], "%s, replay %d" % (name, replay))
+            else:
+                assert torch.equal(eager[name], captured[name]), "%s, replay %d" % (name, replay)
