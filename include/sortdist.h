@@ -59,6 +59,13 @@ const char* sd_last_error(void);
  * "fwd_kernel_direct<4,8>" (global -> LDS loads), "fwd_kernel_pipe<4,8>" (register-staged), "fwd_kernel_lists<2,8>"
  * (gather loads), "fwd_kernel<2,4>" (general): for tests and benchmarks that must know which path they measured. */
 const char* sd_last_forward_kernel(void);
+/* Dense single-group l-p calls at general p queue two kernels for the same result: one that evaluates every term
+ * and one that works from a table of the inputs that can hold a term that counts (per output-channel tile and batch
+ * row).  The share of marked table entries, counted on the device, decides which of the two runs: the table kernel
+ * when it is at most `density` (0 never builds the table, 1 always uses it, negative = the built-in limits, which
+ * are the default: 0.05 to 0.2 depending on the call).  Process-wide; no reference counterpart
+ * (core/cuda/norm_dist_cuda.cu evaluates every term). */
+int sd_set_lp_candidate_density(float density);
 
 /* ---- l-inf distance: struct inf_dist, core/cuda/norm_dist.h:20-31 ---- */
 

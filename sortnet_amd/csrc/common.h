@@ -57,7 +57,16 @@ struct FwdArgs {
     float skip_thr;       // l-p, large p: ratios to the running scale below this cannot change the fp32 result (0 = unused)
     uint32_t seed, t8, t16;
     int mask_mode;        // -1 none, SD_MASK_TERM, SD_MASK_FACTORED
+    // device-side choice between two kernels queued for the same result (gated policies only): the kernel runs
+    // when gate is null or (*gate > gate_limit) == gate_above, and returns at once otherwise
+    const unsigned long long* gate;
+    unsigned long long gate_limit;
+    int gate_above;
 };
+
+__device__ __forceinline__ bool gate_closed(const unsigned long long* gate, unsigned long long limit, int above) {
+    return gate != nullptr && (*gate > limit) != (above != 0);
+}
 
 // ---- error reporting ---------------------------------------------------------------------------
 void set_error(const char* fmt, ...);

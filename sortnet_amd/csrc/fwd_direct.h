@@ -48,6 +48,7 @@ __device__ __forceinline__ int swz(int c, int r) { return c ^ ((r >> 2) & 3); }
 
 template <class P, int TB, int TM, bool MASKED>
 __global__ void __launch_bounds__(256, 4) fwd_kernel_direct(FwdArgs a) {
+    if constexpr (P::GATED) { if (gate_closed(a.gate, a.gate_limit, a.gate_above)) return; }
     constexpr int BB = 16 * TB, BM = 16 * TM, NX = P::NX;
     constexpr int XG = BB / 16, WG = BM / 16;          // 16-row groups of one x tile / of the w tile
     constexpr int NG = NX * XG + WG;                    // wave-wide loads per chunk

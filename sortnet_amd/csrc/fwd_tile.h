@@ -139,6 +139,7 @@ __device__ __forceinline__ void load_w_tile(float (*ws)[LDP], const FwdArgs& a,
 // -------------------------------------------------------------------------------------------
 template <class P, int TB, int TM>
 __global__ void __launch_bounds__(256, P::MIN_WAVES) fwd_kernel(FwdArgs a) {
+    if constexpr (P::GATED) { if (gate_closed(a.gate, a.gate_limit, a.gate_above)) return; }
     constexpr int BB = 16 * TB, BM = 16 * TM, NX = P::NX;
     __shared__ __attribute__((aligned(16))) float xs[NX][BB][LDP];
     __shared__ __attribute__((aligned(16))) float ws[BM][LDP];
@@ -228,6 +229,7 @@ constexpr int pipe_unroll() { return (TM <= 4 && P::UNROLL4_TM4) ? P::UNROLL4_TM
 
 template <class P, int TB, int TM>
 __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_pipe(FwdArgs a) {
+    if constexpr (P::GATED) { if (gate_closed(a.gate, a.gate_limit, a.gate_above)) return; }
     constexpr int BB = 16 * TB, BM = 16 * TM, NX = P::NX;
     constexpr int NXV = (BB * 8 + 255) / 256, NWV = (BM * 8 + 255) / 256;
     __shared__ __attribute__((aligned(16))) float xs[NX][BB][LDP];
@@ -390,6 +392,7 @@ __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_pip
 // -------------------------------------------------------------------------------------------
 template <class P, int TB, int TM>
 __global__ void __launch_bounds__(256, (pipe_waves<P, TB, TM>())) fwd_kernel_lists(FwdArgs a) {
+    if constexpr (P::GATED) { if (gate_closed(a.gate, a.gate_limit, a.gate_above)) return; }
     static_assert(P::NX == 1 && KT == 32, "one input tile, 32 columns per chunk");
     constexpr int BB = 16 * TB, BM = 16 * TM;
     constexpr int NXR = BB / 8, NWR = BM / 8;
@@ -542,6 +545,7 @@ struct PolicyBase {
     static constexpr bool LISTS = false;  // also built as fwd_kernel_lists (ops that accept kept-channel index lists)
     static constexpr bool DIRECT = false; // also built as fwd_kernel_direct (global -> LDS loads, exact dense tiles)
     static constexpr bool MASKABLE = false;  // fwd_kernel_direct is also built with the factored mask patched into LDS
+    static constexpr bool GATED = false;  // the kernels honour FwdArgs::gate
     template <class A> static __device__ __forceinline__ void chunk_end(A&, const FwdArgs&, int, int) {}
     // Per-work-item state next to the per-output accumulators (fwd_kernel_direct only).  A policy with
     // HAS_TSTATE defines TState<N> (N = outputs per work-item), tinit, chunk_end_t and store_t, which then replace
@@ -1055,6 +1059,7 @@ template <int IP, bool FOLD = (IP < 0)>
 struct LpWithMax : PolicyBase {
     static constexpr bool LISTS = true;
     static constexpr bool DIRECT = true;
+    static constexpr bool GATED = true;
     static constexpr int PIPE_WAVES = 3;
     static constexpr int MIN_WAVES = 3;
     // rinv = 1 / maximum; FOLD (general p) keeps c = p log2(1 / maximum) instead, so that a term is

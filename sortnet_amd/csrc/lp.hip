@@ -2,6 +2,7 @@
 #include <cstdlib>
 #include "fwd_tile.h"
 #include "fwd_args.h"
+#include "lp_rows.h"
 
 namespace sd {
 
@@ -12,6 +13,25 @@ namespace sd {
 constexpr float kLpSkipFrom = 0.5f, kLpSkipFromOnline = 0.75f;
 // backward: the dense both-gradient kernel (p of about 65) and the general kernel (p of about 80)
 constexpr float kLpSkipFromFused = 0.68f, kLpSkipFromGeneral = 0.73f;
+
+// largest share of marked (tile, row, input) triples at which the candidate-table kernels run instead of the
+// kernels that evaluate every term (sd_set_lp_candidate_density); negative: the built-in limits below
+static float g_rows_density = -1.f;
+// Measured at B = 512, M = N = 5120 on three kinds of data (normal or uniform inputs against small weights,
+// normal inputs against weights of the same size), in ms against the marked share d:
+//   forward   table kernel 0.54 + 3.6 d   every term 2.8, with wave-level significance tests 1.3 .. 3.6
+//   backward  both gradients 0.13 + 6 d   every term 3.5, with tests 2.8 .. 4.8
+//             grad_input only 0.09 + 5 d  every term 3.15, with tests 1.45 .. 4.3
+// The limits sit where the table kernel meets the fastest case of the kernel it replaces.
+constexpr float kRowsCapForward = 0.55f, kRowsCapForwardSkip = 0.2f;
+constexpr float kRowsCapBackward = 0.5f, kRowsCapBackwardSkip = 0.4f;
+constexpr float kRowsCapBackwardInput = 0.55f, kRowsCapBackwardInputSkip = 0.25f;
+// below this threshold (p of about 12 forward, 20 backward) most inputs are marked on all three
+constexpr float kRowsFromThr = 0.15f;
+static inline float rows_cap(float builtin, float thr) {
+    if (g_rows_density >= 0.f) return g_rows_density;
+    return thr >= kRowsFromThr ? builtin : 0.f;
+}
 
 static inline int int_power(float p) {
     if (p == (float)(int)p && p >= 0.f && p <= 8.f) return (int)p;
@@ -49,9 +69,10 @@ static int launch_lp(int ip, const FwdArgs& a, hipStream_t st) {
 __global__ void __launch_bounds__(256) lp_finalize_kernel(const float* __restrict__ part0, const float* __restrict__ part1,
                                                           const float* __restrict__ scale,
                                                           int nsplit, size_t total, float p, float inv_p,
-                                                          float* __restrict__ y) {
+                                                          float* __restrict__ y, const unsigned long long* gate,
+                                                          unsigned long long gate_limit, int gate_above) {
     size_t o = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (o >= total) return;
+    if (o >= total || gate_closed(gate, gate_limit, gate_above)) return;
     if (part1 == nullptr) {
         float s = 0.f;
         for (int k = 0; k < nsplit; k++) s += part0[(size_t)k * total + o];
@@ -84,7 +105,8 @@ static int lp_split_setup(FwdArgs& a, int BB, int BM, bool online, hipStream_t s
 static int lp_split_finish(const FwdArgs& a, hipStream_t st) {
     if (a.nsplit <= 1) return SD_OK;
     hipLaunchKernelGGL(lp_finalize_kernel, dim3((unsigned)((a.part_stride + 255) / 256)), dim3(256), 0, st,
-                       a.part0, a.part1, a.part1 ? nullptr : a.aux, a.nsplit, a.part_stride, a.p, a.inv_p, a.y0);
+                       a.part0, a.part1, a.part1 ? nullptr : a.aux, a.nsplit, a.part_stride, a.p, a.inv_p, a.y0,
+                       a.gate, a.gate_limit, a.gate_above);
     return check_launch("lp_finalize_kernel");
 }
 
@@ -93,10 +115,20 @@ static int lp_split_finish(const FwdArgs& a, hipStream_t st) {
 // every LDS chunk.  Workspace: the maxima, then the partial sums of the split reduction.
 static int lp_forward_max_first(FwdArgs& a, bool small, hipStream_t st) {
     const size_t total = (size_t)a.R * a.G * a.COg;
+    // dense single-group layers: a sum pass that works from per-row candidate tables is queued in front of the
+    // one that evaluates every term, and a count taken on the device decides which of the two runs
+    const float thr_rows = powf(1e-6f / (float)a.CIg, 1.f / a.p);
+    const float cap = rows_cap(a.skip_thr > 0.f ? kRowsCapForwardSkip : kRowsCapForward, thr_rows);
+    const bool rows = cap > 0.f && a.G == 1 && a.HW == 1 && !a.ci_idx && !a.co_idx && a.W_CIg == a.CIg &&
+                      a.CIg % kRowsChunk == 0 && a.R < (1 << 22) && thr_rows > 0.f && thr_rows < 1.f;
     FwdArgs m = a;
     m.nsplit = pick_nsplit(m, small ? 32 : 64, 128);
     a.nsplit = m.nsplit;
-    float* base = static_cast<float*>(workspace(total * (size_t)(1 + (a.nsplit > 1 ? a.nsplit : 0)) * sizeof(float), st));
+    const int ns_rows = rows ? lp_rows_forward_nsplit(a.R, a.COg, a.CIg) : 1;
+    const int ns_max = ns_rows > a.nsplit ? ns_rows : a.nsplit;
+    const size_t head = total * (size_t)(1 + (ns_max > 1 ? ns_max : 0)) * sizeof(float);
+    const size_t head_al = (head + 255) / 256 * 256;
+    float* base = static_cast<float*>(workspace(head_al + (rows ? lp_rows_workspace(a.R, a.COg, a.CIg) : 0), st));
     if (!base) return SD_ERR_HIP;
     m.y0 = base;
     int rc;
@@ -105,8 +137,19 @@ static int lp_forward_max_first(FwdArgs& a, bool small, hipStream_t st) {
     if (rc) return rc;
     a.aux = base;
     a.part_stride = total;
-    a.part0 = a.nsplit > 1 ? base + total : nullptr;
     a.part1 = nullptr;
+    if (rows) {
+        FwdArgs r = a;
+        r.nsplit = ns_rows;
+        r.part0 = ns_rows > 1 ? base + total : nullptr;
+        rc = lp_rows_forward(a.x0, a.w, base, a.R, a.COg, a.CIg, a.p, thr_rows, ns_rows, a.y0, r.part0,
+                             reinterpret_cast<char*>(base) + head_al, cap, &r.gate, &r.gate_limit, st);
+        if (rc) return rc;
+        r.gate_above = 0;
+        if ((rc = lp_split_finish(r, st))) return rc;
+        a.gate = r.gate; a.gate_limit = r.gate_limit; a.gate_above = 1;
+    }
+    a.part0 = a.nsplit > 1 ? base + total : nullptr;
     if (a.skip_thr > 0.f) rc = small ? launch_fwd<LpWithMaxSkip, 2, 8>(a, st) : launch_fwd<LpWithMaxSkip, 4, 8>(a, st);
     else rc = small ? launch_fwd<LpWithMax<-1>, 2, 8>(a, st) : launch_fwd<LpWithMax<-1>, 4, 8>(a, st);
     if (rc) return rc;
@@ -137,6 +180,11 @@ struct LpBwdArgs {
     int B, R, HW, G, COg, CIg, W_COg, W_CIg;
     float pm1;   // p - 1
     float skip_thr;  // general p: |d| / y below this cannot change the sums (0 = every term is evaluated)
+    const unsigned long long* gate;   // see FwdArgs::gate
+    unsigned long long gate_limit;
+    int gate_above;
+    const float* ry;                  // 1 / y when the caller already holds it, else null
+    bool gx_is_zero;                  // grad_input was zero-filled by the caller
     int zsplit;  // slices of the output-channel range (grad_input then merges with atomic adds)
 };
 
@@ -231,6 +279,7 @@ __device__ __forceinline__ void lp_bwd_chunk(const LpBwdArgs& a, const float2 (&
 template <int IP, bool WGRAD, bool SKIP = false>
 __global__ void __launch_bounds__(256, (SKIP ? 4 : 1)) lp_bwd_kernel(LpBwdArgs a) {
     __shared__ float2 gr[2][MC][RB];   // (g, 1/y) of output channel m0+k, row r0+i; two chunks
+    if (gate_closed(a.gate, a.gate_limit, a.gate_above)) return;
 
     const int tid = threadIdx.x;
     const int g = blockIdx.z % a.G, slice = blockIdx.z / a.G;
@@ -351,13 +400,16 @@ template <int IP, bool SKIP>
 __global__ void __launch_bounds__(256, 3) lp_bwd_fused_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                               const float* __restrict__ g, const float* __restrict__ ry,
                                                               int B, int M, int N, int mr, float pm1, float skip_thr,
-                                                              float* __restrict__ gx, float* __restrict__ gw) {
+                                                              float* __restrict__ gx, float* __restrict__ gw,
+                                                              const unsigned long long* gate, unsigned long long gate_limit,
+                                                              int gate_above) {
     constexpr int TI = 4, TJ = 2;                 // batch rows / weight rows per work-item
     constexpr int PSTRIDE = FN * 16 * TJ + 16;    // plane of one batch-row group, skewed by 16 banks
     constexpr int GSTRIDE = FMR + 32;
     static_assert(FN * 16 * TJ == 256, "one accumulator per work-item and weight tile");
     __shared__ float gwl[FN * GSTRIDE];
     __shared__ float part[16 * PSTRIDE];
+    if (gate_closed(gate, gate_limit, gate_above)) return;
     const int tid = threadIdx.x, tm = tid & 15, tb = tid >> 4;
     const int n0 = blockIdx.x * FN;
     const int m_lo = blockIdx.y * mr, m_hi = m_lo + mr < M ? m_lo + mr : M;
@@ -485,17 +537,22 @@ __global__ void __launch_bounds__(256, 3) lp_bwd_fused_kernel(const float* __res
 static int launch_lp_bwd_fused(int ip, const LpBwdArgs& a, hipStream_t st) {
     const int B = a.R, M = a.COg, N = a.CIg;
     const size_t n = (size_t)B * M;
-    float* ry = static_cast<float*>(workspace(n * sizeof(float), st));
-    if (!ry) return SD_ERR_HIP;
-    hipLaunchKernelGGL(lp_recip_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a.y, n, ry);
-    int rc = check_launch("lp_recip_kernel");
-    if (rc) return rc;
-    if ((rc = fill_zero(a.gx, (size_t)B * N, st))) return rc;
+    int rc;
+    const float* ry = a.ry;   // with it comes a zero-filled grad_input
+    if (!ry) {
+        float* buf = static_cast<float*>(workspace(n * sizeof(float), st));
+        if (!buf) return SD_ERR_HIP;
+        hipLaunchKernelGGL(lp_recip_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a.y, n, buf);
+        if ((rc = check_launch("lp_recip_kernel"))) return rc;
+        if ((rc = fill_zero(a.gx, (size_t)B * N, st))) return rc;
+        ry = buf;
+    }
     const int ranges = (M + FMR - 1) / FMR;
     const int mr = (((M + ranges - 1) / ranges) + 31) / 32 * 32;   // equal ranges, whole weight tiles
     dim3 grid(N / FN, (M + mr - 1) / mr);
     (void)ip;
-    hipLaunchKernelGGL((lp_bwd_fused_kernel<-1, true>), grid, dim3(256), 0, st, a.x, a.w, a.gy, ry, B, M, N, mr, a.pm1, a.skip_thr, a.gx, a.gw);
+    hipLaunchKernelGGL((lp_bwd_fused_kernel<-1, true>), grid, dim3(256), 0, st, a.x, a.w, a.gy, ry, B, M, N, mr, a.pm1,
+                       a.skip_thr, a.gx, a.gw, a.gate, a.gate_limit, a.gate_above);
     return check_launch("lp_bwd_fused_kernel");
 }
 
@@ -516,7 +573,7 @@ static int launch_lp_bwd(int ip, const LpBwdArgs& a_in, hipStream_t st) {
         if (eff > best * 1.03) { best = eff; a.zsplit = z; }
     }
     int rc;
-    if (a.zsplit > 1 && (rc = fill_zero(a.gx, (size_t)a.R * a.G * a.CIg, st))) return rc;
+    if (a.zsplit > 1 && !a.gx_is_zero && (rc = fill_zero(a.gx, (size_t)a.R * a.G * a.CIg, st))) return rc;
     dim3 grid((a.CIg + 255) / 256, (a.R + RB - 1) / RB, a.G * a.zsplit);
 #define SD_CASE(k) case k: hipLaunchKernelGGL((lp_bwd_kernel<k, WGRAD>), grid, dim3(256), 0, st, a); break;
     switch (ip) {
@@ -555,10 +612,31 @@ static int lp_backward(const char* who, const float* grad_output, const float* i
     // test only pays from a higher threshold; everything else goes through the general kernel
     const bool dense = G == 1 && HW == 1 && !ci_idx && !co_idx && f.CIg % FN == 0 && aligned16(input) &&
                        aligned16(weight) && aligned16(grad_weight);
+    // dense layers at general p: a kernel that works from per-row candidate tables is queued in front of the one
+    // that evaluates every term, and a count taken on the device decides which of the two runs
+    const float thr_rows = (ip < 0 && a.pm1 > 1.f) ? powf(1e-16f, 1.f / a.pm1) : 0.f;
+    bool zero_gx = false;
+    // which kernel evaluates every term, and whether it runs its own wave-level tests
+    const bool fused = dense && grad_weight && a.skip_thr >= kLpSkipFromFused;
+    const bool tests = fused || a.skip_thr >= kLpSkipFromGeneral;
+    const float cap = rows_cap(grad_weight ? (tests ? kRowsCapBackwardSkip : kRowsCapBackward)
+                                           : (tests ? kRowsCapBackwardInputSkip : kRowsCapBackwardInput), thr_rows);
+    if (cap > 0.f && dense && thr_rows > 0.f && thr_rows < 1.f && f.CIg % kRowsChunk == 0 && f.W_CIg == f.CIg &&
+        B < (1 << 22)) {
+        void* ws = workspace(lp_rows_workspace(f.R, f.COg, f.CIg) + (size_t)f.R * f.COg * sizeof(float), st);
+        if (!ws) return SD_ERR_HIP;
+        // the general kernel adds to a zero-filled grad_weight, which the table kernel must not find cleared after it ran
+        if (grad_weight && !fused && (rc = fill_zero(grad_weight, (size_t)G * f.W_COg * f.W_CIg, st))) return rc;
+        if ((rc = lp_rows_backward(grad_output, input, weight, output, f.R, f.COg, f.CIg, a.pm1, thr_rows, grad_input,
+                                   grad_weight, ws, cap, &a.ry, &a.gate, &a.gate_limit, st))) return rc;
+        a.gate_above = 1;
+        zero_gx = true;
+    }
     if (dense && grad_weight && a.skip_thr >= kLpSkipFromFused) return launch_lp_bwd_fused(ip, a, st);
     if (a.skip_thr < kLpSkipFromGeneral) a.skip_thr = 0.f;
+    a.gx_is_zero = zero_gx;
     if (grad_weight) {
-        if ((rc = fill_zero(grad_weight, (size_t)G * f.W_COg * f.W_CIg, st))) return rc;
+        if (!zero_gx && (rc = fill_zero(grad_weight, (size_t)G * f.W_COg * f.W_CIg, st))) return rc;
         return launch_lp_bwd<true>(ip, a, st);
     }
     return launch_lp_bwd<false>(ip, a, st);
@@ -567,6 +645,12 @@ static int lp_backward(const char* who, const float* grad_output, const float* i
 }  // namespace sd
 
 using namespace sd;
+
+extern "C" int sd_set_lp_candidate_density(float density) {
+    SD_REQUIRE(density <= 1.f, "set_lp_candidate_density: %g is above 1", (double)density);
+    g_rows_density = density;
+    return SD_OK;
+}
 
 extern "C" int sd_norm_dist_forward(const float* input, const float* weight,
                                     int B, int CO, int CI, int G, int HW, float* output, float p,
