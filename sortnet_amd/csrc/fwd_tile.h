@@ -579,6 +579,12 @@ struct LinfNograd : PolicyBase {
     }
 };
 
+// the same kernel as one of two queued for a result, see FwdArgs::gate (first step of the general-p l-p forward)
+struct LinfNogradGated : LinfNograd {
+    static constexpr bool MASKABLE = false;
+    static constexpr bool GATED = true;
+};
+
 // l-inf forward with arg-max index and sign (core/cuda/inf_dist_cuda.cu:110-212), without paying for
 // index bookkeeping on every term: inside a chunk of KT inputs only the maximum
 // is kept (one subtract per term, one 3-input max per two terms); at the end of the chunk the

@@ -19,13 +19,14 @@ constexpr float kLpSkipFromFused = 0.68f, kLpSkipFromGeneral = 0.73f;
 static float g_rows_density = -1.f;
 // Measured at B = 512, M = N = 5120 on three kinds of data (normal or uniform inputs against small weights,
 // normal inputs against weights of the same size), in ms against the marked share d:
-//   forward   table kernel 0.54 + 3.6 d   every term 2.8, with wave-level significance tests 1.3 .. 3.6
+//   forward   table kernel 0.2 + 3.6 d    every term 2.8, with wave-level significance tests 1.3 .. 3.6
 //   backward  both gradients 0.13 + 6 d   every term 3.5, with tests 2.8 .. 4.8
 //             grad_input only 0.09 + 5 d  every term 3.15, with tests 1.45 .. 4.3
-// The limits sit where the table kernel meets the fastest case of the kernel it replaces.
-constexpr float kRowsCapForward = 0.55f, kRowsCapForwardSkip = 0.2f;
+// The limits sit near where the table kernel meets the fastest case of the kernel it replaces: a little above it
+// where that kernel's slow cases are far slower than its fast ones.
+constexpr float kRowsCapForward = 0.55f, kRowsCapForwardSkip = 0.3f;
 constexpr float kRowsCapBackward = 0.5f, kRowsCapBackwardSkip = 0.4f;
-constexpr float kRowsCapBackwardInput = 0.55f, kRowsCapBackwardInputSkip = 0.25f;
+constexpr float kRowsCapBackwardInput = 0.55f, kRowsCapBackwardInputSkip = 0.3f;
 // below this threshold (p of about 12 forward, 20 backward) most inputs are marked on all three
 constexpr float kRowsFromThr = 0.15f;
 static inline float rows_cap(float builtin, float thr) {
@@ -115,8 +116,8 @@ static int lp_split_finish(const FwdArgs& a, hipStream_t st) {
 // every LDS chunk.  Workspace: the maxima, then the partial sums of the split reduction.
 static int lp_forward_max_first(FwdArgs& a, bool small, hipStream_t st) {
     const size_t total = (size_t)a.R * a.G * a.COg;
-    // dense single-group layers: a sum pass that works from per-row candidate tables is queued in front of the
-    // one that evaluates every term, and a count taken on the device decides which of the two runs
+    // dense single-group layers: a kernel that works from per-row candidate tables and finds the maxima as it goes
+    // is queued in front of the two steps below, and a count taken on the device decides which of the two runs
     const float thr_rows = powf(1e-6f / (float)a.CIg, 1.f / a.p);
     const float cap = rows_cap(a.skip_thr > 0.f ? kRowsCapForwardSkip : kRowsCapForward, thr_rows);
     const bool rows = cap > 0.f && a.G == 1 && a.HW == 1 && !a.ci_idx && !a.co_idx && a.W_CIg == a.CIg &&
@@ -125,31 +126,36 @@ static int lp_forward_max_first(FwdArgs& a, bool small, hipStream_t st) {
     m.nsplit = pick_nsplit(m, small ? 32 : 64, 128);
     a.nsplit = m.nsplit;
     const int ns_rows = rows ? lp_rows_forward_nsplit(a.R, a.COg, a.CIg) : 1;
-    const int ns_max = ns_rows > a.nsplit ? ns_rows : a.nsplit;
-    const size_t head = total * (size_t)(1 + (ns_max > 1 ? ns_max : 0)) * sizeof(float);
+    // maxima, then the slice results of whichever sum kernel runs (the table kernel leaves two values per slice)
+    const int slots = a.nsplit > 1 ? a.nsplit : 0, slots_rows = ns_rows > 1 ? 2 * ns_rows : 0;
+    const size_t head = total * (size_t)(1 + (slots > slots_rows ? slots : slots_rows)) * sizeof(float);
     const size_t head_al = (head + 255) / 256 * 256;
     float* base = static_cast<float*>(workspace(head_al + (rows ? lp_rows_workspace(a.R, a.COg, a.CIg) : 0), st));
     if (!base) return SD_ERR_HIP;
-    m.y0 = base;
     int rc;
-    if (m.nsplit > 1 && (rc = fill_zero(base, total, st))) return rc;
-    rc = small ? launch_fwd<LinfNograd, 2, 8>(m, st) : launch_fwd<LinfNograd, 4, 8>(m, st);
-    if (rc) return rc;
-    a.aux = base;
-    a.part_stride = total;
-    a.part1 = nullptr;
     if (rows) {
         FwdArgs r = a;
         r.nsplit = ns_rows;
+        r.part_stride = total;
         r.part0 = ns_rows > 1 ? base + total : nullptr;
-        rc = lp_rows_forward(a.x0, a.w, base, a.R, a.COg, a.CIg, a.p, thr_rows, ns_rows, a.y0, r.part0,
+        r.part1 = ns_rows > 1 ? base + total * (size_t)(1 + ns_rows) : nullptr;
+        rc = lp_rows_forward(a.x0, a.w, nullptr, a.R, a.COg, a.CIg, a.p, thr_rows, ns_rows, a.y0, r.part0,
                              reinterpret_cast<char*>(base) + head_al, cap, &r.gate, &r.gate_limit, st);
         if (rc) return rc;
         r.gate_above = 0;
         if ((rc = lp_split_finish(r, st))) return rc;
         a.gate = r.gate; a.gate_limit = r.gate_limit; a.gate_above = 1;
+        m.gate = r.gate; m.gate_limit = r.gate_limit; m.gate_above = 1;
     }
+    m.y0 = base;
+    if (m.nsplit > 1 && (rc = fill_zero(base, total, st))) return rc;
+    if (rows) rc = small ? launch_fwd<LinfNogradGated, 2, 8>(m, st) : launch_fwd<LinfNogradGated, 4, 8>(m, st);
+    else rc = small ? launch_fwd<LinfNograd, 2, 8>(m, st) : launch_fwd<LinfNograd, 4, 8>(m, st);
+    if (rc) return rc;
+    a.aux = base;
+    a.part_stride = total;
     a.part0 = a.nsplit > 1 ? base + total : nullptr;
+    a.part1 = nullptr;
     if (a.skip_thr > 0.f) rc = small ? launch_fwd<LpWithMaxSkip, 2, 8>(a, st) : launch_fwd<LpWithMaxSkip, 4, 8>(a, st);
     else rc = small ? launch_fwd<LpWithMax<-1>, 2, 8>(a, st) : launch_fwd<LpWithMax<-1>, 4, 8>(a, st);
     if (rc) return rc;

@@ -25,7 +25,9 @@ size_t lp_rows_workspace(int B, int CO, int CI);
 int lp_rows_forward_nsplit(int B, int CO, int CI);
 
 // sums of (|x - w| / maxv)^p relative to the given maxima.  nsplit == 1: y = maxv * sum^(1/p); otherwise the
-// slice sums go to part[slice][B * CO] for the caller to merge.  ws: lp_rows_workspace bytes.
+// slice sums go to part[slice][B * CO] for the caller to merge.  maxv == nullptr: the kernel finds the maxima itself
+// as it goes (the table then comes from a lower bound of them), and the slices leave (sum, maximum) pairs in
+// part[slice] and part[nsplit + slice].  ws: lp_rows_workspace bytes.
 int lp_rows_forward(const float* x, const float* w, const float* maxv, int B, int CO, int CI, float p, float thr,
                     int nsplit, float* y, float* part, void* ws, float density,
                     const unsigned long long** gate, unsigned long long* gate_limit, hipStream_t st);

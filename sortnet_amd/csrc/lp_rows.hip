@@ -79,6 +79,20 @@ __global__ void __launch_bounds__(256) tile_rowmin_kernel(const float* __restric
     if (lane == 0) ymin[(size_t)t * Bp + b] = r;
 }
 
+// one wavefront per (row, tile): a lower bound of the largest |x[b,n] - w[m,n]| of every output channel m of the
+// tile, max_n (|x[b,n]| - max_m |w[m,n]|), at least the 1e-10 floor of a distance
+__global__ void __launch_bounds__(256) tile_rowlow_kernel(const float* __restrict__ x, const float* __restrict__ wabs,
+                                                          int B, int N, int T, int Bp, float* __restrict__ low) {
+    const int wave = (int)((blockIdx.x * 256u + threadIdx.x) >> 6), lane = threadIdx.x & 63;
+    if (wave >= B * T) return;
+    const int b = wave / T, t = wave - b * T;
+    float r = kEps;
+    for (int n = lane; n < N; n += 64) r = fmaxf(r, fabsf(x[(size_t)b * N + n]) - wabs[(size_t)t * N + n]);
+    #pragma unroll
+    for (int o = 32; o; o >>= 1) r = fmaxf(r, __shfl_xor(r, o));
+    if (lane == 0) low[(size_t)t * Bp + b] = r;
+}
+
 // bit (t, b, n): some output channel m of tile t may have |x[b,n] - w[m,n]| > thr * scale[b,m].  A workgroup takes
 // 64 rows x 32 inputs (one table word per row and tile): |x| goes through LDS so that a work-item can own a row
 // and the words of 64 rows leave as one coalesced store; wavefront v handles the tiles v, v + 4, ...  Every
@@ -135,7 +149,8 @@ int build_tables(const Carve& c, const float* x, const float* w, const float* sc
     int rc = check_launch("tile_wabs_kernel");
     if (rc) return rc;
     const unsigned waves = (unsigned)B * T;
-    if (recip) hipLaunchKernelGGL(tile_rowmin_kernel<true>, dim3((waves + 3) / 4), dim3(256), 0, st, scale, B, M, T, Bp, c.ymin, recip);
+    if (!scale) hipLaunchKernelGGL(tile_rowlow_kernel, dim3((waves + 3) / 4), dim3(256), 0, st, x, c.wabs, B, N, T, Bp, c.ymin);
+    else if (recip) hipLaunchKernelGGL(tile_rowmin_kernel<true>, dim3((waves + 3) / 4), dim3(256), 0, st, scale, B, M, T, Bp, c.ymin, recip);
     else hipLaunchKernelGGL(tile_rowmin_kernel<false>, dim3((waves + 3) / 4), dim3(256), 0, st, scale, B, M, T, Bp, c.ymin, recip);
     if ((rc = check_launch("tile_rowmin_kernel"))) return rc;
     const int NCH = N / kChunk;
@@ -153,7 +168,10 @@ int build_tables(const Carve& c, const float* x, const float* w, const float* sc
 // chunk the wavefront walks the union of its rows' marked inputs: the four weights of an input are read
 // once (one LDS word per lane and column), then every row that marks the input takes its four terms through the
 // significance test of the general kernel (wave-uniform: the group of four, then each term).
-template <int NW>   // wavefronts per workgroup: 4 or 16
+// ONLINE: no maxima are given; every sum is kept relative to the largest term met so far and rescaled when a
+// larger one comes (core/cuda/norm_dist_cuda.cu:36-160), with 1 / maximum in place of the given reciprocal scale.
+// The slice results are (sum, maximum) pairs in part[slice] and part[nsplit + slice].
+template <int NW, bool ONLINE>   // wavefronts per workgroup: 4 or 16
 __global__ void __launch_bounds__(64 * NW, (NW == 4 ? 2 : 1))
 lp_rows_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ maxv,
                    const uint32_t* __restrict__ bits, const unsigned long long* __restrict__ count,
@@ -179,10 +197,15 @@ lp_rows_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w, con
         #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int row = r0 + wave * TB + r, col = m0 + lane + 64 * j;
-            const float mv = (row < B && col < M) ? maxv[(size_t)row * M + col] : 1.f;
-            rinv[r][j] = 1.f / mv;
-            // the virtual term of size 1e-10 belongs to slice 0 only
-            acc[r][j] = split == 0 ? __builtin_amdgcn_exp2f(p * __builtin_amdgcn_logf(kEps * rinv[r][j])) : 0.f;
+            if (ONLINE) {
+                // the virtual term of size 1e-10 (1 relative to a maximum of 1e-10) belongs to slice 0 only
+                rinv[r][j] = 1.f / kEps;
+                acc[r][j] = split == 0 ? 1.f : 0.f;
+            } else {
+                const float mv = (row < B && col < M) ? maxv[(size_t)row * M + col] : 1.f;
+                rinv[r][j] = 1.f / mv;
+                acc[r][j] = split == 0 ? __builtin_amdgcn_exp2f(p * __builtin_amdgcn_logf(kEps * rinv[r][j])) : 0.f;
+            }
         }
     }
 
@@ -238,8 +261,20 @@ lp_rows_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w, con
                     const float xv = xt[buf][(wave * TB + r) * XS + n];
                     // every term of a marked input is evaluated: on data that the table suits, most of them count
                     #pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        acc[r][j] += __builtin_amdgcn_exp2f(p * __builtin_amdgcn_logf(fabsf(xv - wv[j]) * rinv[r][j]));
+                    for (int j = 0; j < 4; j++) {
+                        const float d = fabsf(xv - wv[j]);
+                        const float lg = p * __builtin_amdgcn_logf(d * rinv[r][j]);
+                        if (ONLINE) {
+                            // ratio above 1: a new maximum; the old sum shrinks by ratio^-p and the new term is 1.
+                            // The reciprocal need not be exact: the result is the sum's root divided by the same
+                            // reciprocal, whatever it is; only the rescaling sees its error, p times, and the root
+                            // takes that back.
+                            const bool up = lg > 0.f;
+                            const float e = __builtin_amdgcn_exp2f(up ? -lg : lg);
+                            acc[r][j] = up ? fmaf(acc[r][j], e, 1.f) : acc[r][j] + e;
+                            rinv[r][j] = up ? __builtin_amdgcn_rcpf(d) : rinv[r][j];
+                        } else acc[r][j] += __builtin_amdgcn_exp2f(lg);
+                    }
                 }
             }
         }
@@ -277,7 +312,13 @@ lp_rows_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w, con
             const int row = r0 + wave * TB + r, col = m0 + lane + 64 * j;
             if (row < B && col < M) {
                 const size_t o = (size_t)row * M + col;
-                if (nsplit > 1) part[(size_t)split * B * M + o] = acc[r][j];
+                if (ONLINE) {
+                    const float mx = 1.f / rinv[r][j];
+                    if (nsplit > 1) {
+                        part[(size_t)split * B * M + o] = acc[r][j];
+                        part[(size_t)(nsplit + split) * B * M + o] = mx;
+                    } else y[o] = powf(acc[r][j], inv_p) * mx;
+                } else if (nsplit > 1) part[(size_t)split * B * M + o] = acc[r][j];
                 else y[o] = powf(acc[r][j], inv_p) * maxv[o];
             }
         }
@@ -462,12 +503,13 @@ int lp_rows_forward(const float* x, const float* w, const float* maxv, int B, in
     *gate_limit = mark_limit(B, CO, CI, density);
     const int rows = fwd_rows(B), units = tiles_of(CO) * nsplit, RT = (B + rows - 1) / rows;
     dim3 grid((unsigned)(units * RT));
-    if (rows == 128)
-        hipLaunchKernelGGL((lp_rows_fwd_kernel<16>), grid, dim3(1024), 0, st, x, w, maxv, c.bits, c.count, *gate_limit, B,
-                           bpad_of(B), CO, CI, nsplit, p, 1.f / p, y, part);
-    else
-        hipLaunchKernelGGL((lp_rows_fwd_kernel<4>), grid, dim3(256), 0, st, x, w, maxv, c.bits, c.count, *gate_limit, B,
-                           bpad_of(B), CO, CI, nsplit, p, 1.f / p, y, part);
+    const int Bp = bpad_of(B);
+    const float ip = 1.f / p;
+#define SD_ROWS_FWD(NW, ON) hipLaunchKernelGGL((lp_rows_fwd_kernel<NW, ON>), grid, dim3(64 * NW), 0, st, x, w, maxv, c.bits, \
+                                               c.count, *gate_limit, B, Bp, CO, CI, nsplit, p, ip, y, part)
+    if (rows == 128) { if (maxv) SD_ROWS_FWD(16, false); else SD_ROWS_FWD(16, true); }
+    else { if (maxv) SD_ROWS_FWD(4, false); else SD_ROWS_FWD(4, true); }
+#undef SD_ROWS_FWD
     return check_launch("lp_rows_fwd_kernel");
 }
 
