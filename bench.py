@@ -10,7 +10,8 @@ AdamW update, and the interval-bound (certification) pass with eps = 8/255 throu
 Prints one JSON line.  `value` belongs to the mask named in config.workload (--mask); the same line carries,
 under "secondary", short runs of the other formulations of the same step: the other mask granularity, the pure
 l-inf net (q = 1), the reference's own index-list training form at its published keep probability (p = inf and
-p = 8) with its certification pass, and the wide 64x64-image configuration.  See --help for the knobs.
+p = 8) with its certification pass, one l-p distance layer at p = 8 and p = 64, and the wide 64x64-image
+configuration.  See --help for the knobs.
 """
 import argparse
 import json
@@ -279,6 +280,39 @@ def workload_text(args, mask, q):
                 "factored mask keep_x(b,n)&keep_w(m,n), each output a max over a Bernoulli(q) subset"), args.eps))
 
 
+def run_lp_layer(args, p, steps, warmup):
+    """One l-p distance layer of the headline width: forward, backward (grad_input and grad_weight) and the batch
+    mean shift of the output, inputs ~ N(0, 1) and weights ~ N(0, 1/N) (the p-annealing phase of training)."""
+    import torch
+    from sortnet_amd import ext
+    dev = torch.device("cuda:0")
+    B, N = args.batch, args.width
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(B, N, 1, generator=g).to(dev)
+    w = (torch.randn(N, N, generator=g) * N ** -0.5).to(dev)
+    gy = torch.randn(B, N, 1, generator=g).to(dev)
+    y, ys = torch.empty(B, N, 1, device=dev), torch.empty(B, N, 1, device=dev)
+    mean = torch.empty(N, device=dev)
+    gx, gw = torch.empty_like(x), torch.empty_like(w)
+
+    def step():
+        ext.norm_dist_forward(x, w, y, 1, p)
+        ext.mean_shift_forward(y, mean, None, 0.1, ys)
+        ext.norm_dist_backward_input_weight(gy, x, w, y, gx, gw, 1, p)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {"ms_per_step": ms, "samples_per_s": B / (ms * 1e-3), "steps": steps,
+            "workload": "one l-p distance layer %dx%dx%d at p=%g: forward + mean shift + backward (input and weight), "
+                        "x~N(0,1), w~N(0,1/N)" % (B, N, N, p)}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -349,6 +383,8 @@ def main():
                                             "interval sort neuron for the bounds, all layers, B=%d" % args.batch}
         r = run_index_lists(args, 0.75, 8.0, short, warm)
         sec["index_lists_q0.75_p8"] = {k: r[k] for k in ("ms_per_step", "samples_per_s", "steps", "workload")}
+        for pp in (8.0, 64.0):
+            sec["lp_layer_p%g" % pp] = run_lp_layer(args, pp, short, warm)
         if (args.batch, args.width, args.in_features, args.classes) == (512, 5120, 3072, 10):
             r = run_masked(args, args.mask, args.q, short, warm, batch=256, in_features=12288, width=10240, classes=200,
                            eps=1.0 / 255)

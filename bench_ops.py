@@ -100,6 +100,9 @@ def main():
             t("norm_dist_backward_input_weight p=%g" % p,
               lambda: ext.norm_dist_backward_input_weight(gy, xn, w, y, gx, gw, 1, p), fb)
             t("norm_dist_backward_input p=%g" % p, lambda: ext.norm_dist_backward_input(gy, xn, w, y, gx, 1, p), fb / 2)
+        if not args.json:
+            print("  (general p: the rate counts all B*M*N terms; the candidate-table kernels evaluate marked inputs only,"
+                  " so it can exceed the peak)", flush=True)
     if "idx" in on:
         # index-list ("dropout") form: every 32-sample sub-batch keeps its own ~q share of the inputs and outputs
         qk = args.keep
