@@ -181,3 +181,55 @@ def test_graph_replays_of_the_lds_direct_kernels():
                 _close(captured[name], eager[name], "%s, replay %d" % (name, replay))
             else:
                 assert torch.equal(eager[name], captured[name]), "%s, replay %d" % (name, replay)
+
+
+def test_graph_replays_of_the_candidate_table_kernels(oracle):
+    """Dense l-p calls at general p queue a candidate-table kernel and an every-term kernel for the same result and
+    a count taken on the device picks one, so ONE captured graph serves both kinds of data: replays on weights far
+    smaller than the inputs (the table kernel runs) and on weights as large as the inputs (the every-term kernels
+    run) must both reproduce eager calls, and the oracle."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, CI, CO, p = 160, 1024, 300, 64.0
+    g = torch.Generator().manual_seed(25)
+    x = torch.empty(B, CI, 1, device=dev); w = torch.empty(CO, CI, device=dev); gy = torch.empty(B, CO, 1, device=dev)
+
+    def outputs():
+        return dict(y=torch.empty(B, CO, 1, device=dev), gx=torch.empty_like(x), gw=torch.empty_like(w),
+                    gx2=torch.empty_like(x))
+
+    def run(o):
+        ext.norm_dist_forward(x, w, o["y"], 1, p)
+        ext.norm_dist_backward_input_weight(gy, x, w, o["y"], o["gx"], o["gw"], 1, p)
+        ext.norm_dist_backward_input(gy, x, w, o["y"], o["gx2"], 1, p)
+
+    def new_inputs(wscale):
+        x.copy_(torch.randn(B, CI, 1, generator=g)); w.copy_(torch.randn(CO, CI, generator=g) * wscale)
+        gy.copy_(torch.randn(B, CO, 1, generator=g))
+
+    new_inputs(0.02)
+    eager, captured = outputs(), outputs()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(captured)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run(captured)
+    for replay, wscale in enumerate((0.02, 1.0, 0.02, 1.5)):
+        new_inputs(wscale)
+        run(eager)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name in eager:
+            a, b = captured[name].cpu().numpy(), eager[name].cpu().numpy()
+            np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-4 * float(np.abs(b).max()), err_msg="%s, replay %d" % (name, replay))
+        ry = oracle.norm_dist_forward(x.cpu().numpy(), w.cpu().numpy(), p, 1)
+        np.testing.assert_allclose(captured["y"].cpu().numpy(), ry, rtol=1e-5, err_msg="replay %d" % replay)
+        rgx, rgw = oracle.norm_dist_backward(gy.cpu().numpy(), x.cpu().numpy(), w.cpu().numpy(), ry, p, 1)
+        # the kernels differentiated their own y, which agrees with the oracle's to rel 1e-5: (d/y)^(p-1) moves by p times that
+        for got, ref in ((captured["gx"], rgx), (captured["gw"], rgw), (captured["gx2"], rgx)):
+            np.testing.assert_allclose(got.cpu().numpy(), ref, rtol=2e-3, atol=2e-3 * float(np.abs(ref).max()))
