@@ -47,6 +47,7 @@ _OTHER = {
     "sd_last_error": ([], ctypes.c_char_p),
     "sd_last_forward_kernel": ([], ctypes.c_char_p),
     "sd_set_lp_candidate_density": ([_f], _i),
+    "sd_set_bound_candidate_density": ([_f], _i),
     "sd_rng_word": ([_u, _u, _u, _u], _u),
     "sd_mask_threshold8": ([_f], _u),
     "sd_mask_threshold16": ([_f], _u),
@@ -93,6 +94,14 @@ def set_lp_candidate_density(density):
     rc = lib.sd_set_lp_candidate_density(float(density))
     if rc != 0:
         raise RuntimeError("sd_set_lp_candidate_density failed: %s" % lib.sd_last_error().decode())
+
+
+def set_bound_candidate_density(density):
+    """Share of marked candidate-table entries up to which the dense interval forward works from the table (0: never)."""
+    lib = load()
+    rc = lib.sd_set_bound_candidate_density(float(density))
+    if rc != 0:
+        raise RuntimeError("sd_set_bound_candidate_density failed: %s" % lib.sd_last_error().decode())
 
 
 def last_forward_kernel():

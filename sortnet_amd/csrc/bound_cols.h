@@ -1,0 +1,29 @@
+// Interval-bound forward (values only) of dense single-group layers from per-weight-row candidate tables.
+//
+// yL[b,m] = max(1e-10, max_n max(l[b,n] - w[m,n], w[m,n] - u[b,n])) and yU[b,m] = max(1e-10, max_n max(w[m,n] - l[b,n],
+// u[b,n] - w[m,n])) (core/cuda/bound_inf_dist_cuda.cu:15-118) are maxima, so an input n whose term cannot reach a
+// lower bound of the result can be left out without changing a bit.  Over a tile of 128 batch rows the terms of
+// (m, n) are bracketed by the column minima / maxima of l and u: when the rows of the tile are alike (the bounds
+// of hidden layers) and the weights of a row are not, few inputs per weight row can hold the maximum.  A bit table
+// (tile, 32 inputs, weight row) marks them; the kernel gives a wavefront one weight row at a time (64 lanes =
+// 64 batch rows x 2), so the table is read with scalar instructions and an unmarked input costs nothing.
+#pragma once
+#include "common.h"
+
+namespace sd {
+
+// inputs of one bit-table word; CI must be a multiple of it
+constexpr int kColsChunk = 32;
+
+// bytes of workspace bound_cols_forward needs
+size_t bound_cols_workspace(int B, int CO, int CI);
+
+// Builds the table, counts its marks on the device and queues the table kernel so that it runs only when at most
+// `density` of all (tile, weight row, input) triples are marked; the caller queues the kernel that evaluates every
+// term with the opposite condition on the same counter (*gate, *gate_limit).  outL / outU must be zero-filled:
+// the slices of the input range merge by atomic maximum.
+int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float* outL,
+                       float* outU, void* ws, float density, const unsigned long long** gate,
+                       unsigned long long* gate_limit, hipStream_t st);
+
+}  // namespace sd

@@ -1,0 +1,371 @@
+// Interval-bound forward from per-weight-row candidate tables (see bound_cols.h).
+#include "bound_cols.h"
+
+namespace sd {
+
+namespace {
+
+constexpr int kChunk = kColsChunk;   // inputs per table word
+constexpr int kTileB = 128;          // batch rows of a tile: 64 lanes x 2
+constexpr int kTileW = 128;          // weight rows of a workgroup of the main kernel: 16 wavefronts x 8
+constexpr int kLowSlices = 8;        // slices of the input range in the two table kernels
+constexpr int kSegChunks = 64;       // chunks whose table words the main kernel keeps in LDS at a time
+
+inline size_t align256(size_t b) { return (b + 255) / 256 * 256; }
+inline int tiles_b(int B) { return (B + kTileB - 1) / kTileB; }
+inline int mpad_of(int M) { return (M + kTileW - 1) / kTileW * kTileW; }
+
+struct Carve {
+    float* xr;        // [S][4][N]  per tile and input: min l, max l, min u, max u over the tile's rows (repaired)
+    float* low;       // [S][2][Mp] lower bounds of the upper / lower result of every output of (tile, weight row)
+    unsigned long long* count;   // marks in the table
+    uint32_t* bits;   // [S][NCH][Mp] bit i of word (s, c, m) = input 32 c + i may hold a maximum of weight row m in tile s
+    uint32_t* partial;   // marks per wavefront of the table kernel
+};
+
+Carve carve(void* ws, int B, int M, int N) {
+    const int S = tiles_b(B), Mp = mpad_of(M), NCH = N / kChunk;
+    char* p = static_cast<char*>(ws);
+    Carve c;
+    c.xr = reinterpret_cast<float*>(p); p += align256((size_t)S * 4 * N * 4);
+    c.low = reinterpret_cast<float*>(p); p += (size_t)S * 2 * Mp * 4;   // Mp is a multiple of 128: stays 8-byte aligned
+    c.count = reinterpret_cast<unsigned long long*>(p); p += 256;
+    c.bits = reinterpret_cast<uint32_t*>(p); p += align256((size_t)S * NCH * Mp * 4);
+    c.partial = reinterpret_cast<uint32_t*>(p); p += align256((size_t)(Mp / 64) * kLowSlices * 4 * 4);
+    return c;
+}
+
+// inverted intervals become their midpoint (core/cuda/bound_inf_dist_cuda.cu:63)
+__device__ __forceinline__ void repair(float& l, float& u) {
+    if (l > u) l = u = (l + u) * 0.5f;
+}
+
+// ---- tables ----------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) col_range_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
+                                                        int B, int N, float* __restrict__ xr) {
+    // 64 inputs x 4 groups of 32 rows per workgroup, combined through LDS
+    __shared__ float part[4][4][64];
+    const int nl = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int n = blockIdx.x * 64 + nl, s = blockIdx.y;
+    const int r0 = s * kTileB + grp * (kTileB / 4);
+    const int r1 = r0 + kTileB / 4 < B ? r0 + kTileB / 4 : B;
+    float lmin = __builtin_inff(), lmax = -__builtin_inff(), umin = __builtin_inff(), umax = -__builtin_inff();
+    if (n < N) {
+        #pragma unroll 4
+        for (int r = r0; r < r1; r++) {
+            float l = xl[(size_t)r * N + n], u = xu[(size_t)r * N + n];
+            repair(l, u);
+            lmin = fminf(lmin, l); lmax = fmaxf(lmax, l);
+            umin = fminf(umin, u); umax = fmaxf(umax, u);
+        }
+    }
+    part[grp][0][nl] = lmin; part[grp][1][nl] = lmax; part[grp][2][nl] = umin; part[grp][3][nl] = umax;
+    __syncthreads();
+    if (grp == 0 && n < N) {
+        #pragma unroll
+        for (int g = 1; g < 4; g++) {
+            lmin = fminf(lmin, part[g][0][nl]); lmax = fmaxf(lmax, part[g][1][nl]);
+            umin = fminf(umin, part[g][2][nl]); umax = fmaxf(umax, part[g][3][nl]);
+        }
+        float* o = xr + (size_t)s * 4 * N + n;
+        o[0] = lmin; o[N] = lmax; o[2 * (size_t)N] = umin; o[3 * (size_t)N] = umax;
+    }
+}
+
+// The two table kernels share their tiling: a workgroup takes 64 weight rows (one per lane) and a slice of the
+// inputs; wavefront v works on batch tile v (+ 4, + 8, ...), for which the column ranges are wave-uniform
+// (LDS broadcasts); the weights go through LDS, 64 x 32 at a time, so that a lane can own a row.
+//   LOW:  lower bounds of the results, max_n of the smallest each term can be over the rows of the tile
+//         (fp32 subtraction is monotone, so the bound holds for the rounded terms), merged over the slices by
+//         atomic maximum of the bit patterns (all values >= 1e-10 > 0 on zero-filled memory);
+//   else: one table word per (tile, chunk, weight row): bit n set when the largest the term can be reaches the
+//         lower bound of the upper or of the lower result; the marks are counted.
+template <bool LOW>
+__global__ void __launch_bounds__(256) col_table_kernel(const float* __restrict__ w, const float* __restrict__ xr,
+                                                        int M, int N, int S, int Mp, float* __restrict__ low,
+                                                        uint32_t* __restrict__ bits, uint32_t* __restrict__ partial) {
+    // row stride 36 words: 16-byte rows, and the 128-bit reads of 16 consecutive lanes fall on disjoint banks
+    __shared__ __attribute__((aligned(16))) float wt[64][kChunk + 4];
+    __shared__ __attribute__((aligned(16))) float xs[4][4][kChunk];   // column ranges of the four batch tiles of this pass, current chunk
+    const int tid = threadIdx.x, r = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m0 = blockIdx.x * 64, NCH = N / kChunk;
+    const int per = (NCH + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int c_lo = blockIdx.y * per, c_hi = c_lo + per < NCH ? c_lo + per : NCH;
+    const int lrow = tid >> 2, q = tid & 3;
+    const int mload = m0 + lrow < M ? m0 + lrow : M - 1;
+    const bool valid = m0 + r < M;
+    // this work-item's two values of xs: tile tid / 64 of the pass, range tid / 16 % 4, inputs 2 (tid % 16), + 1
+    const int xt = tid >> 6, xk = (tid >> 4) & 3, xn = 2 * (tid & 15);
+    int marks = 0;
+    for (int sb = 0; sb < S; sb += 4) {
+        const int s = sb + wave;
+        const bool active = s < S;
+        float LU = kEps, LL = kEps;
+        if (!LOW && active) {
+            LU = fmaxf(kEps, low[(size_t)(s * 2) * Mp + m0 + r]);
+            LL = fmaxf(kEps, low[(size_t)(s * 2 + 1) * Mp + m0 + r]);
+        }
+        // the weights and ranges of the next chunk are fetched while the current one is used
+        float4 pa, pb;
+        float2 px;
+        const float* xsrc = xr + ((size_t)(sb + xt < S ? sb + xt : S - 1) * 4 + xk) * N + xn;
+        auto fetch = [&](int c) {
+            const int cc = c < c_hi ? c : c_hi - 1;
+            const float* src = w + (size_t)mload * N + cc * kChunk + 8 * q;
+            pa = *reinterpret_cast<const float4*>(src); pb = *reinterpret_cast<const float4*>(src + 4);
+            px = *reinterpret_cast<const float2*>(xsrc + cc * kChunk);
+        };
+        if (c_lo < c_hi) fetch(c_lo);
+        for (int c = c_lo; c < c_hi; c++) {
+            {
+                *reinterpret_cast<float4*>(&wt[lrow][8 * q]) = pa;
+                *reinterpret_cast<float4*>(&wt[lrow][8 * q + 4]) = pb;
+                *reinterpret_cast<float2*>(&xs[xt][xk][xn]) = px;
+            }
+            fetch(c + 1);
+            __syncthreads();
+            if (active) {
+                uint32_t word = 0;
+                #pragma unroll
+                for (int n4 = 0; n4 < kChunk; n4 += 4) {
+                    const float4 wv4 = *reinterpret_cast<const float4*>(&wt[r][n4]);
+                    const float4 a4 = *reinterpret_cast<const float4*>(&xs[wave][0][n4]);   // min l
+                    const float4 b4 = *reinterpret_cast<const float4*>(&xs[wave][1][n4]);   // max l
+                    const float4 c4 = *reinterpret_cast<const float4*>(&xs[wave][2][n4]);   // min u
+                    const float4 d4 = *reinterpret_cast<const float4*>(&xs[wave][3][n4]);   // max u
+                    const float wv[4] = {wv4.x, wv4.y, wv4.z, wv4.w};
+                    const float lmin[4] = {a4.x, a4.y, a4.z, a4.w}, lmax[4] = {b4.x, b4.y, b4.z, b4.w};
+                    const float umin[4] = {c4.x, c4.y, c4.z, c4.w}, umax[4] = {d4.x, d4.y, d4.z, d4.w};
+                    #pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        if (LOW) {
+                            LU = fmaxf(fmaxf(LU, umin[k] - wv[k]), wv[k] - lmax[k]);
+                            LL = fmaxf(fmaxf(LL, lmin[k] - wv[k]), wv[k] - umax[k]);
+                        } else {
+                            const float capU = fmaxf(wv[k] - lmin[k], umax[k] - wv[k]);
+                            const float capL = fmaxf(lmax[k] - wv[k], wv[k] - umin[k]);
+                            word |= (uint32_t)(capU >= LU || capL >= LL) << (n4 + k);
+                        }
+                    }
+                }
+                if (!LOW) {
+                    if (!valid) word = 0u;
+                    bits[((size_t)s * NCH + c) * Mp + m0 + r] = word;
+                    marks += __builtin_popcount(word);
+                }
+            }
+            __syncthreads();
+        }
+        if (LOW && active && valid) {
+            atomicMax(reinterpret_cast<int*>(low + (size_t)(s * 2) * Mp + m0 + r), __float_as_int(LU));
+            atomicMax(reinterpret_cast<int*>(low + (size_t)(s * 2 + 1) * Mp + m0 + r), __float_as_int(LL));
+        }
+    }
+    if (!LOW) {
+        // one number per wavefront for sum_marks_kernel (atomics on one address would serialise)
+        #pragma unroll
+        for (int o = 32; o; o >>= 1) marks += __shfl_xor(marks, o);
+        if (r == 0) partial[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 4 + wave] = (uint32_t)marks;
+    }
+}
+
+__global__ void __launch_bounds__(1024) sum_marks_kernel(const uint32_t* __restrict__ partial, size_t n,
+                                                         unsigned long long* __restrict__ count) {
+    __shared__ unsigned long long acc[1024];
+    unsigned long long s0 = 0;
+    for (size_t i = threadIdx.x; i < n; i += 1024) s0 += partial[i];
+    acc[threadIdx.x] = s0;
+    __syncthreads();
+    for (int o = 512; o; o >>= 1) {
+        if ((int)threadIdx.x < o) acc[threadIdx.x] += acc[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *count = acc[0];
+}
+
+// ---- main kernel --------------------------------------------------------------------------
+// A workgroup of 16 wavefronts owns 128 batch rows x 128 weight rows and a slice of the inputs.  Lane l holds the
+// batch rows l and l + 64; wavefront v the weight rows 8 v .. 8 v + 7: 32 running minima / maxima per lane.  The
+// inputs go by in chunks of 32: the l, u and weight tiles (128 x 32 each) of the next-but-one chunk are in flight
+// while the current one is used from LDS (always issued, so that the number of loads in flight is the same on every
+// path; a chunk nobody marks re-reads one hot line).  In LDS an input's operands lie together: (l, l', u, u') of a
+// lane's two rows as one 16-byte word, the 128 weights of the input in a row, so that a marked (weight row, input)
+// pair costs a wavefront two LDS reads (its own word and the weight as a broadcast) and eight vector instructions,
+// the terms of the every-term kernel.  The results leave through an
+// LDS transpose (coalesced along the weight rows) and merge over the slices by atomic maximum.
+__global__ void __launch_bounds__(1024, 1)
+bound_cols_kernel(const float* __restrict__ xl, const float* __restrict__ xu, const float* __restrict__ w,
+                  const uint32_t* __restrict__ bits, const unsigned long long* __restrict__ count,
+                  unsigned long long limit, int B, int M, int Mp, int N, int nsplit, float* __restrict__ yL,
+                  float* __restrict__ yU) {
+    constexpr int TW = 8;
+    constexpr int XROW = 4 * 64 + 4;     // floats per input in the l/u tile: 64 lanes x (l, l', u, u'), skewed by 4 banks
+    constexpr int WROW = kTileW + 4;     // floats per input in the weight tile
+    constexpr int kTileFloats = kChunk * (XROW + WROW);
+    static_assert(2 * kTileFloats >= kTileB * (kTileW + 1), "the transpose of the results fits where the tiles were");
+    if (gate_closed(count, limit, 0)) return;
+    __shared__ __attribute__((aligned(16))) float smem[2 * kTileFloats];
+    __shared__ __attribute__((aligned(16))) uint32_t wb[kSegChunks * kTileW];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int TM = (M + kTileW - 1) / kTileW, SB = (B + kTileB - 1) / kTileB, NCH = N / kChunk;
+    const int mt = blockIdx.x % TM, s = (blockIdx.x / TM) % SB, split = blockIdx.x / (TM * SB);
+    const int m0 = mt * kTileW, b0 = s * kTileB;
+    const int per = (NCH + nsplit - 1) / nsplit;
+    const int c_lo = split * per, c_hi = c_lo + per < NCH ? c_lo + per : NCH;
+    auto xt = [&](int buf) { return smem + buf * kTileFloats; };
+    auto wt = [&](int buf) { return smem + buf * kTileFloats + kChunk * XROW; };
+
+    float lo[TW][2], hi[TW][2];
+    #pragma unroll
+    for (int r = 0; r < TW; r++) { lo[r][0] = lo[r][1] = -kEps; hi[r][0] = hi[r][1] = kEps; }
+
+    // word of (chunk c, weight row m0 + i): bw[c * Mp + i]; rows past the last one, up to the padded count, hold zero.
+    // The words of up to kSegChunks chunks are copied to LDS ahead of the loop over them, so that no global load
+    // sits between two chunks.
+    const uint32_t* __restrict__ bw = bits + (size_t)s * NCH * Mp + m0;
+    int seg_lo = c_lo;
+    auto marked = [&](int c) {
+        const uint32_t* q = wb + (c - seg_lo) * kTileW;
+        return __builtin_amdgcn_ballot_w64((q[lane] | q[lane + 64]) != 0u) != 0ull;
+    };
+    const int frow = tid >> 3, fq = tid & 7;
+    const int fb = b0 + frow < B ? b0 + frow : B - 1, fm = m0 + frow < M ? m0 + frow : M - 1;
+    auto fetch = [&](int c, bool need, float4& l4, float4& u4, float4& w4) {
+        const size_t off = (size_t)c * kChunk + 4 * fq;
+        l4 = *reinterpret_cast<const float4*>(need ? xl + (size_t)fb * N + off : xl);
+        u4 = *reinterpret_cast<const float4*>(need ? xu + (size_t)fb * N + off : xu);
+        w4 = *reinterpret_cast<const float4*>(need ? w + (size_t)fm * N + off : w);
+    };
+    auto stash = [&](int buf, float4 l4, float4 u4, const float4& w4) {
+        repair(l4.x, u4.x); repair(l4.y, u4.y); repair(l4.z, u4.z); repair(l4.w, u4.w);
+        // row frow belongs to lane frow % 64, slot frow / 64 of (l, l', u, u')
+        float* dx = xt(buf) + (4 * fq) * XROW + 4 * (frow & 63) + (frow >> 6);
+        dx[0] = l4.x; dx[2] = u4.x;
+        dx[XROW] = l4.y; dx[XROW + 2] = u4.y;
+        dx[2 * XROW] = l4.z; dx[2 * XROW + 2] = u4.z;
+        dx[3 * XROW] = l4.w; dx[3 * XROW + 2] = u4.w;
+        float* dw = wt(buf) + (4 * fq) * WROW + frow;
+        dw[0] = w4.x; dw[WROW] = w4.y; dw[2 * WROW] = w4.z; dw[3 * WROW] = w4.w;
+    };
+    // The scalar unit is shared by the wavefronts of a compute unit, so the walk spends as few scalar instructions
+    // per marked input as it can: one loop per weight row over that row's own marks (find-first-set, clear, branch)
+    // instead of a walk over the union with a test per row.
+    auto compute = [&](int buf, int c) {
+        const float* X = xt(buf) + 4 * lane, *W = wt(buf) + wave * TW;
+        const uint4* rowwords = reinterpret_cast<const uint4*>(wb + (c - seg_lo) * kTileW + wave * TW);
+        const uint4 q0 = rowwords[0], q1 = rowwords[1];
+        const uint32_t words[TW] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        #pragma unroll
+        for (int r = 0; r < TW; r++) {
+            uint32_t bm = __builtin_amdgcn_readfirstlane(words[r]);
+            while (bm) {
+                const int n = __builtin_ctz(bm);
+                bm &= bm - 1;
+                const float4 x = *reinterpret_cast<const float4*>(X + n * XROW);   // l, l', u, u' of the lane's two rows
+                const float wv = W[n * WROW + r];
+                const float a1 = wv - x.x, a2 = x.z - wv, b1 = wv - x.y, b2 = x.w - wv;
+                lo[r][0] = fminf(fminf(lo[r][0], a1), a2);
+                hi[r][0] = fmaxf(fmaxf(hi[r][0], a1), a2);
+                lo[r][1] = fminf(fminf(lo[r][1], b1), b2);
+                hi[r][1] = fmaxf(fmaxf(hi[r][1], b1), b2);
+            }
+        }
+    };
+
+    for (; seg_lo < c_hi; seg_lo += kSegChunks) {
+        const int seg_hi = seg_lo + kSegChunks < c_hi ? seg_lo + kSegChunks : c_hi;
+        __syncthreads();   // the previous segment's words and tiles are no longer read
+        for (int e = tid; e < (seg_hi - seg_lo) * kTileW; e += 1024)
+            wb[e] = bw[(size_t)(seg_lo + (e >> 7)) * Mp + (e & (kTileW - 1))];
+        __syncthreads();
+        float4 la, ua, wa, lb, ub, wc;
+        bool n0 = marked(seg_lo), n1 = seg_lo + 1 < seg_hi ? marked(seg_lo + 1) : false;
+        fetch(seg_lo, n0, la, ua, wa);
+        fetch(seg_lo + 1 < seg_hi ? seg_lo + 1 : seg_lo, n1, lb, ub, wc);
+        if (n0) stash(0, la, ua, wa);
+        __syncthreads();
+        for (int c = seg_lo; c < seg_hi; c += 2) {
+            const bool n2 = c + 2 < seg_hi ? marked(c + 2) : false;
+            fetch(c + 2 < seg_hi ? c + 2 : c, n2, la, ua, wa);
+            if (n0) compute(0, c);
+            if (n1) stash(1, lb, ub, wc);
+            __syncthreads();
+            if (c + 1 >= seg_hi) break;
+            const bool n3 = c + 3 < seg_hi ? marked(c + 3) : false;
+            fetch(c + 3 < seg_hi ? c + 3 : c, n3, lb, ub, wc);
+            if (n1) compute(1, c + 1);
+            if (n2) stash(0, la, ua, wa);
+            __syncthreads();
+            n0 = n2; n1 = n3;
+        }
+    }
+
+    // results: [batch row][weight row] through LDS, lower then upper
+    float* tr = smem;
+    #pragma unroll
+    for (int which = 0; which < 2; which++) {
+        __syncthreads();
+        #pragma unroll
+        for (int r = 0; r < TW; r++) {
+            #pragma unroll
+            for (int j = 0; j < 2; j++)
+                tr[(lane + 64 * j) * (kTileW + 1) + wave * TW + r] = which == 0 ? -lo[r][j] : hi[r][j];
+        }
+        __syncthreads();
+        float* y = which == 0 ? yL : yU;
+        for (int e = tid; e < kTileB * kTileW; e += 1024) {
+            const int bl = e >> 7, ml = e & (kTileW - 1);
+            if (b0 + bl < B && m0 + ml < M) {
+                const float v = tr[bl * (kTileW + 1) + ml];
+                float* dst = y + (size_t)(b0 + bl) * M + m0 + ml;
+                // both results are >= 1e-10 > 0, so their bit patterns order like integers
+                if (nsplit > 1) atomicMax(reinterpret_cast<int*>(dst), __float_as_int(v));
+                else *dst = v;
+            }
+        }
+    }
+}
+
+}  // namespace
+
+size_t bound_cols_workspace(int B, int CO, int CI) {
+    const int S = tiles_b(B), Mp = mpad_of(CO), NCH = CI / kChunk;
+    return align256((size_t)S * 4 * CI * 4) + (size_t)S * 2 * Mp * 4 + 256 + align256((size_t)S * NCH * Mp * 4) +
+           align256((size_t)(Mp / 64) * kLowSlices * 4 * 4);
+}
+
+int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float* outL,
+                       float* outU, void* ws, float density, const unsigned long long** gate,
+                       unsigned long long* gate_limit, hipStream_t st) {
+    if (CI % kChunk != 0 || B < 1 || CO < 1) { set_error("bound_cols_forward: shape not supported"); return SD_ERR_ARG; }
+    const Carve c = carve(ws, B, CO, CI);
+    const int S = tiles_b(B), Mp = mpad_of(CO), NCH = CI / kChunk;
+    int rc;
+    if ((rc = fill_zero(c.low, (size_t)S * 2 * Mp, st))) return rc;
+    hipLaunchKernelGGL(col_range_kernel, dim3((CI + 63) / 64, S), dim3(256), 0, st, xl, xu, B, CI, c.xr);
+    if ((rc = check_launch("col_range_kernel"))) return rc;
+    const int slices = NCH < kLowSlices ? NCH : kLowSlices;
+    hipLaunchKernelGGL(col_table_kernel<true>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial);
+    if ((rc = check_launch("col_table_kernel<low>"))) return rc;
+    hipLaunchKernelGGL(col_table_kernel<false>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial);
+    if ((rc = check_launch("col_table_kernel<bits>"))) return rc;
+    hipLaunchKernelGGL(sum_marks_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count);
+    if ((rc = check_launch("sum_marks_kernel"))) return rc;
+    const double all = (double)S * CO * CI;
+    *gate = c.count;
+    *gate_limit = (unsigned long long)(all * (density < 0.f ? 0.f : density > 1.f ? 1.f : density));
+    // a few workgroups per compute unit over the run: the work of a workgroup follows the marks of its weight rows
+    const int TM = Mp / kTileW;
+    const long long wgs = (long long)TM * S;
+    int nsplit = (int)((2ll * num_cus() + wgs - 1) / wgs);
+    if (nsplit > NCH / 8) nsplit = NCH / 8;
+    if (nsplit > 16) nsplit = 16;
+    if (nsplit < 1) nsplit = 1;
+    hipLaunchKernelGGL(bound_cols_kernel, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.bits, c.count,
+                       *gate_limit, B, CO, Mp, CI, nsplit, outL, outU);
+    return check_launch("bound_cols_kernel");
+}
+
+}  // namespace sd

@@ -749,6 +749,11 @@ struct BoundNograd : PolicyBase {
     }
 };
 
+// the same kernel as one of two queued for a result, see FwdArgs::gate
+struct BoundNogradGated : BoundNograd {
+    static constexpr bool GATED = true;
+};
+
 // interval bounds with indices (core/cuda/bound_inf_dist_cuda.cu:121-238), chunk-tracked like LinfChunk: the lower side tracks the largest
 // -min(t1,t2) (a positive number once it passes 1e-10), the upper side the largest max(t1,t2);
 // resolve_bound_kernel recovers the exact positions and branch bits

@@ -1,10 +1,18 @@
 // l-inf distance, masked order-statistic neuron and interval-bound forward entry points.
 #include "fwd_tile.h"
 #include "fwd_args.h"
+#include "bound_cols.h"
 #include <mutex>
 #include <type_traits>
 
 using namespace sd;
+
+// largest share of marked (tile, weight row, input) triples at which the candidate-table kernel of the interval
+// forward runs instead of the kernel that evaluates every term (sd_set_bound_candidate_density); negative: built-in
+static float g_bound_density = -1.f;
+// measured at B = 512, M = N = 5120: the table kernel takes 0.14 + 3.3 x share ms (140 us of staging, then about 75 SIMD
+// cycles per marked (tile, weight row, input)) and the table 0.08 ms, against 1.04 ms for every term
+constexpr float kBoundColsCap = 0.22f;
 
 // One work-item per (row, chunk): the 32 keep bits of the factored mask for inputs
 // chunk*32 .. chunk*32+31 of an x row (stream 1) or a w row (stream 2).
@@ -209,12 +217,31 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
     static const int kTb42[] = {4, 2};
     const int TB = pick_tb(a, kTb42, 2, 128);
     a.nsplit = pick_nsplit(a, 16 * TB, 16 * 8);
-    if (a.nsplit > 1) {
+    // dense single-group layers: a kernel that works from per-weight-row candidate tables is queued in front of the
+    // one that evaluates every term, and a count taken on the device decides which of the two runs
+    const float cap = g_bound_density >= 0.f ? g_bound_density : kBoundColsCap;
+    const bool cols = cap > 0.f && G == 1 && HW == 1 && CI % kColsChunk == 0 && a.fast_x && a.fast_w;
+    if (a.nsplit > 1 || cols) {
         if ((rc = fill_zero(outputL, (size_t)B * CO * HW, st))) return rc;
         if ((rc = fill_zero(outputU, (size_t)B * CO * HW, st))) return rc;
     }
+    if (cols) {
+        void* ws = workspace(bound_cols_workspace(B, CO, CI), st);
+        if (!ws) return SD_ERR_HIP;
+        if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, outputL, outputU, ws, cap, &a.gate, &a.gate_limit, st)))
+            return rc;
+        a.gate_above = 1;
+        if (TB == 2) return launch_fwd<BoundNogradGated, 2, 8>(a, st);
+        return launch_fwd<BoundNogradGated, 4, 8>(a, st);
+    }
     if (TB == 2) return launch_fwd<BoundNograd, 2, 8>(a, st);
     return launch_fwd<BoundNograd, 4, 8>(a, st);
+}
+
+extern "C" int sd_set_bound_candidate_density(float density) {
+    SD_REQUIRE(density <= 1.f, "set_bound_candidate_density: %g is above 1", (double)density);
+    g_bound_density = density;
+    return SD_OK;
 }
 
 extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* inputU, const float* weight,

@@ -212,10 +212,15 @@ lp_rows_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w, con
     // word of (chunk c, row r0 + i): bw[c * Bp + i]; rows past the batch, up to the padded count, hold zero words
     const uint32_t* __restrict__ bw = bits + (size_t)t * NCH * Bp + r0;
     const int rows_here = Bp - r0 < ROWS ? Bp - r0 : ROWS;
+    // The words of up to SEG chunks are copied to LDS ahead of the loop over them (zero for rows past the padded
+    // count), so that no global load sits between two chunks.
+    constexpr int SEG = NW == 16 ? 64 : 32;
+    __shared__ uint32_t wb[SEG * ROWS];
+    int seg_lo = c_lo;
     auto marked = [&](int c) {   // anything marked in chunk c for the rows of the workgroup
-        const uint32_t* q = bw + (size_t)c * Bp;
-        uint32_t v = lane < rows_here ? q[lane] : 0u;
-        if (ROWS > 64 && lane + 64 < rows_here) v |= q[lane + 64];
+        const uint32_t* q = wb + (c - seg_lo) * ROWS;
+        uint32_t v = lane < ROWS ? q[lane < ROWS ? lane : 0] : 0u;
+        if (ROWS > 64) v |= q[lane + 64];
         return __builtin_amdgcn_ballot_w64(v != 0u) != 0ull;
     };
     // always issued, so that the number of loads in flight is the same on every path (the waits the compiler places
@@ -245,8 +250,7 @@ lp_rows_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w, con
         uint32_t br[TB], u = 0;
         #pragma unroll
         for (int r = 0; r < TB; r++) {
-            const int i = wave * TB + r;
-            br[r] = i < rows_here ? __builtin_amdgcn_readfirstlane(bw[(size_t)c * Bp + i]) : 0u;
+            br[r] = __builtin_amdgcn_readfirstlane(wb[(c - seg_lo) * ROWS + wave * TB + r]);
             u |= br[r];
         }
         while (u) {
@@ -282,22 +286,29 @@ lp_rows_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w, con
 
     // Two chunks are in flight: while chunk c is used from LDS, chunk c + 1 waits in registers and chunk c + 2 is
     // being fetched; a chunk's registers go to the LDS buffer that the chunk before the previous one has left.
-    if (c_lo < c_hi) {
-        float4 wa[WV], xa, wb[WV], xb;
-        bool n0 = marked(c_lo), n1 = c_lo + 1 < c_hi ? marked(c_lo + 1) : false;
-        fetch(c_lo, n0, wa, xa);
-        fetch(c_lo + 1 < c_hi ? c_lo + 1 : c_lo, n1, wb, xb);
+    for (; seg_lo < c_hi; seg_lo += SEG) {
+        const int seg_hi = seg_lo + SEG < c_hi ? seg_lo + SEG : c_hi;
+        __syncthreads();   // the previous segment's words and tiles are no longer read
+        for (int e = tid; e < (seg_hi - seg_lo) * ROWS; e += NT) {
+            const int i = e % ROWS;
+            wb[e] = i < rows_here ? bw[(size_t)(seg_lo + e / ROWS) * Bp + i] : 0u;
+        }
+        __syncthreads();
+        float4 wa[WV], xa, wc[WV], xc;
+        bool n0 = marked(seg_lo), n1 = seg_lo + 1 < seg_hi ? marked(seg_lo + 1) : false;
+        fetch(seg_lo, n0, wa, xa);
+        fetch(seg_lo + 1 < seg_hi ? seg_lo + 1 : seg_lo, n1, wc, xc);
         if (n0) stash(0, wa, xa);
         __syncthreads();
-        for (int c = c_lo; c < c_hi; c += 2) {
-            const bool n2 = c + 2 < c_hi ? marked(c + 2) : false;
-            fetch(c + 2 < c_hi ? c + 2 : c, n2, wa, xa);
+        for (int c = seg_lo; c < seg_hi; c += 2) {
+            const bool n2 = c + 2 < seg_hi ? marked(c + 2) : false;
+            fetch(c + 2 < seg_hi ? c + 2 : c, n2, wa, xa);
             if (n0) compute(0, c);
-            if (n1) stash(1, wb, xb);
+            if (n1) stash(1, wc, xc);
             __syncthreads();
-            if (c + 1 >= c_hi) break;
-            const bool n3 = c + 3 < c_hi ? marked(c + 3) : false;
-            fetch(c + 3 < c_hi ? c + 3 : c, n3, wb, xb);
+            if (c + 1 >= seg_hi) break;
+            const bool n3 = c + 3 < seg_hi ? marked(c + 3) : false;
+            fetch(c + 3 < seg_hi ? c + 3 : c, n3, wc, xc);
             if (n1) compute(1, c + 1);
             if (n2) stash(0, wa, xa);
             __syncthreads();

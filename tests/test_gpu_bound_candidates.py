@@ -1,0 +1,95 @@
+"""GPU parity of the interval-bound forward (values only) that works from candidate tables (dense single-group
+layers, CI % 32 == 0).
+
+`bound_inf_dist_forward_nograd` queues a kernel that evaluates only the inputs a table marks as able to hold a
+maximum, and the kernel that evaluates every term; a count taken on the device picks one.  Both must give the
+bits of the oracle (core/cuda/bound_inf_dist_cuda.cu:15-118 semantics, inverted intervals repaired to their
+midpoint): the tests force either kernel (density 1 / 0) and the built-in limit, on batches whose rows are nearly
+alike (the bounds of hidden layers: the table marks little), on unrelated rows (it marks nearly everything) and on
+inverted intervals."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+@pytest.fixture
+def density():
+    from sortnet_amd import _lib
+
+    def set_(d):
+        _lib.set_bound_candidate_density(d)
+    yield set_
+    _lib.set_bound_candidate_density(-1.0)
+
+
+def _intervals(B, CI, kind, seed):
+    g = torch.Generator().manual_seed(seed)
+    if kind == "rows_alike":
+        x = torch.randn(1, CI, 1, generator=g) * 0.5 + torch.randn(B, CI, 1, generator=g) * 0.01
+    else:
+        x = torch.randn(B, CI, 1, generator=g)
+    r = torch.rand(B, CI, 1, generator=g) * 0.05
+    xl, xu = (x - r).contiguous(), (x + r).contiguous()
+    if kind == "inverted":
+        m = torch.rand(B, CI, 1, generator=g) < 0.1
+        xl, xu = torch.where(m, xu, xl).contiguous(), torch.where(m, xl, xu).contiguous()
+    return xl, xu
+
+
+@pytest.mark.parametrize("dens", [1.0, 0.0, -1.0])
+@pytest.mark.parametrize("B,CI,CO", [(70, 96, 64), (33, 2048, 300), (130, 1024, 513), (1, 32, 1), (257, 320, 129),
+                                     (512, 512, 640)])
+def test_bound_candidate_kernel_matches_oracle(oracle, density, dens, B, CI, CO):
+    """Ragged batch tiles (B not a multiple of 128) and weight tiles (CO not a multiple of 128), one and several of
+    each, input ranges cut in slices or not."""
+    from sortnet_amd import ext
+    dev = _dev()
+    density(dens)
+    for kind in ("rows_alike", "random", "inverted"):
+        for wscale in (0.02, 1.0):
+            xl, xu = _intervals(B, CI, kind, B + CI)
+            g = torch.Generator().manual_seed(2)
+            w = (torch.randn(CO, CI, generator=g) * wscale).contiguous()
+            rl, ru = oracle.bound_inf_dist_forward(xl.numpy(), xu.numpy(), w.numpy(), 1, need_pos=False)
+            yl = torch.full((B, CO, 1), float("nan"), device=dev)
+            yu = torch.full((B, CO, 1), float("nan"), device=dev)
+            ext.bound_inf_dist_forward_nograd(xl.to(dev), xu.to(dev), w.to(dev), yl, yu, 1)
+            tag = "dens=%g %s wscale=%g" % (dens, kind, wscale)
+            assert np.array_equal(yl.cpu().numpy(), rl), tag
+            assert np.array_equal(yu.cpu().numpy(), ru), tag
+
+
+def test_bound_candidate_kernel_at_layer_size(density):
+    """B = 512, N = M = 5120 with rows that are nearly alike (as the bounds of a hidden layer are): the table kernel
+    and the every-term kernel give the same bits, and the built-in limit does too."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, N, M = 512, 5120, 5120
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(1, N, 1, generator=g) * 0.02 + torch.randn(B, N, 1, generator=g) * 0.004
+    r = 0.02 + torch.rand(B, N, 1, generator=g) * 0.002
+    xl, xu = (x - r).contiguous().to(dev), (x + r).contiguous().to(dev)
+    w = (torch.randn(M, N, generator=g) * N ** -0.5).contiguous().to(dev)
+    out = {}
+    for dens in (0.0, 1.0, -1.0):
+        density(dens)
+        yl, yu = torch.empty(B, M, 1, device=dev), torch.empty(B, M, 1, device=dev)
+        ext.bound_inf_dist_forward_nograd(xl, xu, w, yl, yu, 1)
+        out[dens] = (yl, yu)
+    for dens in (1.0, -1.0):
+        assert torch.equal(out[dens][0], out[0.0][0]) and torch.equal(out[dens][1], out[0.0][1]), dens
+
+
+def test_bound_candidate_density_argument(density):
+    from sortnet_amd import _lib
+    with pytest.raises(RuntimeError):
+        _lib.set_bound_candidate_density(1.5)
+    density(0.3)

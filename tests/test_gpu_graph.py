@@ -196,15 +196,20 @@ def test_graph_replays_of_the_candidate_table_kernels(oracle):
 
     def outputs():
         return dict(y=torch.empty(B, CO, 1, device=dev), gx=torch.empty_like(x), gw=torch.empty_like(w),
-                    gx2=torch.empty_like(x))
+                    gx2=torch.empty_like(x), yl=torch.empty(B, CO, 1, device=dev), yu=torch.empty(B, CO, 1, device=dev))
 
     def run(o):
+        # the interval forward makes the same kind of choice (rows of the batch alike or not)
+        ext.bound_inf_dist_forward_nograd(x - 0.03, x + 0.03, w, o["yl"], o["yu"], 1)
         ext.norm_dist_forward(x, w, o["y"], 1, p)
         ext.norm_dist_backward_input_weight(gy, x, w, o["y"], o["gx"], o["gw"], 1, p)
         ext.norm_dist_backward_input(gy, x, w, o["y"], o["gx2"], 1, p)
 
     def new_inputs(wscale):
-        x.copy_(torch.randn(B, CI, 1, generator=g)); w.copy_(torch.randn(CO, CI, generator=g) * wscale)
+        # small weights come with batch rows that are nearly alike, large weights with unrelated rows
+        base = torch.randn(1, CI, 1, generator=g) if wscale < 0.1 else 0.0
+        x.copy_(base + torch.randn(B, CI, 1, generator=g) * (0.01 if wscale < 0.1 else 1.0))
+        w.copy_(torch.randn(CO, CI, generator=g) * wscale)
         gy.copy_(torch.randn(B, CO, 1, generator=g))
 
     new_inputs(0.02)
@@ -225,8 +230,13 @@ def test_graph_replays_of_the_candidate_table_kernels(oracle):
         graph.replay()
         torch.cuda.synchronize()
         for name in eager:
+            if name in ("yl", "yu"):
+                assert torch.equal(captured[name], eager[name]), "%s, replay %d" % (name, replay)
+                continue
             a, b = captured[name].cpu().numpy(), eager[name].cpu().numpy()
             np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-4 * float(np.abs(b).max()), err_msg="%s, replay %d" % (name, replay))
+        rl, ru = oracle.bound_inf_dist_forward((x - 0.03).cpu().numpy(), (x + 0.03).cpu().numpy(), w.cpu().numpy(), 1, need_pos=False)
+        assert np.array_equal(captured["yl"].cpu().numpy(), rl) and np.array_equal(captured["yu"].cpu().numpy(), ru), replay
         ry = oracle.norm_dist_forward(x.cpu().numpy(), w.cpu().numpy(), p, 1)
         np.testing.assert_allclose(captured["y"].cpu().numpy(), ry, rtol=1e-5, err_msg="replay %d" % replay)
         rgx, rgw = oracle.norm_dist_backward(gy.cpu().numpy(), x.cpu().numpy(), w.cpu().numpy(), ry, p, 1)
