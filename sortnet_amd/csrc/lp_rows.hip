@@ -161,13 +161,12 @@ int build_tables(const Carve& c, const float* x, const float* w, const float* sc
 }
 
 // ---- forward ------------------------------------------------------------------------------
-// A workgroup owns 32 batch rows x 256 output channels and a slice of the inputs; wavefront v owns rows
-// 8 v .. 8 v + 7, lane l the columns l + 64 j (j < 4): 32 sums and 32 reciprocal scales in registers.  The inputs
-// go by in chunks of 32: the weight tile (256 x 32) and the input tile (32 x 32) of the next chunk are fetched
-// while the current one is used, unless the table marks nothing in that chunk for any of the 32 rows.  Within a
-// chunk the wavefront walks the union of its rows' marked inputs: the four weights of an input are read
-// once (one LDS word per lane and column), then every row that marks the input takes its four terms through the
-// significance test of the general kernel (wave-uniform: the group of four, then each term).
+// A workgroup of NW wavefronts owns 8 NW batch rows x 256 output channels and a slice of the inputs; wavefront v
+// owns rows 8 v .. 8 v + 7, lane l the columns l + 64 j (j < 4): 32 sums and 32 reciprocal scales in registers.
+// The inputs go by in chunks of 32: the weight tile (256 x 32) and the input tile (8 NW x 32) of the next-but-one
+// chunk are in flight while the current one is used from LDS; a chunk that the table marks for none of the rows is
+// not fetched.  Within a chunk the wavefront takes its rows one after the other and walks each row's own marks:
+// the input of the row as an LDS broadcast, the four weights of the lane's columns, four terms.
 // ONLINE: no maxima are given; every sum is kept relative to the largest term met so far and rescaled when a
 // larger one comes (core/cuda/norm_dist_cuda.cu:36-160), with 1 / maximum in place of the given reciprocal scale.
 // The slice results are (sum, maximum) pairs in part[slice] and part[nsplit + slice].
@@ -246,39 +245,31 @@ lp_rows_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w, con
         }
         *reinterpret_cast<float4*>(&xt[buf][(tid >> 3) * XS + 4 * (tid & 7)]) = xr;
     };
+    // The scalar unit is shared by the wavefronts of a compute unit, so the walk spends as few scalar instructions
+    // per marked input as it can: one loop per row over that row's own marks (find-first-set, clear, branch).
     auto compute = [&](int buf, int c) {
-        uint32_t br[TB], u = 0;
         #pragma unroll
         for (int r = 0; r < TB; r++) {
-            br[r] = __builtin_amdgcn_readfirstlane(wb[(c - seg_lo) * ROWS + wave * TB + r]);
-            u |= br[r];
-        }
-        while (u) {
-            const int n = __builtin_ctz(u);
-            u &= u - 1;
-            float wv[4];
-            #pragma unroll
-            for (int j = 0; j < 4; j++) wv[j] = wt[buf][(lane + 64 * j) * WS + n];
-            #pragma unroll
-            for (int r = 0; r < TB; r++) {
-                if ((br[r] >> n) & 1u) {
-                    const float xv = xt[buf][(wave * TB + r) * XS + n];
-                    // every term of a marked input is evaluated: on data that the table suits, most of them count
-                    #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const float d = fabsf(xv - wv[j]);
-                        const float lg = p * __builtin_amdgcn_logf(d * rinv[r][j]);
-                        if (ONLINE) {
-                            // ratio above 1: a new maximum; the old sum shrinks by ratio^-p and the new term is 1.
-                            // The reciprocal need not be exact: the result is the sum's root divided by the same
-                            // reciprocal, whatever it is; only the rescaling sees its error, p times, and the root
-                            // takes that back.
-                            const bool up = lg > 0.f;
-                            const float e = __builtin_amdgcn_exp2f(up ? -lg : lg);
-                            acc[r][j] = up ? fmaf(acc[r][j], e, 1.f) : acc[r][j] + e;
-                            rinv[r][j] = up ? __builtin_amdgcn_rcpf(d) : rinv[r][j];
-                        } else acc[r][j] += __builtin_amdgcn_exp2f(lg);
-                    }
+            uint32_t bm = __builtin_amdgcn_readfirstlane(wb[(c - seg_lo) * ROWS + wave * TB + r]);
+            while (bm) {
+                const int n = __builtin_ctz(bm);
+                bm &= bm - 1;
+                const float xv = xt[buf][(wave * TB + r) * XS + n];
+                // every term of a marked input is evaluated: on data that the table suits, most of them count
+                #pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float d = fabsf(xv - wt[buf][(lane + 64 * j) * WS + n]);
+                    const float lg = p * __builtin_amdgcn_logf(d * rinv[r][j]);
+                    if (ONLINE) {
+                        // ratio above 1: a new maximum; the old sum shrinks by ratio^-p and the new term is 1.
+                        // The reciprocal need not be exact: the result is the sum's root divided by the same
+                        // reciprocal, whatever it is; only the rescaling sees its error, p times, and the root
+                        // takes that back.
+                        const bool up = lg > 0.f;
+                        const float e = __builtin_amdgcn_exp2f(up ? -lg : lg);
+                        acc[r][j] = up ? fmaf(acc[r][j], e, 1.f) : acc[r][j] + e;
+                        rinv[r][j] = up ? __builtin_amdgcn_rcpf(d) : rinv[r][j];
+                    } else acc[r][j] += __builtin_amdgcn_exp2f(lg);
                 }
             }
         }
