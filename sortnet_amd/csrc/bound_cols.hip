@@ -18,6 +18,7 @@ inline int mpad_of(int M) { return (M + kTileW - 1) / kTileW * kTileW; }
 struct Carve {
     float* xr;        // [S][4][N]  per tile and input: min l, max l, min u, max u over the tile's rows (repaired)
     float* low;       // [S][2][Mp] lower bounds of the upper / lower result of every output of (tile, weight row)
+    float* stat;      // two sums of col_range_kernel's probe, directly behind `low` (one fill clears both)
     unsigned long long* count;   // marks in the table
     uint32_t* bits;   // [S][NCH][Mp] bit i of word (s, c, m) = input 32 c + i may hold a maximum of weight row m in tile s
     uint32_t* partial;   // marks per wavefront of the table kernel
@@ -29,6 +30,7 @@ Carve carve(void* ws, int B, int M, int N) {
     Carve c;
     c.xr = reinterpret_cast<float*>(p); p += align256((size_t)S * 4 * N * 4);
     c.low = reinterpret_cast<float*>(p); p += (size_t)S * 2 * Mp * 4;   // Mp is a multiple of 128: stays 8-byte aligned
+    c.stat = reinterpret_cast<float*>(p); p += 8;
     c.count = reinterpret_cast<unsigned long long*>(p); p += 256;
     c.bits = reinterpret_cast<uint32_t*>(p); p += align256((size_t)S * NCH * Mp * 4);
     c.partial = reinterpret_cast<uint32_t*>(p); p += align256((size_t)(Mp / 64) * kLowSlices * 4 * 4);
@@ -41,15 +43,22 @@ __device__ __forceinline__ void repair(float& l, float& u) {
 }
 
 // ---- tables ----------------------------------------------------------------------------------
+// Also answers whether the table is worth building: it can only prune when the rows of a batch tile are alike
+// compared with the entries of a weight row.  stat[0] collects the widths of the column ranges of l and u over all
+// tiles and columns, stat[1] the ranges of the same columns over the first 16 weight rows (added once, by the
+// workgroups of tile 0); see table_pointless().
 __global__ void __launch_bounds__(256) col_range_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
-                                                        int B, int N, float* __restrict__ xr) {
+                                                        const float* __restrict__ w, int B, int M, int N,
+                                                        float* __restrict__ xr, float* __restrict__ stat) {
     // 64 inputs x 4 groups of 32 rows per workgroup, combined through LDS
     __shared__ float part[4][4][64];
+    __shared__ float wpart[4][2][64];
     const int nl = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int n = blockIdx.x * 64 + nl, s = blockIdx.y;
     const int r0 = s * kTileB + grp * (kTileB / 4);
     const int r1 = r0 + kTileB / 4 < B ? r0 + kTileB / 4 : B;
     float lmin = __builtin_inff(), lmax = -__builtin_inff(), umin = __builtin_inff(), umax = -__builtin_inff();
+    float wlo = __builtin_inff(), whi = -__builtin_inff();
     if (n < N) {
         #pragma unroll 4
         for (int r = r0; r < r1; r++) {
@@ -58,18 +67,46 @@ __global__ void __launch_bounds__(256) col_range_kernel(const float* __restrict_
             lmin = fminf(lmin, l); lmax = fmaxf(lmax, l);
             umin = fminf(umin, u); umax = fmaxf(umax, u);
         }
+        if (s == 0) {
+            #pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int m = grp * 4 + k;
+                if (m < M) { const float v = w[(size_t)m * N + n]; wlo = fminf(wlo, v); whi = fmaxf(whi, v); }
+            }
+        }
     }
     part[grp][0][nl] = lmin; part[grp][1][nl] = lmax; part[grp][2][nl] = umin; part[grp][3][nl] = umax;
+    wpart[grp][0][nl] = wlo; wpart[grp][1][nl] = whi;
     __syncthreads();
-    if (grp == 0 && n < N) {
-        #pragma unroll
-        for (int g = 1; g < 4; g++) {
-            lmin = fminf(lmin, part[g][0][nl]); lmax = fmaxf(lmax, part[g][1][nl]);
-            umin = fminf(umin, part[g][2][nl]); umax = fmaxf(umax, part[g][3][nl]);
+    if (grp == 0) {
+        float bw = 0.f, ww = 0.f;
+        if (n < N) {
+            #pragma unroll
+            for (int g = 1; g < 4; g++) {
+                lmin = fminf(lmin, part[g][0][nl]); lmax = fmaxf(lmax, part[g][1][nl]);
+                umin = fminf(umin, part[g][2][nl]); umax = fmaxf(umax, part[g][3][nl]);
+                wlo = fminf(wlo, wpart[g][0][nl]); whi = fmaxf(whi, wpart[g][1][nl]);
+            }
+            float* o = xr + (size_t)s * 4 * N + n;
+            o[0] = lmin; o[N] = lmax; o[2 * (size_t)N] = umin; o[3 * (size_t)N] = umax;
+            bw = fmaxf(lmax - lmin, umax - umin);
+            if (s == 0) ww = whi - wlo;
+            if (!(bw < 3.0e38f)) bw = 3.0e38f;   // infinite or undefined widths count as very wide
         }
-        float* o = xr + (size_t)s * 4 * N + n;
-        o[0] = lmin; o[N] = lmax; o[2 * (size_t)N] = umin; o[3 * (size_t)N] = umax;
+        #pragma unroll
+        for (int o = 32; o; o >>= 1) { bw += __shfl_xor(bw, o); ww += __shfl_xor(ww, o); }
+        if (nl == 0) {
+            unsafeAtomicAdd(stat, bw);
+            if (s == 0) unsafeAtomicAdd(stat + 1, ww);
+        }
     }
+}
+
+// the batch rows of a tile differ by more than kProbeRatio times what 16 entries of a weight column do: every input
+// would be marked (images against small weights: ratio 15; the bounds of hidden layers: below 1)
+constexpr float kProbeRatio = 2.5f;
+__device__ __forceinline__ bool table_pointless(const float* stat, int S, int force) {
+    return !force && stat[0] > kProbeRatio * (float)S * stat[1];
 }
 
 // The two table kernels share their tiling: a workgroup takes 64 weight rows (one per lane) and a slice of the
@@ -83,7 +120,9 @@ __global__ void __launch_bounds__(256) col_range_kernel(const float* __restrict_
 template <bool LOW>
 __global__ void __launch_bounds__(256) col_table_kernel(const float* __restrict__ w, const float* __restrict__ xr,
                                                         int M, int N, int S, int Mp, float* __restrict__ low,
-                                                        uint32_t* __restrict__ bits, uint32_t* __restrict__ partial) {
+                                                        uint32_t* __restrict__ bits, uint32_t* __restrict__ partial,
+                                                        const float* __restrict__ stat, int force) {
+    if (table_pointless(stat, S, force)) return;   // the probe of col_range_kernel: the table would mark everything
     // row stride 36 words: 16-byte rows, and the 128-bit reads of 16 consecutive lanes fall on disjoint banks
     __shared__ __attribute__((aligned(16))) float wt[64][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float xs[4][4][kChunk];   // column ranges of the four batch tiles of this pass, current chunk
@@ -171,8 +210,10 @@ __global__ void __launch_bounds__(256) col_table_kernel(const float* __restrict_
 }
 
 __global__ void __launch_bounds__(1024) sum_marks_kernel(const uint32_t* __restrict__ partial, size_t n,
-                                                         unsigned long long* __restrict__ count) {
+                                                         unsigned long long* __restrict__ count,
+                                                         const float* __restrict__ stat, int S, int force) {
     __shared__ unsigned long long acc[1024];
+    if (table_pointless(stat, S, force)) { if (threadIdx.x == 0) *count = ~0ull; return; }   // no table: report it full
     unsigned long long s0 = 0;
     for (size_t i = threadIdx.x; i < n; i += 1024) s0 += partial[i];
     acc[threadIdx.x] = s0;
@@ -332,7 +373,7 @@ bound_cols_kernel(const float* __restrict__ xl, const float* __restrict__ xu, co
 
 size_t bound_cols_workspace(int B, int CO, int CI) {
     const int S = tiles_b(B), Mp = mpad_of(CO), NCH = CI / kChunk;
-    return align256((size_t)S * 4 * CI * 4) + (size_t)S * 2 * Mp * 4 + 256 + align256((size_t)S * NCH * Mp * 4) +
+    return align256((size_t)S * 4 * CI * 4) + (size_t)S * 2 * Mp * 4 + 8 + 256 + align256((size_t)S * NCH * Mp * 4) +
            align256((size_t)(Mp / 64) * kLowSlices * 4 * 4);
 }
 
@@ -343,15 +384,16 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
     const Carve c = carve(ws, B, CO, CI);
     const int S = tiles_b(B), Mp = mpad_of(CO), NCH = CI / kChunk;
     int rc;
-    if ((rc = fill_zero(c.low, (size_t)S * 2 * Mp, st))) return rc;
-    hipLaunchKernelGGL(col_range_kernel, dim3((CI + 63) / 64, S), dim3(256), 0, st, xl, xu, B, CI, c.xr);
+    const int force = density >= 1.f ? 1 : 0;
+    if ((rc = fill_zero(c.low, (size_t)S * 2 * Mp + 2, st))) return rc;   // the lower bounds and the two sums behind them
+    hipLaunchKernelGGL(col_range_kernel, dim3((CI + 63) / 64, S), dim3(256), 0, st, xl, xu, w, B, CO, CI, c.xr, c.stat);
     if ((rc = check_launch("col_range_kernel"))) return rc;
     const int slices = NCH < kLowSlices ? NCH : kLowSlices;
-    hipLaunchKernelGGL(col_table_kernel<true>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial);
+    hipLaunchKernelGGL(col_table_kernel<true>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial, c.stat, force);
     if ((rc = check_launch("col_table_kernel<low>"))) return rc;
-    hipLaunchKernelGGL(col_table_kernel<false>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial);
+    hipLaunchKernelGGL(col_table_kernel<false>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial, c.stat, force);
     if ((rc = check_launch("col_table_kernel<bits>"))) return rc;
-    hipLaunchKernelGGL(sum_marks_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count);
+    hipLaunchKernelGGL(sum_marks_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count, c.stat, S, force);
     if ((rc = check_launch("sum_marks_kernel"))) return rc;
     const double all = (double)S * CO * CI;
     *gate = c.count;
