@@ -68,7 +68,7 @@ const char* sd_last_forward_kernel(void);
 int sd_set_lp_candidate_density(float density);
 /* The same for sd_bound_inf_dist_forward_nograd on dense single-group layers (CI a multiple of 32): a kernel that works
  * from a table of the inputs that can hold the maximum of a weight row over a tile of 128 batch rows, and the kernel
- * that evaluates every term; both give the same bits.  Built-in limit 0.22.  No reference counterpart
+ * that evaluates every term; both give the same bits.  Built-in limit 0.26.  No reference counterpart
  * (core/cuda/bound_inf_dist_cuda.cu evaluates every term). */
 int sd_set_bound_candidate_density(float density);
 

@@ -12,7 +12,8 @@ using namespace sd;
 static float g_bound_density = -1.f;
 // measured at B = 512, M = N = 5120: the table kernel takes 0.14 + 3.3 x share ms (140 us of staging, then about 75 SIMD
 // cycles per marked (tile, weight row, input)) and the table 0.08 ms, against 1.04 ms for every term
-constexpr float kBoundColsCap = 0.22f;
+// (the table is paid for by the time the choice is made: the limit sits where 0.14 + 3.3 x share meets 1.04)
+constexpr float kBoundColsCap = 0.26f;
 
 // One work-item per (row, chunk): the 32 keep bits of the factored mask for inputs
 // chunk*32 .. chunk*32+31 of an x row (stream 1) or a w row (stream 2).

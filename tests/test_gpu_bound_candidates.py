@@ -93,3 +93,23 @@ def test_bound_candidate_density_argument(density):
     with pytest.raises(RuntimeError):
         _lib.set_bound_candidate_density(1.5)
     density(0.3)
+
+
+def test_bound_candidate_kernel_long_slices(density):
+    """Enough output tiles that the input range is not cut (B = 2048, CO = 4096) and more than 64 chunks of inputs
+    (CI = 2112): the table kernel stages its mark words in two segments.  Same bits as the every-term kernel."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, CI, CO = 2048, 2112, 4096
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(1, CI, 1, generator=g) * 0.5 + torch.randn(B, CI, 1, generator=g) * 0.01
+    r = torch.rand(B, CI, 1, generator=g) * 0.02
+    xl, xu = (x - r).contiguous().to(dev), (x + r).contiguous().to(dev)
+    w = (torch.randn(CO, CI, generator=g) * 0.3).to(dev)
+    out = {}
+    for dens in (0.0, 1.0):
+        density(dens)
+        yl, yu = torch.empty(B, CO, 1, device=dev), torch.empty(B, CO, 1, device=dev)
+        ext.bound_inf_dist_forward_nograd(xl, xu, w, yl, yu, 1)
+        out[dens] = (yl, yu)
+    assert torch.equal(out[0.0][0], out[1.0][0]) and torch.equal(out[0.0][1], out[1.0][1])

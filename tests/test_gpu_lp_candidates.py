@@ -123,3 +123,29 @@ def test_candidate_kernels_config3_size(oracle, density):
     ext.norm_dist_backward_input(gd[:rows].contiguous(), xd[:rows].contiguous(), wd, yd, gx4, 1, p)
     tol = 1e-6 * p
     np.testing.assert_allclose(gx4.cpu().numpy(), rgx, rtol=tol, atol=tol * float(np.abs(rgx).max()))
+
+
+def test_candidate_kernels_long_slices(density):
+    """Enough output tiles that the forward does not cut its input range (B = 2048, CO = 4096) and more than 64
+    chunks of inputs (CI = 2112): the forward table kernel stages its mark words in two segments.  Against the
+    every-term kernels (held to the oracle elsewhere)."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, CI, CO, p = 2048, 2112, 4096, 64.0
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(B, CI, 1, generator=g).to(dev)
+    w = (torch.randn(CO, CI, generator=g) * 0.02).to(dev)
+    gy = torch.randn(B, CO, 1, generator=g).to(dev)
+    y, grads = {}, {}
+    for dens in (0.0, 1.0):
+        density(dens)
+        y[dens] = torch.empty(B, CO, 1, device=dev)
+        ext.norm_dist_forward(x, w, y[dens], 1, p)
+    np.testing.assert_allclose(y[1.0].cpu().numpy(), y[0.0].cpu().numpy(), rtol=RTOL)
+    for dens in (0.0, 1.0):
+        density(dens)
+        gx, gw = torch.empty_like(x), torch.empty_like(w)
+        ext.norm_dist_backward_input_weight(gy, x, w, y[0.0], gx, gw, 1, p)
+        grads[dens] = (gx.cpu().numpy(), gw.cpu().numpy())
+    for a, b in zip(grads[1.0], grads[0.0]):
+        np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-4 * float(np.abs(b).max()))
