@@ -16,24 +16,43 @@ inline int tiles_b(int B) { return (B + kTileB - 1) / kTileB; }
 inline int mpad_of(int M) { return (M + kTileW - 1) / kTileW * kTileW; }
 
 struct Carve {
-    float* xr;        // [S][4][N]  per tile and input: min l, max l, min u, max u over the tile's rows (repaired)
-    float* low;       // [S][2][Mp] lower bounds of the upper / lower result of every output of (tile, weight row)
+    float* xr;        // [S][4][N]  per batch tile and input: min l, max l, min u, max u over the tile's rows (repaired)
+    float* wr;        // [T][2][N]  per weight tile and input: min w, max w over the tile's rows
+    float* low;       // [S][2][Mp] (or [T][2][Bp]) lower bounds of the upper / lower result of every output of the table's rows
     float* stat;      // two sums of col_range_kernel's probe, directly behind `low` (one fill clears both)
-    unsigned long long* count;   // marks in the table
-    uint32_t* bits;   // [S][NCH][Mp] bit i of word (s, c, m) = input 32 c + i may hold a maximum of weight row m in tile s
+    unsigned long long* count;   // [0] marks of the per-weight-row table, [1] of the per-batch-row table, [2] every-term kernel's turn
+    uint32_t* bits;   // [S][NCH][Mp] (or [T][NCH][Bp]): bit i of a word = input 32 c + i may hold a maximum of that row in that tile
     uint32_t* partial;   // marks per wavefront of the table kernel
 };
 
+inline int bpad_of(int B) { return (B + kTileB - 1) / kTileB * kTileB; }
+inline size_t maxz(size_t a, size_t b) { return a > b ? a : b; }
+
+size_t carve_sizes(int B, int M, int N, size_t (&sz)[6]) {
+    const size_t S = tiles_b(B), Mp = mpad_of(M), Bp = bpad_of(B), T = Mp / kTileW, NCH = N / kChunk;
+    sz[0] = align256(S * 4 * N * 4);                               // xr
+    sz[1] = align256(T * 2 * N * 4);                               // wr
+    sz[2] = align256(maxz(S * 2 * Mp, T * 2 * Bp) * 4 + 8);        // low + stat
+    sz[3] = 256;                                                   // count
+    sz[4] = align256(maxz(S * NCH * Mp, T * NCH * Bp) * 4);        // bits
+    sz[5] = align256(maxz(Mp / 64, Bp / 64 * ((T + 3) / 4)) * kLowSlices * 4 * 4);   // partial
+    return sz[0] + sz[1] + sz[2] + sz[3] + sz[4] + sz[5];
+}
+
 Carve carve(void* ws, int B, int M, int N) {
-    const int S = tiles_b(B), Mp = mpad_of(M), NCH = N / kChunk;
+    size_t sz[6];
+    carve_sizes(B, M, N, sz);
+    const size_t S = tiles_b(B), Mp = mpad_of(M), Bp = bpad_of(B), T = Mp / kTileW;
     char* p = static_cast<char*>(ws);
     Carve c;
-    c.xr = reinterpret_cast<float*>(p); p += align256((size_t)S * 4 * N * 4);
-    c.low = reinterpret_cast<float*>(p); p += (size_t)S * 2 * Mp * 4;   // Mp is a multiple of 128: stays 8-byte aligned
-    c.stat = reinterpret_cast<float*>(p); p += 8;
-    c.count = reinterpret_cast<unsigned long long*>(p); p += 256;
-    c.bits = reinterpret_cast<uint32_t*>(p); p += align256((size_t)S * NCH * Mp * 4);
-    c.partial = reinterpret_cast<uint32_t*>(p); p += align256((size_t)(Mp / 64) * kLowSlices * 4 * 4);
+    c.xr = reinterpret_cast<float*>(p); p += sz[0];
+    c.wr = reinterpret_cast<float*>(p); p += sz[1];
+    c.low = reinterpret_cast<float*>(p);
+    c.stat = c.low + maxz(S * 2 * Mp, T * 2 * Bp);
+    p += sz[2];
+    c.count = reinterpret_cast<unsigned long long*>(p); p += sz[3];
+    c.bits = reinterpret_cast<uint32_t*>(p); p += sz[4];
+    c.partial = reinterpret_cast<uint32_t*>(p);
     return c;
 }
 
@@ -102,11 +121,13 @@ __global__ void __launch_bounds__(256) col_range_kernel(const float* __restrict_
     }
 }
 
-// the batch rows of a tile differ by more than kProbeRatio times what 16 entries of a weight column do: every input
-// would be marked (images against small weights: ratio 15; the bounds of hidden layers: below 1)
+// The batch rows of a tile differ by more than kProbeRatio times what 16 entries of a weight column do (images
+// against small weights: ratio 15; the bounds of hidden layers: below 1): a table per weight row would mark every
+// input, because it is the batch row that decides where the maximum sits.  Then the table is built the other way
+// round, per batch row and tile of 128 weight rows (row_* kernels below); otherwise per weight row (col_*).
 constexpr float kProbeRatio = 2.5f;
-__device__ __forceinline__ bool table_pointless(const float* stat, int S, int force) {
-    return !force && stat[0] > kProbeRatio * (float)S * stat[1];
+__device__ __forceinline__ bool rows_decide(const float* stat, int S) {
+    return stat[0] > kProbeRatio * (float)S * stat[1];
 }
 
 // The two table kernels share their tiling: a workgroup takes 64 weight rows (one per lane) and a slice of the
@@ -121,8 +142,8 @@ template <bool LOW>
 __global__ void __launch_bounds__(256) col_table_kernel(const float* __restrict__ w, const float* __restrict__ xr,
                                                         int M, int N, int S, int Mp, float* __restrict__ low,
                                                         uint32_t* __restrict__ bits, uint32_t* __restrict__ partial,
-                                                        const float* __restrict__ stat, int force) {
-    if (table_pointless(stat, S, force)) return;   // the probe of col_range_kernel: the table would mark everything
+                                                        const float* __restrict__ stat) {
+    if (rows_decide(stat, S)) return;   // the probe of col_range_kernel: this table would mark everything
     // row stride 36 words: 16-byte rows, and the 128-bit reads of 16 consecutive lanes fall on disjoint banks
     __shared__ __attribute__((aligned(16))) float wt[64][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float xs[4][4][kChunk];   // column ranges of the four batch tiles of this pass, current chunk
@@ -211,9 +232,9 @@ __global__ void __launch_bounds__(256) col_table_kernel(const float* __restrict_
 
 __global__ void __launch_bounds__(1024) sum_marks_kernel(const uint32_t* __restrict__ partial, size_t n,
                                                          unsigned long long* __restrict__ count,
-                                                         const float* __restrict__ stat, int S, int force) {
+                                                         const float* __restrict__ stat, int S) {
     __shared__ unsigned long long acc[1024];
-    if (table_pointless(stat, S, force)) { if (threadIdx.x == 0) *count = ~0ull; return; }   // no table: report it full
+    if (rows_decide(stat, S)) { if (threadIdx.x == 0) *count = ~0ull; return; }   // no table: report it full
     unsigned long long s0 = 0;
     for (size_t i = threadIdx.x; i < n; i += 1024) s0 += partial[i];
     acc[threadIdx.x] = s0;
@@ -369,12 +390,279 @@ bound_cols_kernel(const float* __restrict__ xl, const float* __restrict__ xu, co
     }
 }
 
+// ---- the other orientation: tables per batch row and tile of 128 weight rows ----------------------
+// Over a tile of 128 weight rows the terms of (b, n) are bracketed by the column minimum and maximum of the weights.
+// Same three steps with the roles exchanged: ranges of W per (tile, input), lower bounds of the results per
+// (tile, batch row), marks per (tile, chunk, batch row).  All of them return at once unless rows_decide().
+__global__ void __launch_bounds__(256) row_range_kernel(const float* __restrict__ w, int M, int N, int S,
+                                                        float* __restrict__ wr, const float* __restrict__ stat) {
+    if (!rows_decide(stat, S)) return;
+    __shared__ float part[4][2][64];
+    const int nl = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int n = blockIdx.x * 64 + nl, t = blockIdx.y;
+    const int r0 = t * kTileW + grp * (kTileW / 4);
+    const int r1 = r0 + kTileW / 4 < M ? r0 + kTileW / 4 : M;
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    if (n < N) {
+        #pragma unroll 4
+        for (int m = r0; m < r1; m++) { const float v = w[(size_t)m * N + n]; lo = fminf(lo, v); hi = fmaxf(hi, v); }
+    }
+    part[grp][0][nl] = lo; part[grp][1][nl] = hi;
+    __syncthreads();
+    if (grp == 0 && n < N) {
+        #pragma unroll
+        for (int g = 1; g < 4; g++) { lo = fminf(lo, part[g][0][nl]); hi = fmaxf(hi, part[g][1][nl]); }
+        wr[(size_t)(t * 2) * N + n] = lo;
+        wr[(size_t)(t * 2 + 1) * N + n] = hi;
+    }
+}
+
+// a workgroup takes 64 batch rows (one per lane; l and u through LDS, repaired) and a slice of the inputs; wavefront
+// v works on weight tile 4 blockIdx.z + v, whose column ranges are LDS broadcasts
+template <bool LOW>
+__global__ void __launch_bounds__(256) row_table_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
+                                                        const float* __restrict__ wr, int B, int N, int T, int Bp, int S,
+                                                        float* __restrict__ low, uint32_t* __restrict__ bits,
+                                                        uint32_t* __restrict__ partial, const float* __restrict__ stat) {
+    if (!rows_decide(stat, S)) return;
+    __shared__ __attribute__((aligned(16))) float lt[64][kChunk + 4];
+    __shared__ __attribute__((aligned(16))) float ut[64][kChunk + 4];
+    __shared__ __attribute__((aligned(16))) float ws[4][2][kChunk];   // min w, max w of the four weight tiles of this pass
+    const int tid = threadIdx.x, r = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int b0 = blockIdx.x * 64, NCH = N / kChunk;
+    const int per = (NCH + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int c_lo = blockIdx.y * per, c_hi = c_lo + per < NCH ? c_lo + per : NCH;
+    const int lrow = tid >> 2, q = tid & 3;
+    const int bload = b0 + lrow < B ? b0 + lrow : B - 1;
+    const bool valid = b0 + r < B;
+    const int xt = tid >> 6, xk = (tid >> 5) & 1, xn = tid & 31;   // this work-item's value of ws
+    int marks = 0;
+    {
+        const int tb = blockIdx.z * 4;
+        const int t = tb + wave;
+        const bool active = t < T;
+        float LU = kEps, LL = kEps;
+        if (!LOW && active) {
+            LU = fmaxf(kEps, low[(size_t)(t * 2) * Bp + b0 + r]);
+            LL = fmaxf(kEps, low[(size_t)(t * 2 + 1) * Bp + b0 + r]);
+        }
+        float4 la, lb, ua, ub;
+        float px;
+        const float* wsrc = wr + ((size_t)(tb + xt < T ? tb + xt : T - 1) * 2 + xk) * N + xn;
+        auto fetch = [&](int c) {
+            const int cc = c < c_hi ? c : c_hi - 1;
+            const size_t off = (size_t)bload * N + cc * kChunk + 8 * q;
+            la = *reinterpret_cast<const float4*>(xl + off); lb = *reinterpret_cast<const float4*>(xl + off + 4);
+            ua = *reinterpret_cast<const float4*>(xu + off); ub = *reinterpret_cast<const float4*>(xu + off + 4);
+            px = wsrc[cc * kChunk];
+        };
+        if (c_lo < c_hi) fetch(c_lo);
+        for (int c = c_lo; c < c_hi; c++) {
+            {
+                float4 a = la, b = lb, d = ua, e = ub;
+                repair(a.x, d.x); repair(a.y, d.y); repair(a.z, d.z); repair(a.w, d.w);
+                repair(b.x, e.x); repair(b.y, e.y); repair(b.z, e.z); repair(b.w, e.w);
+                *reinterpret_cast<float4*>(&lt[lrow][8 * q]) = a; *reinterpret_cast<float4*>(&lt[lrow][8 * q + 4]) = b;
+                *reinterpret_cast<float4*>(&ut[lrow][8 * q]) = d; *reinterpret_cast<float4*>(&ut[lrow][8 * q + 4]) = e;
+                ws[xt][xk][xn] = px;
+            }
+            fetch(c + 1);
+            __syncthreads();
+            if (active) {
+                uint32_t word = 0;
+                #pragma unroll
+                for (int n4 = 0; n4 < kChunk; n4 += 4) {
+                    const float4 l4 = *reinterpret_cast<const float4*>(&lt[r][n4]);
+                    const float4 u4 = *reinterpret_cast<const float4*>(&ut[r][n4]);
+                    const float4 a4 = *reinterpret_cast<const float4*>(&ws[wave][0][n4]);   // min w
+                    const float4 b4 = *reinterpret_cast<const float4*>(&ws[wave][1][n4]);   // max w
+                    const float l[4] = {l4.x, l4.y, l4.z, l4.w}, u[4] = {u4.x, u4.y, u4.z, u4.w};
+                    const float wmin[4] = {a4.x, a4.y, a4.z, a4.w}, wmax[4] = {b4.x, b4.y, b4.z, b4.w};
+                    #pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        if (LOW) {
+                            LU = fmaxf(fmaxf(LU, wmin[k] - l[k]), u[k] - wmax[k]);
+                            LL = fmaxf(fmaxf(LL, l[k] - wmax[k]), wmin[k] - u[k]);
+                        } else {
+                            const float capU = fmaxf(wmax[k] - l[k], u[k] - wmin[k]);
+                            const float capL = fmaxf(l[k] - wmin[k], wmax[k] - u[k]);
+                            word |= (uint32_t)(capU >= LU || capL >= LL) << (n4 + k);
+                        }
+                    }
+                }
+                if (!LOW) {
+                    if (!valid) word = 0u;
+                    bits[((size_t)t * NCH + c) * Bp + b0 + r] = word;
+                    marks += __builtin_popcount(word);
+                }
+            }
+            __syncthreads();
+        }
+        if (LOW && active && valid) {
+            atomicMax(reinterpret_cast<int*>(low + (size_t)(t * 2) * Bp + b0 + r), __float_as_int(LU));
+            atomicMax(reinterpret_cast<int*>(low + (size_t)(t * 2 + 1) * Bp + b0 + r), __float_as_int(LL));
+        }
+    }
+    if (!LOW) {
+        #pragma unroll
+        for (int o = 32; o; o >>= 1) marks += __shfl_xor(marks, o);
+        if (r == 0)
+            partial[(((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 4 + wave] = (uint32_t)marks;
+    }
+}
+
+// count[1] = marks of the row table (full when it was not built); count[2] = 1 when neither table kernel will run,
+// which is what the every-term kernel waits for
+__global__ void __launch_bounds__(1024) sum_rows_kernel(const uint32_t* __restrict__ partial, size_t n,
+                                                        unsigned long long* __restrict__ count,
+                                                        const float* __restrict__ stat, int S,
+                                                        unsigned long long limit_col, unsigned long long limit_row) {
+    __shared__ unsigned long long acc[1024];
+    unsigned long long s0 = 0;
+    const bool built = rows_decide(stat, S);
+    if (built) for (size_t i = threadIdx.x; i < n; i += 1024) s0 += partial[i];
+    acc[threadIdx.x] = s0;
+    __syncthreads();
+    for (int o = 512; o; o >>= 1) {
+        if ((int)threadIdx.x < o) acc[threadIdx.x] += acc[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const unsigned long long rows = built ? acc[0] : ~0ull;
+        count[1] = rows;
+        count[2] = (count[0] > limit_col && rows > limit_row) ? 1ull : 0ull;
+    }
+}
+
+// Main kernel of this orientation: the kernel above with the roles exchanged.  Lane l holds the weight rows l and
+// l + 64 of the tile ((w, w') of an input as one 8-byte word), wavefront v the batch rows 8 v .. 8 v + 7, whose
+// (l, u) of an input are one 8-byte broadcast; the results are written along the weight rows as they are.
+__global__ void __launch_bounds__(1024, 1)
+bound_rows_kernel(const float* __restrict__ xl, const float* __restrict__ xu, const float* __restrict__ w,
+                  const uint32_t* __restrict__ bits, const unsigned long long* __restrict__ count,
+                  unsigned long long limit, int B, int Bp, int M, int N, int nsplit, float* __restrict__ yL,
+                  float* __restrict__ yU) {
+    constexpr int TR = 8;
+    constexpr int WROW = 2 * 64 + 4;      // floats per input in the weight tile: 64 lanes x (w, w')
+    constexpr int XROW = 2 * kTileB + 4;  // floats per input in the l/u tile: 128 batch rows x (l, u)
+    constexpr int kTileFloats = kChunk * (XROW + WROW);
+    if (gate_closed(count, limit, 0)) return;
+    __shared__ __attribute__((aligned(16))) float smem[2 * kTileFloats];
+    __shared__ __attribute__((aligned(16))) uint32_t wb[kSegChunks * kTileB];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int TM = (M + kTileW - 1) / kTileW, SB = Bp / kTileB, NCH = N / kChunk;
+    const int bt = blockIdx.x % SB, t = (blockIdx.x / SB) % TM, split = blockIdx.x / (TM * SB);
+    const int m0 = t * kTileW, b0 = bt * kTileB;
+    const int per = (NCH + nsplit - 1) / nsplit;
+    const int c_lo = split * per, c_hi = c_lo + per < NCH ? c_lo + per : NCH;
+    auto xt = [&](int buf) { return smem + buf * kTileFloats; };
+    auto wt = [&](int buf) { return smem + buf * kTileFloats + kChunk * XROW; };
+
+    float lo[TR][2], hi[TR][2];
+    #pragma unroll
+    for (int r = 0; r < TR; r++) { lo[r][0] = lo[r][1] = -kEps; hi[r][0] = hi[r][1] = kEps; }
+
+    // word of (chunk c, batch row b0 + i): bw[c * Bp + i]; rows past the batch, up to the padded count, hold zero
+    const uint32_t* __restrict__ bw = bits + (size_t)t * NCH * Bp + b0;
+    int seg_lo = c_lo;
+    auto marked = [&](int c) {
+        const uint32_t* q = wb + (c - seg_lo) * kTileB;
+        return __builtin_amdgcn_ballot_w64((q[lane] | q[lane + 64]) != 0u) != 0ull;
+    };
+    const int frow = tid >> 3, fq = tid & 7;
+    const int fb = b0 + frow < B ? b0 + frow : B - 1, fm = m0 + frow < M ? m0 + frow : M - 1;
+    auto fetch = [&](int c, bool need, float4& l4, float4& u4, float4& w4) {
+        const size_t off = (size_t)c * kChunk + 4 * fq;
+        l4 = *reinterpret_cast<const float4*>(need ? xl + (size_t)fb * N + off : xl);
+        u4 = *reinterpret_cast<const float4*>(need ? xu + (size_t)fb * N + off : xu);
+        w4 = *reinterpret_cast<const float4*>(need ? w + (size_t)fm * N + off : w);
+    };
+    auto stash = [&](int buf, float4 l4, float4 u4, const float4& w4) {
+        repair(l4.x, u4.x); repair(l4.y, u4.y); repair(l4.z, u4.z); repair(l4.w, u4.w);
+        float* dx = xt(buf) + (4 * fq) * XROW + 2 * frow;
+        *reinterpret_cast<float2*>(dx) = make_float2(l4.x, u4.x);
+        *reinterpret_cast<float2*>(dx + XROW) = make_float2(l4.y, u4.y);
+        *reinterpret_cast<float2*>(dx + 2 * XROW) = make_float2(l4.z, u4.z);
+        *reinterpret_cast<float2*>(dx + 3 * XROW) = make_float2(l4.w, u4.w);
+        // weight row frow belongs to lane frow % 64, slot frow / 64
+        float* dw = wt(buf) + (4 * fq) * WROW + 2 * (frow & 63) + (frow >> 6);
+        dw[0] = w4.x; dw[WROW] = w4.y; dw[2 * WROW] = w4.z; dw[3 * WROW] = w4.w;
+    };
+    auto compute = [&](int buf, int c) {
+        const float* X = xt(buf) + 2 * (wave * TR), *W = wt(buf) + 2 * lane;
+        const uint4* rowwords = reinterpret_cast<const uint4*>(wb + (c - seg_lo) * kTileB + wave * TR);
+        const uint4 q0 = rowwords[0], q1 = rowwords[1];
+        const uint32_t words[TR] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        #pragma unroll
+        for (int r = 0; r < TR; r++) {
+            uint32_t bm = __builtin_amdgcn_readfirstlane(words[r]);
+            while (bm) {
+                const int n = __builtin_ctz(bm);
+                bm &= bm - 1;
+                const float2 ww = *reinterpret_cast<const float2*>(W + n * WROW);        // the lane's two weights
+                const float2 lu = *reinterpret_cast<const float2*>(X + n * XROW + 2 * r);   // l, u of the row
+                const float a1 = ww.x - lu.x, a2 = lu.y - ww.x, b1 = ww.y - lu.x, b2 = lu.y - ww.y;
+                lo[r][0] = fminf(fminf(lo[r][0], a1), a2);
+                hi[r][0] = fmaxf(fmaxf(hi[r][0], a1), a2);
+                lo[r][1] = fminf(fminf(lo[r][1], b1), b2);
+                hi[r][1] = fmaxf(fmaxf(hi[r][1], b1), b2);
+            }
+        }
+    };
+
+    for (; seg_lo < c_hi; seg_lo += kSegChunks) {
+        const int seg_hi = seg_lo + kSegChunks < c_hi ? seg_lo + kSegChunks : c_hi;
+        __syncthreads();
+        for (int e = tid; e < (seg_hi - seg_lo) * kTileB; e += 1024)
+            wb[e] = bw[(size_t)(seg_lo + (e >> 7)) * Bp + (e & (kTileB - 1))];
+        __syncthreads();
+        float4 la, ua, wa, lb, ub, wc;
+        bool n0 = marked(seg_lo), n1 = seg_lo + 1 < seg_hi ? marked(seg_lo + 1) : false;
+        fetch(seg_lo, n0, la, ua, wa);
+        fetch(seg_lo + 1 < seg_hi ? seg_lo + 1 : seg_lo, n1, lb, ub, wc);
+        if (n0) stash(0, la, ua, wa);
+        __syncthreads();
+        for (int c = seg_lo; c < seg_hi; c += 2) {
+            const bool n2 = c + 2 < seg_hi ? marked(c + 2) : false;
+            fetch(c + 2 < seg_hi ? c + 2 : c, n2, la, ua, wa);
+            if (n0) compute(0, c);
+            if (n1) stash(1, lb, ub, wc);
+            __syncthreads();
+            if (c + 1 >= seg_hi) break;
+            const bool n3 = c + 3 < seg_hi ? marked(c + 3) : false;
+            fetch(c + 3 < seg_hi ? c + 3 : c, n3, lb, ub, wc);
+            if (n1) compute(1, c + 1);
+            if (n2) stash(0, la, ua, wa);
+            __syncthreads();
+            n0 = n2; n1 = n3;
+        }
+    }
+
+    #pragma unroll
+    for (int r = 0; r < TR; r++) {
+        const int row = b0 + wave * TR + r;
+        #pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int col = m0 + lane + 64 * j;
+            if (row < B && col < M) {
+                const size_t o = (size_t)row * M + col;
+                // both results are >= 1e-10 > 0, so their bit patterns order like integers
+                if (nsplit > 1) {
+                    atomicMax(reinterpret_cast<int*>(yL + o), __float_as_int(-lo[r][j]));
+                    atomicMax(reinterpret_cast<int*>(yU + o), __float_as_int(hi[r][j]));
+                } else { yL[o] = -lo[r][j]; yU[o] = hi[r][j]; }
+            }
+        }
+    }
+}
+
 }  // namespace
 
 size_t bound_cols_workspace(int B, int CO, int CI) {
-    const int S = tiles_b(B), Mp = mpad_of(CO), NCH = CI / kChunk;
-    return align256((size_t)S * 4 * CI * 4) + (size_t)S * 2 * Mp * 4 + 8 + 256 + align256((size_t)S * NCH * Mp * 4) +
-           align256((size_t)(Mp / 64) * kLowSlices * 4 * 4);
+    size_t sz[6];
+    return carve_sizes(B, CO, CI, sz);
 }
 
 int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float* outL,
@@ -382,32 +670,47 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
                        unsigned long long* gate_limit, hipStream_t st) {
     if (CI % kChunk != 0 || B < 1 || CO < 1) { set_error("bound_cols_forward: shape not supported"); return SD_ERR_ARG; }
     const Carve c = carve(ws, B, CO, CI);
-    const int S = tiles_b(B), Mp = mpad_of(CO), NCH = CI / kChunk;
+    const int S = tiles_b(B), Mp = mpad_of(CO), Bp = bpad_of(B), T = Mp / kTileW, NCH = CI / kChunk;
+    const size_t lown = maxz((size_t)S * 2 * Mp, (size_t)T * 2 * Bp);
     int rc;
-    const int force = density >= 1.f ? 1 : 0;
-    if ((rc = fill_zero(c.low, (size_t)S * 2 * Mp + 2, st))) return rc;   // the lower bounds and the two sums behind them
+    if ((rc = fill_zero(c.low, lown + 2, st))) return rc;   // the lower bounds and the two sums behind them
     hipLaunchKernelGGL(col_range_kernel, dim3((CI + 63) / 64, S), dim3(256), 0, st, xl, xu, w, B, CO, CI, c.xr, c.stat);
     if ((rc = check_launch("col_range_kernel"))) return rc;
     const int slices = NCH < kLowSlices ? NCH : kLowSlices;
-    hipLaunchKernelGGL(col_table_kernel<true>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial, c.stat, force);
+    const float d = density < 0.f ? 0.f : density > 1.f ? 1.f : density;
+    const unsigned long long limit_col = (unsigned long long)((double)S * CO * CI * d);
+    const unsigned long long limit_row = (unsigned long long)((double)T * B * CI * d);
+    // per weight row (batch rows alike)
+    hipLaunchKernelGGL(col_table_kernel<true>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial, c.stat);
     if ((rc = check_launch("col_table_kernel<low>"))) return rc;
-    hipLaunchKernelGGL(col_table_kernel<false>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial, c.stat, force);
+    hipLaunchKernelGGL(col_table_kernel<false>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial, c.stat);
     if ((rc = check_launch("col_table_kernel<bits>"))) return rc;
-    hipLaunchKernelGGL(sum_marks_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count, c.stat, S, force);
+    hipLaunchKernelGGL(sum_marks_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count, c.stat, S);
     if ((rc = check_launch("sum_marks_kernel"))) return rc;
-    const double all = (double)S * CO * CI;
-    *gate = c.count;
-    *gate_limit = (unsigned long long)(all * (density < 0.f ? 0.f : density > 1.f ? 1.f : density));
-    // a few workgroups per compute unit over the run: the work of a workgroup follows the marks of its weight rows
-    const int TM = Mp / kTileW;
-    const long long wgs = (long long)TM * S;
+    // per batch row (the batch rows decide)
+    hipLaunchKernelGGL(row_range_kernel, dim3((CI + 63) / 64, T), dim3(256), 0, st, w, CO, CI, S, c.wr, c.stat);
+    if ((rc = check_launch("row_range_kernel"))) return rc;
+    hipLaunchKernelGGL(row_table_kernel<true>, dim3(Bp / 64, slices, (T + 3) / 4), dim3(256), 0, st, xl, xu, c.wr, B, CI, T, Bp, S, c.low, c.bits, c.partial, c.stat);
+    if ((rc = check_launch("row_table_kernel<low>"))) return rc;
+    hipLaunchKernelGGL(row_table_kernel<false>, dim3(Bp / 64, slices, (T + 3) / 4), dim3(256), 0, st, xl, xu, c.wr, B, CI, T, Bp, S, c.low, c.bits, c.partial, c.stat);
+    if ((rc = check_launch("row_table_kernel<bits>"))) return rc;
+    hipLaunchKernelGGL(sum_rows_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Bp / 64) * slices * ((T + 3) / 4) * 4, c.count, c.stat, S, limit_col, limit_row);
+    if ((rc = check_launch("sum_rows_kernel"))) return rc;
+    // the every-term kernel runs when count[2] > 0
+    *gate = c.count + 2;
+    *gate_limit = 0ull;
+    // a few workgroups per compute unit over the run: the work of a workgroup follows the marks of its rows
+    const long long wgs = (long long)T * S;
     int nsplit = (int)((2ll * num_cus() + wgs - 1) / wgs);
     if (nsplit > NCH / 8) nsplit = NCH / 8;
     if (nsplit > 16) nsplit = 16;
     if (nsplit < 1) nsplit = 1;
     hipLaunchKernelGGL(bound_cols_kernel, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.bits, c.count,
-                       *gate_limit, B, CO, Mp, CI, nsplit, outL, outU);
-    return check_launch("bound_cols_kernel");
+                       limit_col, B, CO, Mp, CI, nsplit, outL, outU);
+    if ((rc = check_launch("bound_cols_kernel"))) return rc;
+    hipLaunchKernelGGL(bound_rows_kernel, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.bits, c.count + 1,
+                       limit_row, B, Bp, CO, CI, nsplit, outL, outU);
+    return check_launch("bound_rows_kernel");
 }
 
 }  // namespace sd

@@ -34,6 +34,8 @@ def _intervals(B, CI, kind, seed):
     g = torch.Generator().manual_seed(seed)
     if kind == "rows_alike":
         x = torch.randn(1, CI, 1, generator=g) * 0.5 + torch.randn(B, CI, 1, generator=g) * 0.01
+    elif kind == "images":
+        x = torch.rand(B, CI, 1, generator=g)
     else:
         x = torch.randn(B, CI, 1, generator=g)
     r = torch.rand(B, CI, 1, generator=g) * 0.05
@@ -53,7 +55,7 @@ def test_bound_candidate_kernel_matches_oracle(oracle, density, dens, B, CI, CO)
     from sortnet_amd import ext
     dev = _dev()
     density(dens)
-    for kind in ("rows_alike", "random", "inverted"):
+    for kind in ("rows_alike", "random", "inverted", "images"):
         for wscale in (0.02, 1.0):
             xl, xu = _intervals(B, CI, kind, B + CI)
             g = torch.Generator().manual_seed(2)
