@@ -240,8 +240,9 @@ void sdo_bound_inf_dist_forward(const float* xL, const float* xU, const float* w
                 float l = xL[xo + (size_t)n * HW], u = xU[xo + (size_t)n * HW];
                 if (l > u) l = u = (l + u) * 0.5f;
                 float t1 = wr[n] - l, t2 = u - wr[n];
-                float a = t1 < t2 ? t1 : t2, bb = t1 > t2 ? t1 : t2;
-                /* fminf/fmaxf semantics for NaN are irrelevant to the strict compares below */
+                /* min / max of the device code return the defined operand when the other is undefined
+                   (bound_inf_dist_cuda.cu:95-96, 204); an undefined result fails the strict compares below */
+                float a = fminf(t1, t2), bb = fmaxf(t1, t2);
                 uint32_t p = (uint32_t)n | (t1 <= t2 ? 0u : SDO_SIGN);
                 if (a < lo) { lo = a; pl = p; }
                 if (bb > hi) { hi = bb; pu = p; }
@@ -391,7 +392,10 @@ int sdo_bound_sort_neuron_forward(const float* xL, const float* xU, const float*
                 float l = xL[xo + (size_t)n * HW], u = xU[xo + (size_t)n * HW];
                 if (l > u) l = u = (l + u) * 0.5f;
                 float t1 = wr[n] - l, t2 = u - wr[n];
-                float a = t1 < t2 ? t1 : t2, bb = t1 > t2 ? t1 : t2;
+                /* min / max as on the device (sort_neuron.cu:280).  A term whose operands are both undefined is
+                   dropped here, while the reference's min/max insertion (:283-287) then duplicates the largest
+                   entry of the list: undefined inputs to the sort neuron are outside what this restatement pins. */
+                float a = fminf(t1, t2), bb = fmaxf(t1, t2);
                 sdo_insert(resL, dummy, K, -a, 0);
                 sdo_insert(resU, dummy, K, bb, 0);
             }

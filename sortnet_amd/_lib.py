@@ -48,6 +48,7 @@ _OTHER = {
     "sd_last_forward_kernel": ([], ctypes.c_char_p),
     "sd_set_lp_candidate_density": ([_f], _i),
     "sd_set_bound_candidate_density": ([_f], _i),
+    "sd_set_sort_candidate_density": ([_f], _i),
     "sd_rng_word": ([_u, _u, _u, _u], _u),
     "sd_mask_threshold8": ([_f], _u),
     "sd_mask_threshold16": ([_f], _u),
@@ -102,6 +103,15 @@ def set_bound_candidate_density(density):
     rc = lib.sd_set_bound_candidate_density(float(density))
     if rc != 0:
         raise RuntimeError("sd_set_bound_candidate_density failed: %s" % lib.sd_last_error().decode())
+
+
+def set_sort_candidate_density(density):
+    """Share of marked candidate-table entries up to which the dense sort neuron (values only) and its interval
+    bounds work from the table (0: never; negative: built-in limit, large layers only)."""
+    lib = load()
+    rc = lib.sd_set_sort_candidate_density(float(density))
+    if rc != 0:
+        raise RuntimeError("sd_set_sort_candidate_density failed: %s" % lib.sd_last_error().decode())
 
 
 def last_forward_kernel():

@@ -70,7 +70,7 @@ __global__ void __launch_bounds__(256) col_range_kernel(const float* __restrict_
                                                         const float* __restrict__ w, int B, int M, int N,
                                                         float* __restrict__ xr, float* __restrict__ stat) {
     // 64 inputs x 4 groups of 32 rows per workgroup, combined through LDS
-    __shared__ float part[4][4][64];
+    __shared__ float part[4][5][64];
     __shared__ float wpart[4][2][64];
     const int nl = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int n = blockIdx.x * 64 + nl, s = blockIdx.y;
@@ -78,10 +78,12 @@ __global__ void __launch_bounds__(256) col_range_kernel(const float* __restrict_
     const int r1 = r0 + kTileB / 4 < B ? r0 + kTileB / 4 : B;
     float lmin = __builtin_inff(), lmax = -__builtin_inff(), umin = __builtin_inff(), umax = -__builtin_inff();
     float wlo = __builtin_inff(), whi = -__builtin_inff();
+    float odd = 0.f;   // stays 0 while every l and u of the column is finite
     if (n < N) {
         #pragma unroll 4
         for (int r = r0; r < r1; r++) {
             float l = xl[(size_t)r * N + n], u = xu[(size_t)r * N + n];
+            odd += (l - l) + (u - u);
             repair(l, u);
             lmin = fminf(lmin, l); lmax = fmaxf(lmax, l);
             umin = fminf(umin, u); umax = fmaxf(umax, u);
@@ -95,6 +97,7 @@ __global__ void __launch_bounds__(256) col_range_kernel(const float* __restrict_
         }
     }
     part[grp][0][nl] = lmin; part[grp][1][nl] = lmax; part[grp][2][nl] = umin; part[grp][3][nl] = umax;
+    part[grp][4][nl] = odd;
     wpart[grp][0][nl] = wlo; wpart[grp][1][nl] = whi;
     __syncthreads();
     if (grp == 0) {
@@ -105,7 +108,11 @@ __global__ void __launch_bounds__(256) col_range_kernel(const float* __restrict_
                 lmin = fminf(lmin, part[g][0][nl]); lmax = fmaxf(lmax, part[g][1][nl]);
                 umin = fminf(umin, part[g][2][nl]); umax = fmaxf(umax, part[g][3][nl]);
                 wlo = fminf(wlo, wpart[g][0][nl]); whi = fmaxf(whi, wpart[g][1][nl]);
+                odd += part[g][4][nl];
             }
+            // A row whose l or u is undefined or infinite at this input drops terms the other rows keep, so nothing
+            // may be concluded from the column: its range becomes everything (no lower bound, always a candidate).
+            if (!(odd == 0.f)) { lmin = umin = -__builtin_inff(); lmax = umax = __builtin_inff(); }
             float* o = xr + (size_t)s * 4 * N + n;
             o[0] = lmin; o[N] = lmax; o[2 * (size_t)N] = umin; o[3 * (size_t)N] = umax;
             bw = fmaxf(lmax - lmin, umax - umin);
@@ -205,7 +212,7 @@ __global__ void __launch_bounds__(256) col_table_kernel(const float* __restrict_
                         } else {
                             const float capU = fmaxf(wv[k] - lmin[k], umax[k] - wv[k]);
                             const float capL = fmaxf(lmax[k] - wv[k], wv[k] - umin[k]);
-                            word |= (uint32_t)(capU >= LU || capL >= LL) << (n4 + k);
+                            word |= (uint32_t)(!(capU < LU) || !(capL < LL)) << (n4 + k);   // undefined counts as a candidate
                         }
                     }
                 }
@@ -397,21 +404,26 @@ bound_cols_kernel(const float* __restrict__ xl, const float* __restrict__ xu, co
 __global__ void __launch_bounds__(256) row_range_kernel(const float* __restrict__ w, int M, int N, int S,
                                                         float* __restrict__ wr, const float* __restrict__ stat) {
     if (!rows_decide(stat, S)) return;
-    __shared__ float part[4][2][64];
+    __shared__ float part[4][3][64];
     const int nl = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int n = blockIdx.x * 64 + nl, t = blockIdx.y;
     const int r0 = t * kTileW + grp * (kTileW / 4);
     const int r1 = r0 + kTileW / 4 < M ? r0 + kTileW / 4 : M;
-    float lo = __builtin_inff(), hi = -__builtin_inff();
+    float lo = __builtin_inff(), hi = -__builtin_inff(), odd = 0.f;
     if (n < N) {
         #pragma unroll 4
-        for (int m = r0; m < r1; m++) { const float v = w[(size_t)m * N + n]; lo = fminf(lo, v); hi = fmaxf(hi, v); }
+        for (int m = r0; m < r1; m++) {
+            const float v = w[(size_t)m * N + n];
+            lo = fminf(lo, v); hi = fmaxf(hi, v); odd += v - v;
+        }
     }
-    part[grp][0][nl] = lo; part[grp][1][nl] = hi;
+    part[grp][0][nl] = lo; part[grp][1][nl] = hi; part[grp][2][nl] = odd;
     __syncthreads();
     if (grp == 0 && n < N) {
         #pragma unroll
-        for (int g = 1; g < 4; g++) { lo = fminf(lo, part[g][0][nl]); hi = fmaxf(hi, part[g][1][nl]); }
+        for (int g = 1; g < 4; g++) { lo = fminf(lo, part[g][0][nl]); hi = fmaxf(hi, part[g][1][nl]); odd += part[g][2][nl]; }
+        // an undefined or infinite weight drops terms its neighbours keep: the column's range becomes everything
+        if (!(odd == 0.f)) { lo = -__builtin_inff(); hi = __builtin_inff(); }
         wr[(size_t)(t * 2) * N + n] = lo;
         wr[(size_t)(t * 2 + 1) * N + n] = hi;
     }
@@ -487,7 +499,7 @@ __global__ void __launch_bounds__(256) row_table_kernel(const float* __restrict_
                         } else {
                             const float capU = fmaxf(wmax[k] - l[k], u[k] - wmin[k]);
                             const float capL = fmaxf(l[k] - wmin[k], wmax[k] - u[k]);
-                            word |= (uint32_t)(capU >= LU || capL >= LL) << (n4 + k);
+                            word |= (uint32_t)(!(capU < LU) || !(capL < LL)) << (n4 + k);   // undefined counts as a candidate
                         }
                     }
                 }

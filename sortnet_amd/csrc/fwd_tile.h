@@ -818,6 +818,7 @@ __device__ __forceinline__ float geo_sum(const float (&res)[K], float q) {
 
 template <int K>
 struct SortNograd : PolicyBase {
+    static constexpr bool GATED = true;   // one of two queued for a result when FwdArgs::gate is set
     struct Acc { float res[K]; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
         #pragma unroll
@@ -886,6 +887,7 @@ __device__ __forceinline__ void key_insert(uint32_t (&key)[KP], uint32_t v) {
 
 template <int K>
 struct SortChunkKeys : PolicyBase {
+    static constexpr bool GATED = true;   // one of two queued for a result when FwdArgs::gate is set
     static constexpr int KP = K + kKeySlack;
     static constexpr int PIPE_WAVES = 2;
     static constexpr int MIN_WAVES = 2;
@@ -920,6 +922,7 @@ struct SortChunkKeys : PolicyBase {
 // the negated K most negative values of min(t1,t2), so both sides share the insertion routine.
 template <int K>
 struct BoundSort : PolicyBase {
+    static constexpr bool GATED = true;   // one of two queued for a result when FwdArgs::gate is set
     static constexpr int NX = 2;
     struct Acc { float lo[K], hi[K]; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
@@ -1105,12 +1108,16 @@ struct LpWithMax : PolicyBase {
 // relative.  Nearly every term is of that kind once p reaches ~100, and the two transcendentals of r^p are
 // the whole cost of the kernel: they are evaluated only when some lane of the wavefront holds a significant
 // term (wave-uniform branches, first for the group of four inputs, then for each of them).
+// The ratios are >= 0, where the bit patterns order like the values; an undefined ratio (an undefined input or
+// weight) has a pattern above every number, so it counts as significant and reaches the sum as in the reference.
 __device__ __forceinline__ void lp_add_significant(float& s, float r0, float r1, float r2, float r3, float p, float thr) {
-    if (__builtin_amdgcn_ballot_w64(fmaxf(fmaxf(r0, r1), fmaxf(r2, r3)) > thr) == 0ull) return;
-    if (__builtin_amdgcn_ballot_w64(r0 > thr) != 0ull) s += pow_pos<-1>(r0, p);
-    if (__builtin_amdgcn_ballot_w64(r1 > thr) != 0ull) s += pow_pos<-1>(r1, p);
-    if (__builtin_amdgcn_ballot_w64(r2 > thr) != 0ull) s += pow_pos<-1>(r2, p);
-    if (__builtin_amdgcn_ballot_w64(r3 > thr) != 0ull) s += pow_pos<-1>(r3, p);
+    const int i0 = __builtin_bit_cast(int, r0), i1 = __builtin_bit_cast(int, r1);
+    const int i2 = __builtin_bit_cast(int, r2), i3 = __builtin_bit_cast(int, r3), it = __builtin_bit_cast(int, thr);
+    if (__builtin_amdgcn_ballot_w64(max(max(i0, i1), max(i2, i3)) > it) == 0ull) return;
+    if (__builtin_amdgcn_ballot_w64(i0 > it) != 0ull) s += pow_pos<-1>(r0, p);
+    if (__builtin_amdgcn_ballot_w64(i1 > it) != 0ull) s += pow_pos<-1>(r1, p);
+    if (__builtin_amdgcn_ballot_w64(i2 > it) != 0ull) s += pow_pos<-1>(r2, p);
+    if (__builtin_amdgcn_ballot_w64(i3 > it) != 0ull) s += pow_pos<-1>(r3, p);
 }
 
 struct LpWithMaxSkip : LpWithMax<-1, false> {   // the significance test needs the ratio itself

@@ -46,15 +46,18 @@ __global__ void __launch_bounds__(256) tile_wabs_kernel(const float* __restrict_
     if (n >= N) return;
     const int m0 = t * kTileM, m1 = m0 + kTileM < M ? m0 + kTileM : M;
     float v0 = 0.f, v1 = 0.f, v2 = 0.f, v3 = 0.f;
+    float odd = 0.f;   // stays 0 while every weight of the column is finite
     int m = m0;
     for (; m + 4 <= m1; m += 4) {
-        v0 = fmaxf(v0, fabsf(w[(size_t)m * N + n]));
-        v1 = fmaxf(v1, fabsf(w[(size_t)(m + 1) * N + n]));
-        v2 = fmaxf(v2, fabsf(w[(size_t)(m + 2) * N + n]));
-        v3 = fmaxf(v3, fabsf(w[(size_t)(m + 3) * N + n]));
+        const float a = w[(size_t)m * N + n], b = w[(size_t)(m + 1) * N + n];
+        const float c = w[(size_t)(m + 2) * N + n], d = w[(size_t)(m + 3) * N + n];
+        v0 = fmaxf(v0, fabsf(a)); v1 = fmaxf(v1, fabsf(b)); v2 = fmaxf(v2, fabsf(c)); v3 = fmaxf(v3, fabsf(d));
+        odd += ((a - a) + (b - b)) + ((c - c) + (d - d));
     }
-    for (; m < m1; m++) v0 = fmaxf(v0, fabsf(w[(size_t)m * N + n]));
-    wabs[(size_t)t * N + n] = fmaxf(fmaxf(v0, v1), fmaxf(v2, v3));
+    for (; m < m1; m++) { const float a = w[(size_t)m * N + n]; v0 = fmaxf(v0, fabsf(a)); odd += a - a; }
+    // an undefined weight must reach the outputs it belongs to: the column's bound becomes undefined, which
+    // cand_bits_kernel takes for a candidate in every row
+    wabs[(size_t)t * N + n] = fmaxf(fmaxf(v0, v1), fmaxf(v2, v3)) + odd;
 }
 
 // one wavefront per (row, tile): smallest scale of the tile's outputs; RECIP also writes 1 / v for every output
@@ -117,7 +120,8 @@ __global__ void __launch_bounds__(256) cand_bits_kernel(const float* __restrict_
         const float* __restrict__ wa = wabs + (size_t)t * N + c * kChunk;
         uint32_t word = 0;
         #pragma unroll
-        for (int n = 0; n < kChunk; n++) word |= (uint32_t)((xs[r][n] + wa[n]) * kMargin > lim) << n;
+        for (int n = 0; n < kChunk; n++) word |= (uint32_t)(!((xs[r][n] + wa[n]) * kMargin <= lim)) << n;   // undefined counts
+        if (b >= B) word = 0u;
         bits[((size_t)t * NCH + c) * Bp + b] = word;
         marks += __builtin_popcount(word);
     }

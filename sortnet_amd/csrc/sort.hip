@@ -2,6 +2,7 @@
 // in the reference's instantiation table (core/cuda/sort_neuron.cu:403-534).
 #include "fwd_tile.h"
 #include "fwd_args.h"
+#include "sort_cols.h"
 
 using namespace sd;
 
@@ -30,6 +31,7 @@ template <int K, bool VALUES>
 __global__ void __launch_bounds__(256) sort_rows_kernel(FwdArgs a, const int* __restrict__ keys) {
     constexpr int KP = K + kKeySlack;
     extern __shared__ __attribute__((aligned(16))) float wrow[];
+    if (gate_closed(a.gate, a.gate_limit, a.gate_above)) return;   // one of two queued for the result
     const int c = blockIdx.x;                      // g * COg + m
     const int g = c / a.COg;
     const float* wsrc = a.w + (size_t)c * a.CIg;
@@ -125,6 +127,35 @@ static int run_two_level(FwdArgs& a, bool small, hipStream_t st) {
     return check_launch("sort_rows_kernel");
 }
 
+// Dense single-group layers: a kernel that works from per-weight-row candidate tables is queued in front of the
+// kernels that evaluate every term, and a count taken on the device decides which of the two runs (at most
+// kSortColsCap of the terms marked: the table kernel).  Negative g_sort_density: built-in limit, and only layers
+// large enough for the tables to pay; 0 never; up to 1: that share, at any size.
+static float g_sort_density = -1.f;
+constexpr float kSortColsCap = 0.10f;
+constexpr long long kSortColsMinTerms = 1ll << 24;
+
+static bool sort_cols_ok(const FwdArgs& a, int B, int CO, int CI, int G, int HW) {
+    if (g_sort_density == 0.f || G != 1 || HW != 1 || CI % kSortColsChunk != 0 || !a.fast_x || !a.fast_w) return false;
+    return g_sort_density > 0.f || (long long)B * CO * CI >= kSortColsMinTerms;
+}
+
+static int queue_sort_cols(FwdArgs& a, const float* xl, const float* xu, const float* w, int B, int CO, int CI, float q,
+                           int K, float* outL, float* outU, hipStream_t st) {
+    void* ws = workspace(sort_cols_workspace(B, CO, CI, K), st);
+    if (!ws) return SD_ERR_HIP;
+    const float cap = g_sort_density > 0.f ? g_sort_density : kSortColsCap;
+    int rc = sort_cols_forward(xl, xu, w, B, CO, CI, q, K, outL, outU, ws, cap, &a.gate, &a.gate_limit, st);
+    a.gate_above = 1;
+    return rc;
+}
+
+extern "C" int sd_set_sort_candidate_density(float density) {
+    SD_REQUIRE(density <= 1.f, "set_sort_candidate_density: %g is above 1", (double)density);
+    g_sort_density = density;
+    return SD_OK;
+}
+
 // few output tiles: 16 x 32 tiles instead of 32 x 64 (the top-K lists do not merge across a split reduction)
 static bool few_tiles(const FwdArgs& a, int BB, int BM) {
     long long tiles = (long long)((a.R + BB - 1) / BB) * ((a.COg + BM - 1) / BM) * a.G;
@@ -142,6 +173,8 @@ extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* we
     a.y0 = output; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 64);
+    if (sort_cols_ok(a, B, CO, CI, G, HW) &&
+        (rc = queue_sort_cols(a, input, nullptr, weight, B, CO, CI, q, K, nullptr, output, st))) return rc;
     switch (K) {
 #define X(k) case k: if (k <= 12 && two_level_ok(a, k)) return run_two_level<(k <= 12 ? k : 2), true>(a, small, st); \
                      return small ? launch_fwd<SortNograd<k>, 1, 2>(a, st) : launch_fwd<SortNograd<k>, 2, 4>(a, st);
@@ -184,6 +217,8 @@ extern "C" int sd_bound_sort_neuron_forward(const float* inputL, const float* in
     a.y0 = outputL; a.y1 = outputU; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 32);
+    if (sort_cols_ok(a, B, CO, CI, G, HW) &&
+        (rc = queue_sort_cols(a, inputL, inputU, weight, B, CO, CI, q, K, outputL, outputU, st))) return rc;
     switch (K) {
 #define X(k) case k: return small ? launch_fwd<BoundSort<k>, 1, 2>(a, st) : launch_fwd<BoundSort<k>, 2, 2>(a, st);
         SD_FOR_EACH_K(X)

@@ -1,0 +1,31 @@
+// Sort neuron (values only) and its interval bounds for dense single-group layers, from per-weight-row candidate
+// tables.
+//
+// Both are sums over the K largest terms of a row of terms (core/cuda/sort_neuron.cu:16-109, 216-314), so an input
+// whose term cannot reach a lower bound of the K-th largest term can be left out without changing a bit.  Over a
+// tile of 128 batch rows the terms of (m, n) are bracketed by the column minima / maxima of the inputs; when the
+// rows of a tile are alike compared with the entries of a weight row (weights of unit scale against activations
+// that a mean shift has centred), the same few dozen inputs per weight row hold the K largest terms of every batch
+// row.  A bit table (tile, weight row, 32 inputs) marks them, and a wavefront that owns a weight row and 128 batch
+// rows (two per lane) walks the row's marks, fetching one weight and one transposed row of inputs per mark.
+#pragma once
+#include "common.h"
+
+namespace sd {
+
+// inputs of one bit-table word; CI must be a multiple of it
+constexpr int kSortColsChunk = 32;
+
+// bytes of workspace sort_cols_forward needs
+size_t sort_cols_workspace(int B, int CO, int CI, int K);
+
+// Builds the table, counts its marks on the device and queues the table kernel so that it runs only when at most
+// `density` of all (tile, weight row, input) triples are marked; the caller queues the kernels that evaluate every
+// term with the opposite condition on the same counter (*gate, *gate_limit).
+//   xu != nullptr: interval form, outL / outU receive the bounds;
+//   xu == nullptr: value form on xl, outU receives the values (outL is not used).
+int sort_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float q, int K,
+                      float* outL, float* outU, void* ws, float density, const unsigned long long** gate,
+                      unsigned long long* gate_limit, hipStream_t st);
+
+}  // namespace sd

@@ -69,6 +69,44 @@ def test_bound_candidate_kernel_matches_oracle(oracle, density, dens, B, CI, CO)
             assert np.array_equal(yu.cpu().numpy(), ru), tag
 
 
+@pytest.mark.parametrize("dens", [1.0, 0.0])
+@pytest.mark.parametrize("kind", ["rows_alike", "images"])
+def test_bound_candidate_kernel_undefined_and_infinite_entries(oracle, density, dens, kind):
+    """A term with an undefined operand is dropped by the reference's strict compares (an interval with one
+    undefined end keeps the other end's term), so a row that holds NaN where its neighbours hold their maximum has
+    a smaller result than they do: the tables must not conclude anything from such a column.  Infinite ends and
+    weights likewise.  Both orientations of the table (rows alike / images) and the every-term kernel."""
+    from sortnet_amd import ext
+    dev = _dev()
+    density(dens)
+    B, CI, CO = 200, 256, 150
+    xl, xu = _intervals(B, CI, kind, 5)
+    g = torch.Generator().manual_seed(6)
+    w = (torch.randn(CO, CI, generator=g) * (0.02 if kind == "images" else 0.5)).contiguous()
+    # the column where most outputs have their maximum gets an undefined entry in a few rows
+    rl, ru = oracle.bound_inf_dist_forward(xl.numpy(), xu.numpy(), w.numpy(), 1, need_pos=False)
+    t = np.maximum(w.numpy()[None] - xl.numpy()[:, :, 0][:, None], xu.numpy()[:, :, 0][:, None] - w.numpy()[None])
+    hot = np.bincount(t.argmax(2).ravel(), minlength=CI).argsort()[::-1][:6]
+    nan, inf = float("nan"), float("inf")
+    xl[3, hot[0], 0] = nan; xu[3, hot[0], 0] = nan
+    xl[150, hot[1], 0] = nan
+    xu[77, hot[2], 0] = nan
+    xl[10, hot[3], 0] = -inf
+    xu[11, hot[4], 0] = inf
+    xl[12, hot[5], 0] = inf; xu[12, hot[5], 0] = inf
+    w[5, hot[0]] = nan
+    w[6, hot[1]] = inf
+    w[7, hot[5]] = inf
+    w[8, 17] = -inf
+    with np.errstate(invalid="ignore"):
+        rl, ru = oracle.bound_inf_dist_forward(xl.numpy(), xu.numpy(), w.numpy(), 1, need_pos=False)
+    yl = torch.full((B, CO, 1), float("nan"), device=dev)
+    yu = torch.full((B, CO, 1), float("nan"), device=dev)
+    ext.bound_inf_dist_forward_nograd(xl.to(dev), xu.to(dev), w.to(dev), yl, yu, 1)
+    assert np.array_equal(yl.cpu().numpy(), rl, equal_nan=True)
+    assert np.array_equal(yu.cpu().numpy(), ru, equal_nan=True)
+
+
 def test_bound_candidate_kernel_at_layer_size(density):
     """B = 512, N = M = 5120 with rows that are nearly alike (as the bounds of a hidden layer are): the table kernel
     and the every-term kernel give the same bits, and the built-in limit does too."""

@@ -81,6 +81,29 @@ def test_candidate_kernels_ties_and_zero_rows(oracle, density, dens):
         _check(oracle, x.contiguous(), w.contiguous(), gy, p, "dens=%g p=%g" % (dens, p))
 
 
+@pytest.mark.parametrize("dens", [1.0, 0.0])
+def test_candidate_kernels_undefined_entries_reach_their_outputs(oracle, density, dens):
+    """An undefined input makes every output of its row undefined, an undefined weight every output of its channel
+    (the reference sums all terms): the table must keep such entries as candidates whatever their size."""
+    from sortnet_amd import ext
+    dev = _dev()
+    density(dens)
+    B, CI, CO, p = 70, 256, 300, 64.0
+    x, w = _gen((B, CI, 1), 21), _gen((CO, CI), 22, 0.05)
+    x[5, 100, 0] = float("nan")
+    w[17, 3] = float("nan")
+    w[280, 200] = float("nan")
+    with np.errstate(invalid="ignore"):
+        ry = oracle.norm_dist_forward(x.numpy(), w.numpy(), p, 1)
+    assert np.isnan(ry[5]).all() and np.isnan(ry[:, 17]).all() and np.isnan(ry).sum() == CO + 2 * B - 2
+    y = torch.zeros(B, CO, 1, device=dev)
+    ext.norm_dist_forward(x.to(dev), w.to(dev), y, 1, p)
+    got = y.cpu().numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(ry))
+    ok = ~np.isnan(ry)
+    np.testing.assert_allclose(got[ok], ry[ok], rtol=RTOL)
+
+
 def test_candidate_density_argument(density):
     from sortnet_amd import _lib
     with pytest.raises(RuntimeError):

@@ -1,0 +1,125 @@
+"""GPU parity of the sort neuron (values only) and its interval bounds when they work from candidate tables (dense
+single-group layers, CI % 32 == 0).
+
+Both entry points queue a kernel that evaluates only the inputs a table marks as able to be among the K largest
+terms of a weight row, and the kernels that evaluate every term; a count taken on the device picks one.  Both must
+give the results of the oracle (core/cuda/sort_neuron.cu:16-109, 216-314 semantics; the geometric sum is taken in the
+reference's order over the same K values, so the comparison is exact): the tests force either side (density 1 / 0)
+and the built-in limit, on batches whose rows are alike against weights of unit scale (the table marks little), on
+unrelated rows (it marks nearly everything), on inverted intervals and on ties."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+@pytest.fixture
+def density():
+    from sortnet_amd import _lib
+
+    def set_(d):
+        _lib.set_sort_candidate_density(d)
+    yield set_
+    _lib.set_sort_candidate_density(-1.0)
+
+
+def _data(B, CI, CO, kind, seed):
+    g = torch.Generator().manual_seed(seed)
+    if kind == "rows_alike":
+        x = torch.randn(1, CI, 1, generator=g) * 0.3 + torch.randn(B, CI, 1, generator=g) * 0.05
+    elif kind == "images":
+        x = torch.rand(B, CI, 1, generator=g)
+    else:
+        x = torch.randn(B, CI, 1, generator=g)
+    r = torch.rand(B, CI, 1, generator=g) * 0.05
+    xl, xu = (x - r).contiguous(), (x + r).contiguous()
+    if kind == "inverted":
+        m = torch.rand(B, CI, 1, generator=g) < 0.1
+        xl, xu = torch.where(m, xu, xl).contiguous(), torch.where(m, xl, xu).contiguous()
+    w = torch.randn(CO, CI, generator=g).contiguous()
+    if kind == "ties":
+        x, w = torch.round(x * 4) / 4, torch.round(w * 4) / 4
+        xl, xu = x - 0.25, x + 0.25
+    return x.contiguous(), xl.contiguous(), xu.contiguous(), w.contiguous()
+
+
+RTOL = 1e-5
+
+
+def _run(x, xl, xu, w, q, K):
+    from sortnet_amd import ext
+    dev = _dev()
+    B, CO = x.shape[0], w.shape[0]
+    y, yl, yu = (torch.full((B, CO, 1), float("nan"), device=dev) for _ in range(3))
+    ext.sort_neuron_forward_nograd(x.to(dev), w.to(dev), y, 1, q, K)
+    ext.bound_sort_neuron_forward(xl.to(dev), xu.to(dev), w.to(dev), yl, yu, 1, q, K)
+    return y.cpu().numpy(), yl.cpu().numpy(), yu.cpu().numpy()
+
+
+def _check(oracle, density, dens, x, xl, xu, w, q, K, tag):
+    """Against the oracle at the sort neuron's bar (rel 1e-5), and bit for bit against the every-term kernels."""
+    ry = oracle.sort_neuron_forward(x.numpy(), w.numpy(), q, K, need_pos=False)
+    rl, ru = oracle.bound_sort_neuron_forward(xl.numpy(), xu.numpy(), w.numpy(), q, K)
+    density(dens)
+    got = _run(x, xl, xu, w, q, K)
+    for g, r in zip(got, (ry, rl, ru)):
+        np.testing.assert_allclose(g, r, rtol=RTOL, err_msg=tag)
+    if dens != 0.0:
+        density(0.0)
+        for g, e in zip(got, _run(x, xl, xu, w, q, K)):
+            assert np.array_equal(g, e), tag
+
+
+@pytest.mark.parametrize("dens", [1.0, 0.0, -1.0])
+@pytest.mark.parametrize("B,CI,CO", [(70, 96, 64), (33, 2048, 300), (130, 1024, 513), (1, 32, 1), (257, 320, 129),
+                                     (512, 1088, 96)])
+def test_sort_candidate_kernels_match_oracle(oracle, density, dens, B, CI, CO):
+    """Ragged batch tiles (B not a multiple of 128) and weight rows (CO not a multiple of 32 / 64 / 128), rows of
+    more than 32 chunks (several batches of marks per row), rows shorter than K."""
+    for kind in ("rows_alike", "random", "inverted", "images", "ties"):
+        for q, K in ((0.3, 10), (0.75, 4)):
+            x, xl, xu, w = _data(B, CI, CO, kind, B + CI)
+            _check(oracle, density, dens, x, xl, xu, w, q, K, "dens=%g %s K=%d" % (dens, kind, K))
+
+
+@pytest.mark.parametrize("K", [2, 3, 7, 13, 16, 25])
+def test_sort_candidate_kernels_every_k(oracle, density, K):
+    x, xl, xu, w = _data(140, 512, 100, "rows_alike", K)
+    _check(oracle, density, 1.0, x, xl, xu, w, 0.4, K, "K=%d" % K)
+
+
+def test_sort_candidate_kernels_at_layer_size(density):
+    """B = 512, N = M = 5120, unit-scale weights against rows that are nearly alike: the table kernels and the
+    every-term kernels give the same bits, and the built-in limit picks the table."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, N, M, q, K = 512, 5120, 5120, 0.75, 10
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(1, N, 1, generator=g) * 0.3 + torch.randn(B, N, 1, generator=g) * 0.1).to(dev)
+    r = 0.03 + torch.rand(B, N, 1, generator=g).to(dev) * 0.01
+    xl, xu = (x - r).contiguous(), (x + r).contiguous()
+    w = torch.randn(M, N, generator=g).contiguous().to(dev)
+    out = {}
+    for dens in (0.0, 1.0, -1.0):
+        density(dens)
+        y, yl, yu = (torch.empty(B, M, 1, device=dev) for _ in range(3))
+        ext.sort_neuron_forward_nograd(x.contiguous(), w, y, 1, q, K)
+        ext.bound_sort_neuron_forward(xl, xu, w, yl, yu, 1, q, K)
+        out[dens] = (y, yl, yu)
+    for dens in (1.0, -1.0):
+        for a, b in zip(out[dens], out[0.0]):
+            assert torch.equal(a, b), dens
+
+
+def test_sort_candidate_density_argument(density):
+    from sortnet_amd import _lib
+    with pytest.raises(RuntimeError):
+        _lib.set_sort_candidate_density(1.5)
+    density(0.3)
