@@ -65,7 +65,7 @@ __device__ __forceinline__ void repair(float& l, float& u) {
 // Also answers whether the table is worth building: it can only prune when the rows of a batch tile are alike
 // compared with the entries of a weight row.  stat[0] collects the widths of the column ranges of l and u over all
 // tiles and columns, stat[1] the ranges of the same columns over the first 16 weight rows (added once, by the
-// workgroups of tile 0); see table_pointless().
+// workgroups of tile 0); see rows_decide().
 __global__ void __launch_bounds__(256) col_range_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
                                                         const float* __restrict__ w, int B, int M, int N,
                                                         float* __restrict__ xr, float* __restrict__ stat) {

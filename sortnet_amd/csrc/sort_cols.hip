@@ -34,6 +34,7 @@ struct Carve {
     uint32_t* bits;   // [S][Mp][NCH] bit i of a word = input 32 c + i may be among the K largest of that row in that tile
     uint32_t* partial;   // marks per wavefront of the table kernel
     unsigned long long* count;
+    float* stat;      // two sums of sc_range_kernel's probe, 16 bytes behind the count (one fill clears all of it)
 };
 
 size_t carve_sizes(int B, int M, int N, int K, size_t (&sz)[7]) {
@@ -62,6 +63,7 @@ Carve carve(void* ws, int B, int M, int N, int K) {
     c.bits = reinterpret_cast<uint32_t*>(p); p += sz[4];
     c.partial = reinterpret_cast<uint32_t*>(p); p += sz[5];
     c.count = reinterpret_cast<unsigned long long*>(p);
+    c.stat = reinterpret_cast<float*>(p + 16);
     return c;
 }
 
@@ -96,11 +98,17 @@ __device__ __forceinline__ float geo_sum_bits(const int (&res)[K], float q) {
 // ---- tables ----------------------------------------------------------------------------------
 // Column ranges of a tile of 128 batch rows x 64 inputs, and the transposed copy of the tile the main kernel reads
 // (one row of 128 values per input).  Value form: l = u = x.
+// Also answers whether the table is worth building: it can only prune when the rows of a batch tile are alike
+// compared with the entries of a weight row.  stat[0] collects the widths of the column ranges over all tiles and
+// columns, stat[1] the ranges of the same columns over the first 16 weight rows (added once, by the workgroups of
+// tile 0); see table_pointless().
 template <bool IV>
 __global__ void __launch_bounds__(256) sc_range_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
-                                                       int B, int N, int Bp, float* __restrict__ xr,
-                                                       float* __restrict__ xT) {
+                                                       const float* __restrict__ w, int B, int M, int N, int Bp,
+                                                       float* __restrict__ xr, float* __restrict__ xT,
+                                                       float* __restrict__ stat) {
     __shared__ float part[4][5][64];
+    __shared__ float wpart[4][2][64];
     __shared__ float tl[64][kTileB + 1];
     __shared__ float tu[IV ? 64 : 1][kTileB + 1];
     const int tid = threadIdx.x, nl = tid & 63, grp = tid >> 6;
@@ -122,21 +130,44 @@ __global__ void __launch_bounds__(256) sc_range_kernel(const float* __restrict__
         tl[nl][col] = l;
         if (IV) tu[nl][col] = u;
     }
+    // the probe: ranges of the same columns over the first 16 weight rows (tile 0 only)
+    float wlo = __builtin_inff(), whi = -__builtin_inff();
+    if (s == 0 && n < N) {
+        #pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int m = grp * 4 + k;
+            if (m < M) { const float v = w[(size_t)m * N + n]; wlo = fminf(wlo, v); whi = fmaxf(whi, v); }
+        }
+    }
     part[grp][0][nl] = lmin; part[grp][1][nl] = lmax; part[grp][2][nl] = umin; part[grp][3][nl] = umax;
     part[grp][4][nl] = odd;
+    wpart[grp][0][nl] = wlo; wpart[grp][1][nl] = whi;
     __syncthreads();
-    if (grp == 0 && n < N) {
-        #pragma unroll
-        for (int g = 1; g < 4; g++) {
-            lmin = fminf(lmin, part[g][0][nl]); lmax = fmaxf(lmax, part[g][1][nl]);
-            umin = fminf(umin, part[g][2][nl]); umax = fmaxf(umax, part[g][3][nl]);
-            odd += part[g][4][nl];
+    if (grp == 0) {
+        float bw = 0.f, ww = 0.f;
+        if (n < N) {
+            #pragma unroll
+            for (int g = 1; g < 4; g++) {
+                lmin = fminf(lmin, part[g][0][nl]); lmax = fmaxf(lmax, part[g][1][nl]);
+                umin = fminf(umin, part[g][2][nl]); umax = fmaxf(umax, part[g][3][nl]);
+                wlo = fminf(wlo, wpart[g][0][nl]); whi = fmaxf(whi, wpart[g][1][nl]);
+                odd += part[g][4][nl];
+            }
+            // A row whose value is undefined or infinite at this input drops terms the other rows keep, so nothing
+            // may be concluded from the column: its range becomes everything (no lower bound, always a candidate).
+            if (!(odd == 0.f)) { lmin = umin = -__builtin_inff(); lmax = umax = __builtin_inff(); }
+            float* o = xr + (size_t)s * 4 * N + n;
+            o[0] = lmin; o[N] = lmax; o[2 * (size_t)N] = umin; o[3 * (size_t)N] = umax;
+            bw = fmaxf(lmax - lmin, umax - umin);
+            if (s == 0) ww = whi - wlo;
+            if (!(bw < 3.0e38f)) bw = 3.0e38f;   // infinite or undefined widths count as very wide
         }
-        // A row whose value is undefined or infinite at this input drops terms the other rows keep, so nothing may
-        // be concluded from the column: its range becomes everything (no lower bound, always a candidate).
-        if (!(odd == 0.f)) { lmin = umin = -__builtin_inff(); lmax = umax = __builtin_inff(); }
-        float* o = xr + (size_t)s * 4 * N + n;
-        o[0] = lmin; o[N] = lmax; o[2 * (size_t)N] = umin; o[3 * (size_t)N] = umax;
+        #pragma unroll
+        for (int o = 32; o; o >>= 1) { bw += __shfl_xor(bw, o); ww += __shfl_xor(ww, o); }
+        if (nl == 0) {
+            unsafeAtomicAdd(stat, bw);
+            if (s == 0) unsafeAtomicAdd(stat + 1, ww);
+        }
     }
     for (int e = tid; e < 64 * kTileB; e += 256) {
         const int nn = e >> 7, col = e & (kTileB - 1);
@@ -148,6 +179,13 @@ __global__ void __launch_bounds__(256) sc_range_kernel(const float* __restrict__
     }
 }
 
+// The batch rows of a tile differ by more than kProbeRatio times what 16 entries of a weight column do (images
+// against small weights): the table would mark nearly every input, so it is not built and reported as full.
+constexpr float kProbeRatio = 2.5f;
+__device__ __forceinline__ bool table_pointless(const float* stat, int S) {
+    return stat[0] > kProbeRatio * (float)S * stat[1];
+}
+
 // The two table kernels share their tiling: a workgroup takes 64 weight rows (one per lane) and a slice of the
 // inputs; wavefront v works on batch tile v (+ 4, + 8, ...), for which the column ranges are wave-uniform (LDS
 // broadcasts); the weights go through LDS, 64 x 32 at a time, so that a lane can own a row.
@@ -157,7 +195,9 @@ __global__ void __launch_bounds__(256) sc_range_kernel(const float* __restrict__
 // (one insertion per 32 inputs), whose K-th largest over all slices bounds the K-th largest term.
 template <int K, bool IV>
 __global__ void __launch_bounds__(256) sc_low_kernel(const float* __restrict__ w, const float* __restrict__ xr,
-                                                     int M, int N, int S, int Mp, float* __restrict__ lists) {
+                                                     int M, int N, int S, int Mp, float* __restrict__ lists,
+                                                     const float* __restrict__ stat) {
+    if (table_pointless(stat, S)) return;
     __shared__ __attribute__((aligned(16))) float wt[64][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float xs[4][4][kChunk];
     const int tid = threadIdx.x, r = tid & 63;
@@ -230,7 +270,8 @@ __global__ void __launch_bounds__(256) sc_low_kernel(const float* __restrict__ w
 // K-th largest of the slices' lists (0 when fewer than K lower bounds are positive)
 template <int K>
 __global__ void __launch_bounds__(256) sc_merge_kernel(const float* __restrict__ lists, int slices, int Mp, int nw,
-                                                       float* __restrict__ low) {
+                                                       float* __restrict__ low, const float* __restrict__ stat) {
+    if (table_pointless(stat, gridDim.y / nw)) return;
     const int m = blockIdx.x * 256 + threadIdx.x;
     if (m >= Mp) return;
     const int s = blockIdx.y / nw, which = blockIdx.y % nw;
@@ -252,7 +293,9 @@ __global__ void __launch_bounds__(256) sc_merge_kernel(const float* __restrict__
 template <bool IV>
 __global__ void __launch_bounds__(256) sc_bits_kernel(const float* __restrict__ w, const float* __restrict__ xr,
                                                       const float* __restrict__ low, int M, int N, int S, int Mp,
-                                                      uint32_t* __restrict__ bits, uint32_t* __restrict__ partial) {
+                                                      uint32_t* __restrict__ bits, uint32_t* __restrict__ partial,
+                                                      const float* __restrict__ stat) {
+    if (table_pointless(stat, S)) return;
     __shared__ __attribute__((aligned(16))) float wt[64][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float xs[4][4][kChunk];
     __shared__ uint32_t wd[4][64][kMaxPer + 1];
@@ -332,7 +375,9 @@ __global__ void __launch_bounds__(256) sc_bits_kernel(const float* __restrict__ 
 }
 
 __global__ void __launch_bounds__(1024) sc_sum_kernel(const uint32_t* __restrict__ partial, size_t n,
-                                                      unsigned long long* __restrict__ count) {
+                                                      unsigned long long* __restrict__ count,
+                                                      const float* __restrict__ stat, int S) {
+    if (table_pointless(stat, S)) { if (threadIdx.x == 0) *count = ~0ull; return; }   // no table: report it full
     __shared__ unsigned long long acc[1024];
     unsigned long long s0 = 0;
     for (size_t i = threadIdx.x; i < n; i += 1024) s0 += partial[i];
@@ -481,16 +526,17 @@ int run(const float* xl, const float* xu, const float* w, int B, int M, int N, f
         const Carve& c, unsigned long long limit, hipStream_t st) {
     const int S = tiles_b(B), Bp = S * kTileB, Mp = mpad_of(M), NCH = N / kChunk, slices = slices_of(NCH);
     int rc;
-    hipLaunchKernelGGL((sc_range_kernel<IV>), dim3((N + 63) / 64, S), dim3(256), 0, st, xl, xu, B, N, Bp, c.xr, c.xT);
+    if ((rc = fill_zero(c.count, 8, st))) return rc;   // the count and the two sums of the probe behind it
+    hipLaunchKernelGGL((sc_range_kernel<IV>), dim3((N + 63) / 64, S), dim3(256), 0, st, xl, xu, w, B, M, N, Bp, c.xr, c.xT, c.stat);
     if ((rc = check_launch("sc_range_kernel"))) return rc;
-    hipLaunchKernelGGL((sc_low_kernel<K, IV>), dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, M, N, S, Mp, c.lists);
+    hipLaunchKernelGGL((sc_low_kernel<K, IV>), dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, M, N, S, Mp, c.lists, c.stat);
     if ((rc = check_launch("sc_low_kernel"))) return rc;
     const int nw = IV ? 2 : 1;
-    hipLaunchKernelGGL((sc_merge_kernel<K>), dim3((Mp + 255) / 256, S * nw), dim3(256), 0, st, c.lists, slices, Mp, nw, c.low);
+    hipLaunchKernelGGL((sc_merge_kernel<K>), dim3((Mp + 255) / 256, S * nw), dim3(256), 0, st, c.lists, slices, Mp, nw, c.low, c.stat);
     if ((rc = check_launch("sc_merge_kernel"))) return rc;
-    hipLaunchKernelGGL((sc_bits_kernel<IV>), dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, c.low, M, N, S, Mp, c.bits, c.partial);
+    hipLaunchKernelGGL((sc_bits_kernel<IV>), dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, c.low, M, N, S, Mp, c.bits, c.partial, c.stat);
     if ((rc = check_launch("sc_bits_kernel"))) return rc;
-    hipLaunchKernelGGL(sc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count);
+    hipLaunchKernelGGL(sc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count, c.stat, S);
     if ((rc = check_launch("sc_sum_kernel"))) return rc;
     hipLaunchKernelGGL((sc_main_kernel<K, IV>), dim3((unsigned)(S * (Mp / kMainTile))), dim3(64 * kMainWaves), 0, st,
                        c.xT, w, c.bits, c.count, limit, B, Bp, M, Mp, N, q, outL, outU);

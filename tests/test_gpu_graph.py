@@ -184,8 +184,8 @@ def test_graph_replays_of_the_lds_direct_kernels():
 
 
 def test_graph_replays_of_the_candidate_table_kernels(oracle):
-    """Dense l-p calls at general p queue a candidate-table kernel and an every-term kernel for the same result and
-    a count taken on the device picks one, so ONE captured graph serves both kinds of data: replays on weights far
+    """Dense l-p calls at general p (and the interval forward, the sort neuron and its interval bounds) queue a
+    candidate-table kernel and an every-term kernel for the same result and a count taken on the device picks one, so ONE captured graph serves both kinds of data: replays on weights far
     smaller than the inputs (the table kernel runs) and on weights as large as the inputs (the every-term kernels
     run) must both reproduce eager calls, and the oracle."""
     from sortnet_amd import ext
@@ -196,11 +196,16 @@ def test_graph_replays_of_the_candidate_table_kernels(oracle):
 
     def outputs():
         return dict(y=torch.empty(B, CO, 1, device=dev), gx=torch.empty_like(x), gw=torch.empty_like(w),
-                    gx2=torch.empty_like(x), yl=torch.empty(B, CO, 1, device=dev), yu=torch.empty(B, CO, 1, device=dev))
+                    gx2=torch.empty_like(x), yl=torch.empty(B, CO, 1, device=dev), yu=torch.empty(B, CO, 1, device=dev),
+                    ys=torch.empty(B, CO, 1, device=dev), ysl=torch.empty(B, CO, 1, device=dev),
+                    ysu=torch.empty(B, CO, 1, device=dev))
 
     def run(o):
         # the interval forward makes the same kind of choice (rows of the batch alike or not)
         ext.bound_inf_dist_forward_nograd(x - 0.03, x + 0.03, w, o["yl"], o["yu"], 1)
+        # so do the sort neuron and its interval bounds
+        ext.sort_neuron_forward_nograd(x, w, o["ys"], 1, 0.5, 6)
+        ext.bound_sort_neuron_forward(x - 0.03, x + 0.03, w, o["ysl"], o["ysu"], 1, 0.5, 6)
         ext.norm_dist_forward(x, w, o["y"], 1, p)
         ext.norm_dist_backward_input_weight(gy, x, w, o["y"], o["gx"], o["gw"], 1, p)
         ext.norm_dist_backward_input(gy, x, w, o["y"], o["gx2"], 1, p)
@@ -230,13 +235,18 @@ def test_graph_replays_of_the_candidate_table_kernels(oracle):
         graph.replay()
         torch.cuda.synchronize()
         for name in eager:
-            if name in ("yl", "yu"):
+            if name in ("yl", "yu", "ys", "ysl", "ysu"):
                 assert torch.equal(captured[name], eager[name]), "%s, replay %d" % (name, replay)
                 continue
             a, b = captured[name].cpu().numpy(), eager[name].cpu().numpy()
             np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-4 * float(np.abs(b).max()), err_msg="%s, replay %d" % (name, replay))
         rl, ru = oracle.bound_inf_dist_forward((x - 0.03).cpu().numpy(), (x + 0.03).cpu().numpy(), w.cpu().numpy(), 1, need_pos=False)
         assert np.array_equal(captured["yl"].cpu().numpy(), rl) and np.array_equal(captured["yu"].cpu().numpy(), ru), replay
+        rs = oracle.sort_neuron_forward(x.cpu().numpy(), w.cpu().numpy(), 0.5, 6, need_pos=False)
+        np.testing.assert_allclose(captured["ys"].cpu().numpy(), rs, rtol=1e-5, err_msg="replay %d" % replay)
+        rsl, rsu = oracle.bound_sort_neuron_forward((x - 0.03).cpu().numpy(), (x + 0.03).cpu().numpy(), w.cpu().numpy(), 0.5, 6)
+        np.testing.assert_allclose(captured["ysl"].cpu().numpy(), rsl, rtol=1e-5, err_msg="replay %d" % replay)
+        np.testing.assert_allclose(captured["ysu"].cpu().numpy(), rsu, rtol=1e-5, err_msg="replay %d" % replay)
         ry = oracle.norm_dist_forward(x.cpu().numpy(), w.cpu().numpy(), p, 1)
         np.testing.assert_allclose(captured["y"].cpu().numpy(), ry, rtol=1e-5, err_msg="replay %d" % replay)
         rgx, rgw = oracle.norm_dist_backward(gy.cpu().numpy(), x.cpu().numpy(), w.cpu().numpy(), ry, p, 1)
