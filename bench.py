@@ -52,6 +52,9 @@ def parse():
                          "pass (sort neuron and interval sort neuron), without roofline / cpu_baseline")
     ap.add_argument("--p", type=float, default=float("inf"),
                     help="index-lists workload: norm of the distance layers during training (the reference anneals it from 8 to 1000, then inf)")
+    ap.add_argument("--weight-std", type=float, default=None,
+                    help="standard deviation of the initial weights of the masked workload (default fan_in ** -0.5; "
+                         "the reference initialises with 1.0)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the short runs of the other formulations")
     ap.add_argument("--calib-copy", action="store_true",
@@ -168,7 +171,7 @@ def run_index_lists(args, q, p, steps, warmup, certify_runs=0):
 
 
 def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width=None, classes=None, eps=None,
-               time_ibp=False, calib_copy=False):
+               time_ibp=False, calib_copy=False, weight_std=None):
     """K timed steps of the fused-mask formulation; returns timings, phase split and the per-launch events of the
     interval-bound forward of the width x width layers."""
     import torch
@@ -182,7 +185,8 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     mode = ext.MASK_TERM if mask == "term" else ext.MASK_FACTORED
-    model = DistanceMLP(in_features, width, args.depth, classes, q=q, device=dev, seed=0, mask_mode=mode)
+    model = DistanceMLP(in_features, width, args.depth, classes, q=q, device=dev, seed=0, mask_mode=mode,
+                        weight_std=weight_std)
     opt = torch.optim.AdamW(model.parameters(), lr=1e-4, fused=True)
     g = torch.Generator().manual_seed(0)
     x = torch.rand(batch, in_features, generator=g).to(dev)
@@ -299,11 +303,12 @@ def committed_traffic():
 
 def workload_text(args, mask, q):
     return ("SortNet-MLP training step: %d->%s->%d distance layers, B=%d, q=%.2f (%s), "
-            "forward+hinge loss+backward+AdamW+interval bounds eps=%.4f"
+            "forward+hinge loss+backward+AdamW+interval bounds eps=%.4f, weights ~ N(0, %s)"
             % (args.in_features, "x".join([str(args.width)] * (args.depth - 1)), args.classes, args.batch, q,
                "no mask: pure l-inf net" if q >= 1.0 else
                ("independent Bernoulli draw per term" if mask == "term" else
-                "factored mask keep_x(b,n)&keep_w(m,n), each output a max over a Bernoulli(q) subset"), args.eps))
+                "factored mask keep_x(b,n)&keep_w(m,n), each output a max over a Bernoulli(q) subset"), args.eps,
+               "1/fan_in" if args.weight_std is None else "%g^2" % args.weight_std))
 
 
 def run_lp_layer(args, p, steps, warmup):
@@ -356,7 +361,8 @@ def main():
             "config": {"workload": r["workload"]}, "certification_ms": r["certification_ms"]}))
         return
 
-    head = run_masked(args, args.mask, args.q, args.steps, args.warmup, time_ibp=True, calib_copy=args.calib_copy)
+    head = run_masked(args, args.mask, args.q, args.steps, args.warmup, time_ibp=True, calib_copy=args.calib_copy,
+                      weight_std=args.weight_std)
     step_s = head["ms_per_step"] * 1e-3
     step_flops = head["terms_per_step"] * (2 + 6)         # forward 2 flops/term, interval bounds 6 flops/term
     layer_terms = args.batch * args.width * args.width
@@ -411,6 +417,10 @@ def main():
         other = "term" if args.mask == "factored" else "factored"
         sec[other + "_mask"] = dict(masked_entry(other, args.q), workload=workload_text(args, other, args.q))
         sec["q1"] = dict(masked_entry(args.mask, 1.0), workload=workload_text(args, args.mask, 1.0))
+        # the same step from the reference's own initialisation (weights of unit scale, core/models/norm_dist.py:30)
+        sec["unit_weights"] = dict(masked_entry(args.mask, args.q, weight_std=1.0),
+                                   workload=workload_text(args, args.mask, args.q).replace("N(0, 1/fan_in)", "N(0, 1)")
+                                   + " as the reference initialises them")
         # the reference's own training form at the keep probability of its published commands (0.7-0.85)
         r = run_index_lists(args, 0.75, float("inf"), short, warm, certify_runs=3)
         sec["index_lists_q0.75_inf"] = {k: r[k] for k in ("ms_per_step", "samples_per_s", "steps", "workload")}

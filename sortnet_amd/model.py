@@ -17,12 +17,14 @@ from .losses import hinge_loss  # noqa: F401  (the benchmark's loss)
 
 class DistanceMLP:
     def __init__(self, in_features, width, depth, num_classes, q=0.3, device="cuda", seed=0, mask_mode=MASK_TERM,
-                 momentum=0.1):
+                 momentum=0.1, weight_std=None):
+        """weight_std: standard deviation of the initial weights; None = fan_in ** -0.5 (the scale the benchmark
+        configurations state for single layers), 1.0 = the reference's own initialisation (core/models/norm_dist.py:30)."""
         g = torch.Generator().manual_seed(seed)
         dims = [in_features] + [width] * (depth - 1) + [num_classes]
         self.weights = []
         for fan_in, fan_out in zip(dims[:-1], dims[1:]):
-            w = torch.randn(fan_out, fan_in, generator=g) * fan_in ** -0.5
+            w = torch.randn(fan_out, fan_in, generator=g) * (fan_in ** -0.5 if weight_std is None else weight_std)
             self.weights.append(w.to(device).requires_grad_())
         self.bias = torch.zeros(num_classes, device=device, requires_grad=True)
         self.running_mean = [torch.zeros(d, device=device) for d in dims[1:-1]]
