@@ -111,12 +111,14 @@ static bool two_level_ok(const FwdArgs& a, int K) {
            nchunks <= (1 << kKeyIdBits);
 }
 
+// bytes of the two-level path's key lists
+static size_t two_level_bytes(const FwdArgs& a, int K) {
+    return (size_t)(K + kKeySlack) * ((size_t)a.R * a.G * a.COg) * sizeof(int);
+}
+
+// `keys`: two_level_bytes() of workspace
 template <int K, bool VALUES>
-static int run_two_level(FwdArgs& a, bool small, hipStream_t st) {
-    constexpr int KP = K + kKeySlack;
-    const size_t total = (size_t)a.R * a.G * a.COg;
-    int* keys = static_cast<int*>(workspace((size_t)KP * total * sizeof(int), st));
-    if (!keys) return SD_ERR_HIP;
+static int run_two_level(FwdArgs& a, bool small, int* keys, hipStream_t st) {
     FwdArgs t = a;
     t.p0 = keys;
     int rc = small ? launch_fwd<SortChunkKeys<K>, 1, 2>(t, st) : launch_fwd<SortChunkKeys<K>, 2, 4>(t, st);
@@ -140,10 +142,11 @@ static bool sort_cols_ok(const FwdArgs& a, int B, int CO, int CI, int G, int HW)
     return g_sort_density > 0.f || (long long)B * CO * CI >= kSortColsMinTerms;
 }
 
+// `ws`: sort_cols_workspace() bytes.  The gate it leaves in `a` points into `ws`: the kernels queued behind it must
+// not be given memory that overlaps it, and `ws` must stay allocated until they have run (one workspace request
+// per call, carved by the caller).
 static int queue_sort_cols(FwdArgs& a, const float* xl, const float* xu, const float* w, int B, int CO, int CI, float q,
-                           int K, float* outL, float* outU, hipStream_t st) {
-    void* ws = workspace(sort_cols_workspace(B, CO, CI, K), st);
-    if (!ws) return SD_ERR_HIP;
+                           int K, float* outL, float* outU, void* ws, hipStream_t st) {
     const float cap = g_sort_density > 0.f ? g_sort_density : kSortColsCap;
     int rc = sort_cols_forward(xl, xu, w, B, CO, CI, q, K, outL, outU, ws, cap, &a.gate, &a.gate_limit, st);
     a.gate_above = 1;
@@ -173,10 +176,19 @@ extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* we
     a.y0 = output; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 64);
-    if (sort_cols_ok(a, B, CO, CI, G, HW) &&
-        (rc = queue_sort_cols(a, input, nullptr, weight, B, CO, CI, q, K, nullptr, output, st))) return rc;
+    const bool two = K <= 12 && two_level_ok(a, K), cols = sort_cols_ok(a, B, CO, CI, G, HW);
+    // one request for both users of the workspace: the tables (with the counter the gates read) first, the key
+    // lists of the two-level path behind them
+    const size_t tbytes = cols ? (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256 : 0;
+    char* base = nullptr;
+    if (cols || two) {
+        base = static_cast<char*>(workspace(tbytes + (two ? two_level_bytes(a, K) : 0), st));
+        if (!base) return SD_ERR_HIP;
+    }
+    int* keys = reinterpret_cast<int*>(base + tbytes);
+    if (cols && (rc = queue_sort_cols(a, input, nullptr, weight, B, CO, CI, q, K, nullptr, output, base, st))) return rc;
     switch (K) {
-#define X(k) case k: if (k <= 12 && two_level_ok(a, k)) return run_two_level<(k <= 12 ? k : 2), true>(a, small, st); \
+#define X(k) case k: if (k <= 12 && two) return run_two_level<(k <= 12 ? k : 2), true>(a, small, keys, st); \
                      return small ? launch_fwd<SortNograd<k>, 1, 2>(a, st) : launch_fwd<SortNograd<k>, 2, 4>(a, st);
         SD_FOR_EACH_K(X)
 #undef X
@@ -196,8 +208,14 @@ extern "C" int sd_sort_neuron_forward(const float* input, const float* weight,
     a.y0 = output; a.p0 = pos; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 32);
+    const bool two = K <= 12 && two_level_ok(a, K);
+    int* keys = nullptr;
+    if (two) {
+        keys = static_cast<int*>(workspace(two_level_bytes(a, K), st));
+        if (!keys) return SD_ERR_HIP;
+    }
     switch (K) {
-#define X(k) case k: if (k <= 12 && two_level_ok(a, k)) return run_two_level<(k <= 12 ? k : 2), false>(a, few_tiles(a, 32, 64), st); \
+#define X(k) case k: if (k <= 12 && two) return run_two_level<(k <= 12 ? k : 2), false>(a, few_tiles(a, 32, 64), keys, st); \
                      return small ? launch_fwd<SortPos<k>, 1, 2>(a, st) : launch_fwd<SortPos<k>, 2, 2>(a, st);
         SD_FOR_EACH_K(X)
 #undef X
@@ -217,8 +235,11 @@ extern "C" int sd_bound_sort_neuron_forward(const float* inputL, const float* in
     a.y0 = outputL; a.y1 = outputU; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 32);
-    if (sort_cols_ok(a, B, CO, CI, G, HW) &&
-        (rc = queue_sort_cols(a, inputL, inputU, weight, B, CO, CI, q, K, outputL, outputU, st))) return rc;
+    if (sort_cols_ok(a, B, CO, CI, G, HW)) {
+        void* ws = workspace(sort_cols_workspace(B, CO, CI, K), st);   // the only request of this call
+        if (!ws) return SD_ERR_HIP;
+        if ((rc = queue_sort_cols(a, inputL, inputU, weight, B, CO, CI, q, K, outputL, outputU, ws, st))) return rc;
+    }
     switch (K) {
 #define X(k) case k: return small ? launch_fwd<BoundSort<k>, 1, 2>(a, st) : launch_fwd<BoundSort<k>, 2, 2>(a, st);
         SD_FOR_EACH_K(X)
