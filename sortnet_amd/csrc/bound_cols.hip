@@ -146,19 +146,18 @@ __device__ __forceinline__ bool rows_decide(const float* stat, int S) {
 //   else: one table word per (tile, chunk, weight row): bit n set when the largest the term can be reaches the
 //         lower bound of the upper or of the lower result; the marks are counted.
 template <bool LOW>
-__global__ void __launch_bounds__(256) col_table_kernel(const float* __restrict__ w, const float* __restrict__ xr,
-                                                        int M, int N, int S, int Mp, float* __restrict__ low,
-                                                        uint32_t* __restrict__ bits, uint32_t* __restrict__ partial,
-                                                        const float* __restrict__ stat) {
-    if (rows_decide(stat, S)) return;   // the probe of col_range_kernel: this table would mark everything
+__device__ __forceinline__ void col_table_body(const float* __restrict__ w, const float* __restrict__ xr,
+                                               int M, int N, int S, int Mp, float* __restrict__ low,
+                                               uint32_t* __restrict__ bits, uint32_t* __restrict__ partial,
+                                               int bx, int by, int gx, int gy) {
     // row stride 36 words: 16-byte rows, and the 128-bit reads of 16 consecutive lanes fall on disjoint banks
     __shared__ __attribute__((aligned(16))) float wt[64][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float xs[4][4][kChunk];   // column ranges of the four batch tiles of this pass, current chunk
     const int tid = threadIdx.x, r = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int m0 = blockIdx.x * 64, NCH = N / kChunk;
-    const int per = (NCH + (int)gridDim.y - 1) / (int)gridDim.y;
-    const int c_lo = blockIdx.y * per, c_hi = c_lo + per < NCH ? c_lo + per : NCH;
+    const int m0 = bx * 64, NCH = N / kChunk;
+    const int per = (NCH + gy - 1) / gy;
+    const int c_lo = by * per, c_hi = c_lo + per < NCH ? c_lo + per : NCH;
     const int lrow = tid >> 2, q = tid & 3;
     const int mload = m0 + lrow < M ? m0 + lrow : M - 1;
     const bool valid = m0 + r < M;
@@ -230,27 +229,11 @@ __global__ void __launch_bounds__(256) col_table_kernel(const float* __restrict_
         }
     }
     if (!LOW) {
-        // one number per wavefront for sum_marks_kernel (atomics on one address would serialise)
+        // one number per wavefront for sum_tables_kernel (atomics on one address would serialise)
         #pragma unroll
         for (int o = 32; o; o >>= 1) marks += __shfl_xor(marks, o);
-        if (r == 0) partial[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 4 + wave] = (uint32_t)marks;
+        if (r == 0) partial[((size_t)by * gx + bx) * 4 + wave] = (uint32_t)marks;
     }
-}
-
-__global__ void __launch_bounds__(1024) sum_marks_kernel(const uint32_t* __restrict__ partial, size_t n,
-                                                         unsigned long long* __restrict__ count,
-                                                         const float* __restrict__ stat, int S) {
-    __shared__ unsigned long long acc[1024];
-    if (rows_decide(stat, S)) { if (threadIdx.x == 0) *count = ~0ull; return; }   // no table: report it full
-    unsigned long long s0 = 0;
-    for (size_t i = threadIdx.x; i < n; i += 1024) s0 += partial[i];
-    acc[threadIdx.x] = s0;
-    __syncthreads();
-    for (int o = 512; o; o >>= 1) {
-        if ((int)threadIdx.x < o) acc[threadIdx.x] += acc[threadIdx.x + o];
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) *count = acc[0];
 }
 
 // ---- main kernel --------------------------------------------------------------------------
@@ -263,19 +246,19 @@ __global__ void __launch_bounds__(1024) sum_marks_kernel(const uint32_t* __restr
 // pair costs a wavefront two LDS reads (its own word and the weight as a broadcast) and eight vector instructions,
 // the terms of the every-term kernel.  The results leave through an
 // LDS transpose (coalesced along the weight rows) and merge over the slices by atomic maximum.
-__global__ void __launch_bounds__(1024, 1)
-bound_cols_kernel(const float* __restrict__ xl, const float* __restrict__ xu, const float* __restrict__ w,
-                  const uint32_t* __restrict__ bits, const unsigned long long* __restrict__ count,
-                  unsigned long long limit, int B, int M, int Mp, int N, int nsplit, float* __restrict__ yL,
-                  float* __restrict__ yU) {
+constexpr int kMainTileFloats = kChunk * (4 * 64 + 4 + kTileW + 4);   // l/u tile + weight tile of one chunk, either orientation
+constexpr int kMainWords = kSegChunks * kTileW;
+
+__device__ __forceinline__ void bound_cols_body(const float* __restrict__ xl, const float* __restrict__ xu,
+                                                const float* __restrict__ w, const uint32_t* __restrict__ bits, int B,
+                                                int M, int Mp, int N, int nsplit, float* __restrict__ yL,
+                                                float* __restrict__ yU, float* smem, uint32_t* wb) {
     constexpr int TW = 8;
     constexpr int XROW = 4 * 64 + 4;     // floats per input in the l/u tile: 64 lanes x (l, l', u, u'), skewed by 4 banks
     constexpr int WROW = kTileW + 4;     // floats per input in the weight tile
     constexpr int kTileFloats = kChunk * (XROW + WROW);
     static_assert(2 * kTileFloats >= kTileB * (kTileW + 1), "the transpose of the results fits where the tiles were");
-    if (gate_closed(count, limit, 0)) return;
-    __shared__ __attribute__((aligned(16))) float smem[2 * kTileFloats];
-    __shared__ __attribute__((aligned(16))) uint32_t wb[kSegChunks * kTileW];
+    static_assert(kTileFloats == kMainTileFloats, "LDS of the shared kernel");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int TM = (M + kTileW - 1) / kTileW, SB = (B + kTileB - 1) / kTileB, NCH = N / kChunk;
@@ -432,26 +415,25 @@ __global__ void __launch_bounds__(256) row_range_kernel(const float* __restrict_
 // a workgroup takes 64 batch rows (one per lane; l and u through LDS, repaired) and a slice of the inputs; wavefront
 // v works on weight tile 4 blockIdx.z + v, whose column ranges are LDS broadcasts
 template <bool LOW>
-__global__ void __launch_bounds__(256) row_table_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
-                                                        const float* __restrict__ wr, int B, int N, int T, int Bp, int S,
-                                                        float* __restrict__ low, uint32_t* __restrict__ bits,
-                                                        uint32_t* __restrict__ partial, const float* __restrict__ stat) {
-    if (!rows_decide(stat, S)) return;
+__device__ __forceinline__ void row_table_body(const float* __restrict__ xl, const float* __restrict__ xu,
+                                               const float* __restrict__ wr, int B, int N, int T, int Bp,
+                                               float* __restrict__ low, uint32_t* __restrict__ bits,
+                                               uint32_t* __restrict__ partial, int bx, int by, int bz, int gx, int gy) {
     __shared__ __attribute__((aligned(16))) float lt[64][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float ut[64][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float ws[4][2][kChunk];   // min w, max w of the four weight tiles of this pass
     const int tid = threadIdx.x, r = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int b0 = blockIdx.x * 64, NCH = N / kChunk;
-    const int per = (NCH + (int)gridDim.y - 1) / (int)gridDim.y;
-    const int c_lo = blockIdx.y * per, c_hi = c_lo + per < NCH ? c_lo + per : NCH;
+    const int b0 = bx * 64, NCH = N / kChunk;
+    const int per = (NCH + gy - 1) / gy;
+    const int c_lo = by * per, c_hi = c_lo + per < NCH ? c_lo + per : NCH;
     const int lrow = tid >> 2, q = tid & 3;
     const int bload = b0 + lrow < B ? b0 + lrow : B - 1;
     const bool valid = b0 + r < B;
     const int xt = tid >> 6, xk = (tid >> 5) & 1, xn = tid & 31;   // this work-item's value of ws
     int marks = 0;
     {
-        const int tb = blockIdx.z * 4;
+        const int tb = bz * 4;
         const int t = tb + wave;
         const bool active = t < T;
         float LU = kEps, LL = kEps;
@@ -520,20 +502,42 @@ __global__ void __launch_bounds__(256) row_table_kernel(const float* __restrict_
         #pragma unroll
         for (int o = 32; o; o >>= 1) marks += __shfl_xor(marks, o);
         if (r == 0)
-            partial[(((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 4 + wave] = (uint32_t)marks;
+            partial[(((size_t)bz * gy + by) * gx + bx) * 4 + wave] = (uint32_t)marks;
     }
 }
 
-// count[1] = marks of the row table (full when it was not built); count[2] = 1 when neither table kernel will run,
-// which is what the every-term kernel waits for
-__global__ void __launch_bounds__(1024) sum_rows_kernel(const uint32_t* __restrict__ partial, size_t n,
-                                                        unsigned long long* __restrict__ count,
-                                                        const float* __restrict__ stat, int S,
-                                                        unsigned long long limit_col, unsigned long long limit_row) {
+// Both table steps as one launch each: the probe picks the orientation, and workgroups beyond the grid of that
+// orientation return at once.
+template <bool LOW>
+__global__ void __launch_bounds__(256) table_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
+                                                    const float* __restrict__ w, const float* __restrict__ xr,
+                                                    const float* __restrict__ wr, int B, int M, int N, int S, int T,
+                                                    int Mp, int Bp, int slices, float* __restrict__ low,
+                                                    uint32_t* __restrict__ bits, uint32_t* __restrict__ partial,
+                                                    const float* __restrict__ stat) {
+    const int id = blockIdx.x;
+    if (rows_decide(stat, S)) {
+        const int gx = Bp / 64, gy = slices, gz = (T + 3) / 4;
+        if (id >= gx * gy * gz) return;
+        row_table_body<LOW>(xl, xu, wr, B, N, T, Bp, low, bits, partial, id % gx, (id / gx) % gy, id / (gx * gy), gx, gy);
+    } else {
+        const int gx = Mp / 64, gy = slices;
+        if (id >= gx * gy) return;
+        col_table_body<LOW>(w, xr, M, N, S, Mp, low, bits, partial, id % gx, id / gx, gx, gy);
+    }
+}
+
+// count[0] = marks of the table per weight row, count[1] = of the table per batch row (the one that was not built
+// counts as full), count[2] = 1 when neither is below its limit, which is what the every-term kernel waits for
+__global__ void __launch_bounds__(1024) sum_tables_kernel(const uint32_t* __restrict__ partial, size_t n_col,
+                                                          size_t n_row, unsigned long long* __restrict__ count,
+                                                          const float* __restrict__ stat, int S,
+                                                          unsigned long long limit_col, unsigned long long limit_row) {
     __shared__ unsigned long long acc[1024];
+    const bool rows = rows_decide(stat, S);
+    const size_t n = rows ? n_row : n_col;
     unsigned long long s0 = 0;
-    const bool built = rows_decide(stat, S);
-    if (built) for (size_t i = threadIdx.x; i < n; i += 1024) s0 += partial[i];
+    for (size_t i = threadIdx.x; i < n; i += 1024) s0 += partial[i];
     acc[threadIdx.x] = s0;
     __syncthreads();
     for (int o = 512; o; o >>= 1) {
@@ -541,27 +545,25 @@ __global__ void __launch_bounds__(1024) sum_rows_kernel(const uint32_t* __restri
         __syncthreads();
     }
     if (threadIdx.x == 0) {
-        const unsigned long long rows = built ? acc[0] : ~0ull;
-        count[1] = rows;
-        count[2] = (count[0] > limit_col && rows > limit_row) ? 1ull : 0ull;
+        const unsigned long long c = rows ? ~0ull : acc[0], r = rows ? acc[0] : ~0ull;
+        count[0] = c;
+        count[1] = r;
+        count[2] = (c > limit_col && r > limit_row) ? 1ull : 0ull;
     }
 }
 
 // Main kernel of this orientation: the kernel above with the roles exchanged.  Lane l holds the weight rows l and
 // l + 64 of the tile ((w, w') of an input as one 8-byte word), wavefront v the batch rows 8 v .. 8 v + 7, whose
 // (l, u) of an input are one 8-byte broadcast; the results are written along the weight rows as they are.
-__global__ void __launch_bounds__(1024, 1)
-bound_rows_kernel(const float* __restrict__ xl, const float* __restrict__ xu, const float* __restrict__ w,
-                  const uint32_t* __restrict__ bits, const unsigned long long* __restrict__ count,
-                  unsigned long long limit, int B, int Bp, int M, int N, int nsplit, float* __restrict__ yL,
-                  float* __restrict__ yU) {
+__device__ __forceinline__ void bound_rows_body(const float* __restrict__ xl, const float* __restrict__ xu,
+                                                const float* __restrict__ w, const uint32_t* __restrict__ bits, int B,
+                                                int Bp, int M, int N, int nsplit, float* __restrict__ yL,
+                                                float* __restrict__ yU, float* smem, uint32_t* wb) {
     constexpr int TR = 8;
     constexpr int WROW = 2 * 64 + 4;      // floats per input in the weight tile: 64 lanes x (w, w')
     constexpr int XROW = 2 * kTileB + 4;  // floats per input in the l/u tile: 128 batch rows x (l, u)
     constexpr int kTileFloats = kChunk * (XROW + WROW);
-    if (gate_closed(count, limit, 0)) return;
-    __shared__ __attribute__((aligned(16))) float smem[2 * kTileFloats];
-    __shared__ __attribute__((aligned(16))) uint32_t wb[kSegChunks * kTileB];
+    static_assert(kTileFloats == kMainTileFloats && kSegChunks * kTileB == kMainWords, "LDS of the shared kernel");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int TM = (M + kTileW - 1) / kTileW, SB = Bp / kTileB, NCH = N / kChunk;
@@ -670,6 +672,18 @@ bound_rows_kernel(const float* __restrict__ xl, const float* __restrict__ xu, co
     }
 }
 
+// One launch for both orientations (same grid, same LDS): whichever table is below its limit is used
+__global__ void __launch_bounds__(1024, 1)
+bound_table_kernel(const float* __restrict__ xl, const float* __restrict__ xu, const float* __restrict__ w,
+                   const uint32_t* __restrict__ bits, const unsigned long long* __restrict__ count,
+                   unsigned long long limit_col, unsigned long long limit_row, int B, int Bp, int M, int Mp, int N,
+                   int nsplit, float* __restrict__ yL, float* __restrict__ yU) {
+    __shared__ __attribute__((aligned(16))) float smem[2 * kMainTileFloats];
+    __shared__ __attribute__((aligned(16))) uint32_t wb[kMainWords];
+    if (count[0] <= limit_col) bound_cols_body(xl, xu, w, bits, B, M, Mp, N, nsplit, yL, yU, smem, wb);
+    else if (count[1] <= limit_row) bound_rows_body(xl, xu, w, bits, B, Bp, M, N, nsplit, yL, yU, smem, wb);
+}
+
 }  // namespace
 
 size_t bound_cols_workspace(int B, int CO, int CI) {
@@ -692,22 +706,20 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
     const float d = density < 0.f ? 0.f : density > 1.f ? 1.f : density;
     const unsigned long long limit_col = (unsigned long long)((double)S * CO * CI * d);
     const unsigned long long limit_row = (unsigned long long)((double)T * B * CI * d);
-    // per weight row (batch rows alike)
-    hipLaunchKernelGGL(col_table_kernel<true>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial, c.stat);
-    if ((rc = check_launch("col_table_kernel<low>"))) return rc;
-    hipLaunchKernelGGL(col_table_kernel<false>, dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, CO, CI, S, Mp, c.low, c.bits, c.partial, c.stat);
-    if ((rc = check_launch("col_table_kernel<bits>"))) return rc;
-    hipLaunchKernelGGL(sum_marks_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count, c.stat, S);
-    if ((rc = check_launch("sum_marks_kernel"))) return rc;
-    // per batch row (the batch rows decide)
+    // ranges of W per tile of weight rows: only when the probe picks the tables per batch row
     hipLaunchKernelGGL(row_range_kernel, dim3((CI + 63) / 64, T), dim3(256), 0, st, w, CO, CI, S, c.wr, c.stat);
     if ((rc = check_launch("row_range_kernel"))) return rc;
-    hipLaunchKernelGGL(row_table_kernel<true>, dim3(Bp / 64, slices, (T + 3) / 4), dim3(256), 0, st, xl, xu, c.wr, B, CI, T, Bp, S, c.low, c.bits, c.partial, c.stat);
-    if ((rc = check_launch("row_table_kernel<low>"))) return rc;
-    hipLaunchKernelGGL(row_table_kernel<false>, dim3(Bp / 64, slices, (T + 3) / 4), dim3(256), 0, st, xl, xu, c.wr, B, CI, T, Bp, S, c.low, c.bits, c.partial, c.stat);
-    if ((rc = check_launch("row_table_kernel<bits>"))) return rc;
-    hipLaunchKernelGGL(sum_rows_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Bp / 64) * slices * ((T + 3) / 4) * 4, c.count, c.stat, S, limit_col, limit_row);
-    if ((rc = check_launch("sum_rows_kernel"))) return rc;
+    const int wg_col = (Mp / 64) * slices, wg_row = (Bp / 64) * slices * ((T + 3) / 4);
+    const int wg_tab = wg_col > wg_row ? wg_col : wg_row;
+    hipLaunchKernelGGL(table_kernel<true>, dim3(wg_tab), dim3(256), 0, st, xl, xu, w, c.xr, c.wr, B, CO, CI, S, T, Mp, Bp,
+                       slices, c.low, c.bits, c.partial, c.stat);
+    if ((rc = check_launch("table_kernel<low>"))) return rc;
+    hipLaunchKernelGGL(table_kernel<false>, dim3(wg_tab), dim3(256), 0, st, xl, xu, w, c.xr, c.wr, B, CO, CI, S, T, Mp, Bp,
+                       slices, c.low, c.bits, c.partial, c.stat);
+    if ((rc = check_launch("table_kernel<bits>"))) return rc;
+    hipLaunchKernelGGL(sum_tables_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)wg_col * 4, (size_t)wg_row * 4,
+                       c.count, c.stat, S, limit_col, limit_row);
+    if ((rc = check_launch("sum_tables_kernel"))) return rc;
     // the every-term kernel runs when count[2] > 0
     *gate = c.count + 2;
     *gate_limit = 0ull;
@@ -717,12 +729,9 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
     if (nsplit > NCH / 8) nsplit = NCH / 8;
     if (nsplit > 16) nsplit = 16;
     if (nsplit < 1) nsplit = 1;
-    hipLaunchKernelGGL(bound_cols_kernel, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.bits, c.count,
-                       limit_col, B, CO, Mp, CI, nsplit, outL, outU);
-    if ((rc = check_launch("bound_cols_kernel"))) return rc;
-    hipLaunchKernelGGL(bound_rows_kernel, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.bits, c.count + 1,
-                       limit_row, B, Bp, CO, CI, nsplit, outL, outU);
-    return check_launch("bound_rows_kernel");
+    hipLaunchKernelGGL(bound_table_kernel, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.bits, c.count,
+                       limit_col, limit_row, B, Bp, CO, Mp, CI, nsplit, outL, outU);
+    return check_launch("bound_table_kernel");
 }
 
 }  // namespace sd
