@@ -87,6 +87,17 @@ int num_cus();
 // Growing waits for that stream and re-allocates (bytes == 0 returns the current buffer).
 void* workspace(size_t bytes, hipStream_t stream);
 
+// Whether a call site's candidate tables have paid lately.  Calls that queue a table kernel and an every-term kernel
+// for one result let the device choose, and report afterwards which ran (hint_record: an 8-byte copy of the device's
+// flag into pinned host memory, read by a later call once its event has completed; nothing waits).  When the every-term
+// kernel ran kHintStreak times in a row for a (site, weight matrix, shape) - a layer - the next kHintSkip calls do not build tables at all
+// (hint_build_tables returns false), then one call probes again.  A performance hint only: results do not depend on
+// it.  Neither function does anything while `stream` is being captured (tables are then always built).
+constexpr int kHintStreak = 3, kHintSkip = 31;
+bool hint_build_tables(int site, const void* weight, int B, int CO, int CI, hipStream_t stream);
+void hint_record(int site, const void* weight, int B, int CO, int CI, const unsigned long long* every_term_ran,
+                 hipStream_t stream);
+
 // zero-fill n floats on `stream` with a kernel (graph-capture friendly, no memset node)
 int fill_zero(void* ptr, size_t n_words, hipStream_t stream);
 

@@ -14,6 +14,7 @@ static float g_bound_density = -1.f;
 // cycles per marked (tile, weight row, input)) and the table 0.08 ms, against 1.04 ms for every term
 // (the table is paid for by the time the choice is made: the limit sits where 0.14 + 3.3 x share meets 1.04)
 constexpr float kBoundColsCap = 0.26f;
+constexpr int kHintSiteBound = 1;
 
 // One work-item per (row, chunk): the 32 keep bits of the factored mask for inputs
 // chunk*32 .. chunk*32+31 of an x row (stream 1) or a w row (stream 2).
@@ -221,7 +222,10 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
     // dense single-group layers: a kernel that works from per-weight-row candidate tables is queued in front of the
     // one that evaluates every term, and a count taken on the device decides which of the two runs
     const float cap = g_bound_density >= 0.f ? g_bound_density : kBoundColsCap;
-    const bool cols = cap > 0.f && G == 1 && HW == 1 && CI % kColsChunk == 0 && a.fast_x && a.fast_w;
+    bool cols = cap > 0.f && G == 1 && HW == 1 && CI % kColsChunk == 0 && a.fast_x && a.fast_w;
+    // with the built-in limit, a layer whose tables have not paid lately is not given any for a while
+    const bool hinted = cols && g_bound_density < 0.f;
+    if (hinted && !hint_build_tables(kHintSiteBound, weight, B, CO, CI, st)) cols = false;
     if (a.nsplit > 1 || cols) {
         if ((rc = fill_zero(outputL, (size_t)B * CO * HW, st))) return rc;
         if ((rc = fill_zero(outputU, (size_t)B * CO * HW, st))) return rc;
@@ -232,8 +236,9 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
         if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, outputL, outputU, ws, cap, &a.gate, &a.gate_limit, st)))
             return rc;
         a.gate_above = 1;
-        if (TB == 2) return launch_fwd<BoundNogradGated, 2, 8>(a, st);
-        return launch_fwd<BoundNogradGated, 4, 8>(a, st);
+        rc = TB == 2 ? launch_fwd<BoundNogradGated, 2, 8>(a, st) : launch_fwd<BoundNogradGated, 4, 8>(a, st);
+        if (hinted && rc == SD_OK) hint_record(kHintSiteBound, weight, B, CO, CI, a.gate, st);   // the gate is 1 when every term ran
+        return rc;
     }
     if (TB == 2) return launch_fwd<BoundNograd, 2, 8>(a, st);
     return launch_fwd<BoundNograd, 4, 8>(a, st);

@@ -71,6 +71,74 @@ void* workspace(size_t bytes, hipStream_t stream) {
     return slot->buf;
 }
 
+namespace {
+struct HintSlot {
+    int dev, site, B, CO, CI;
+    const void* weight;         // the layer: same shapes with other weights are other layers
+    unsigned long long* host;   // pinned: the flag of the last recorded call
+    hipEvent_t ev;
+    bool pending;               // a copy is queued and not yet looked at
+    int streak, skip_left;
+};
+std::mutex g_hint_mu;
+std::vector<HintSlot> g_hints;
+
+bool capturing(hipStream_t stream) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) { (void)hipGetLastError(); return false; }
+    return cap != hipStreamCaptureStatusNone;
+}
+
+HintSlot* hint_slot(int site, const void* weight, int B, int CO, int CI, bool create) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    for (HintSlot& h : g_hints)
+        if (h.dev == dev && h.site == site && h.weight == weight && h.B == B && h.CO == CO && h.CI == CI) return &h;
+    if (!create || g_hints.size() >= 256) return nullptr;
+    HintSlot h{dev, site, B, CO, CI, weight, nullptr, nullptr, false, 0, 0};
+    if (hipHostMalloc(reinterpret_cast<void**>(&h.host), sizeof(unsigned long long), hipHostMallocDefault) != hipSuccess ||
+        hipEventCreateWithFlags(&h.ev, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    *h.host = 0;
+    g_hints.push_back(h);
+    return &g_hints.back();
+}
+}  // namespace
+
+bool hint_build_tables(int site, const void* weight, int B, int CO, int CI, hipStream_t stream) {
+    if (capturing(stream)) return true;
+    std::lock_guard<std::mutex> lock(g_hint_mu);
+    HintSlot* h = hint_slot(site, weight, B, CO, CI, false);
+    if (!h) return true;
+    if (h->pending) {
+        const hipError_t e = hipEventQuery(h->ev);
+        if (e == hipSuccess) {
+            h->pending = false;
+            h->streak = *h->host != 0ull ? h->streak + 1 : 0;
+        } else (void)hipGetLastError();   // not ready: look again at the next call
+    }
+    if (h->streak < kHintStreak) return true;
+    if (h->skip_left > 0) { h->skip_left--; return false; }
+    h->skip_left = kHintSkip;   // probe once, then skip again unless the tables pay now
+    return true;
+}
+
+void hint_record(int site, const void* weight, int B, int CO, int CI, const unsigned long long* every_term_ran,
+                 hipStream_t stream) {
+    if (capturing(stream)) return;
+    std::lock_guard<std::mutex> lock(g_hint_mu);
+    HintSlot* h = hint_slot(site, weight, B, CO, CI, true);
+    if (!h || h->pending) return;
+    if (hipMemcpyAsync(h->host, every_term_ran, sizeof(unsigned long long), hipMemcpyDeviceToHost, stream) != hipSuccess ||
+        hipEventRecord(h->ev, stream) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    h->pending = true;
+}
+
 __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t* __restrict__ p, size_t n) {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     size_t stride = (size_t)gridDim.x * 256;

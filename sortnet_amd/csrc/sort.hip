@@ -137,9 +137,17 @@ static float g_sort_density = -1.f;
 constexpr float kSortColsCap = 0.10f;
 constexpr long long kSortColsMinTerms = 1ll << 24;
 
-static bool sort_cols_ok(const FwdArgs& a, int B, int CO, int CI, int G, int HW) {
+// `site`: which entry point asks (with the built-in limit, a layer whose tables have not paid lately is not given
+// any for a while, see hint_build_tables)
+constexpr int kHintSiteSort = 2, kHintSiteBoundSort = 3;
+static bool sort_cols_ok(const FwdArgs& a, int site, int B, int CO, int CI, int G, int HW, hipStream_t st) {
     if (g_sort_density == 0.f || G != 1 || HW != 1 || CI % kSortColsChunk != 0 || !a.fast_x || !a.fast_w) return false;
-    return g_sort_density > 0.f || (long long)B * CO * CI >= kSortColsMinTerms;
+    if (g_sort_density > 0.f) return true;
+    return (long long)B * CO * CI >= kSortColsMinTerms && hint_build_tables(site, a.w, B, CO, CI, st);
+}
+// after the every-term kernels have been queued behind the table kernel
+static void sort_cols_report(const FwdArgs& a, int site, int B, int CO, int CI, hipStream_t st) {
+    if (g_sort_density < 0.f && a.gate) hint_record(site, a.w, B, CO, CI, a.gate + 1, st);
 }
 
 // `ws`: sort_cols_workspace() bytes.  The gate it leaves in `a` points into `ws`: the kernels queued behind it must
@@ -176,7 +184,7 @@ extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* we
     a.y0 = output; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 64);
-    const bool two = K <= 12 && two_level_ok(a, K), cols = sort_cols_ok(a, B, CO, CI, G, HW);
+    const bool two = K <= 12 && two_level_ok(a, K), cols = sort_cols_ok(a, kHintSiteSort, B, CO, CI, G, HW, st);
     // one request for both users of the workspace: the tables (with the counter the gates read) first, the key
     // lists of the two-level path behind them
     const size_t tbytes = cols ? (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256 : 0;
@@ -187,13 +195,16 @@ extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* we
     }
     int* keys = reinterpret_cast<int*>(base + tbytes);
     if (cols && (rc = queue_sort_cols(a, input, nullptr, weight, B, CO, CI, q, K, nullptr, output, base, st))) return rc;
+    rc = SD_ERR_ARG;
     switch (K) {
-#define X(k) case k: if (k <= 12 && two) return run_two_level<(k <= 12 ? k : 2), true>(a, small, keys, st); \
-                     return small ? launch_fwd<SortNograd<k>, 1, 2>(a, st) : launch_fwd<SortNograd<k>, 2, 4>(a, st);
+#define X(k) case k: if (k <= 12 && two) rc = run_two_level<(k <= 12 ? k : 2), true>(a, small, keys, st); \
+                     else rc = small ? launch_fwd<SortNograd<k>, 1, 2>(a, st) : launch_fwd<SortNograd<k>, 2, 4>(a, st); \
+                     break;
         SD_FOR_EACH_K(X)
 #undef X
     }
-    return SD_ERR_ARG;
+    if (cols && rc == SD_OK) sort_cols_report(a, kHintSiteSort, B, CO, CI, st);
+    return rc;
 }
 
 extern "C" int sd_sort_neuron_forward(const float* input, const float* weight,
@@ -235,15 +246,18 @@ extern "C" int sd_bound_sort_neuron_forward(const float* inputL, const float* in
     a.y0 = outputL; a.y1 = outputU; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 32);
-    if (sort_cols_ok(a, B, CO, CI, G, HW)) {
+    const bool cols = sort_cols_ok(a, kHintSiteBoundSort, B, CO, CI, G, HW, st);
+    if (cols) {
         void* ws = workspace(sort_cols_workspace(B, CO, CI, K), st);   // the only request of this call
         if (!ws) return SD_ERR_HIP;
         if ((rc = queue_sort_cols(a, inputL, inputU, weight, B, CO, CI, q, K, outputL, outputU, ws, st))) return rc;
     }
+    rc = SD_ERR_ARG;
     switch (K) {
-#define X(k) case k: return small ? launch_fwd<BoundSort<k>, 1, 2>(a, st) : launch_fwd<BoundSort<k>, 2, 2>(a, st);
+#define X(k) case k: rc = small ? launch_fwd<BoundSort<k>, 1, 2>(a, st) : launch_fwd<BoundSort<k>, 2, 2>(a, st); break;
         SD_FOR_EACH_K(X)
 #undef X
     }
-    return SD_ERR_ARG;
+    if (cols && rc == SD_OK) sort_cols_report(a, kHintSiteBoundSort, B, CO, CI, st);
+    return rc;
 }

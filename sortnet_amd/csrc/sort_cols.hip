@@ -34,7 +34,7 @@ struct Carve {
     uint32_t* bits;   // [S][Mp][NCH] bit i of a word = input 32 c + i may be among the K largest of that row in that tile
     uint32_t* partial;   // marks per wavefront of the table kernel
     unsigned long long* count;
-    float* stat;      // two sums of sc_range_kernel's probe, 16 bytes behind the count (one fill clears all of it)
+    float* stat;      // two sums of sc_range_kernel's probe, 16 bytes behind the count and its flag (one fill clears all of it)
 };
 
 size_t carve_sizes(int B, int M, int N, int K, size_t (&sz)[7]) {
@@ -374,10 +374,11 @@ __global__ void __launch_bounds__(256) sc_bits_kernel(const float* __restrict__ 
     if (r == 0) partial[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 4 + wave] = (uint32_t)marks;
 }
 
+// count[0] = marks (a table that was not built counts as full), count[1] = 1 when that is above the limit
 __global__ void __launch_bounds__(1024) sc_sum_kernel(const uint32_t* __restrict__ partial, size_t n,
                                                       unsigned long long* __restrict__ count,
-                                                      const float* __restrict__ stat, int S) {
-    if (table_pointless(stat, S)) { if (threadIdx.x == 0) *count = ~0ull; return; }   // no table: report it full
+                                                      const float* __restrict__ stat, int S, unsigned long long limit) {
+    if (table_pointless(stat, S)) { if (threadIdx.x == 0) { count[0] = ~0ull; count[1] = 1ull; } return; }
     __shared__ unsigned long long acc[1024];
     unsigned long long s0 = 0;
     for (size_t i = threadIdx.x; i < n; i += 1024) s0 += partial[i];
@@ -387,7 +388,7 @@ __global__ void __launch_bounds__(1024) sc_sum_kernel(const uint32_t* __restrict
         if ((int)threadIdx.x < o) acc[threadIdx.x] += acc[threadIdx.x + o];
         __syncthreads();
     }
-    if (threadIdx.x == 0) *count = acc[0];
+    if (threadIdx.x == 0) { count[0] = acc[0]; count[1] = acc[0] > limit ? 1ull : 0ull; }
 }
 
 // ---- main kernel -------------------------------------------------------------------------------
@@ -536,7 +537,7 @@ int run(const float* xl, const float* xu, const float* w, int B, int M, int N, f
     if ((rc = check_launch("sc_merge_kernel"))) return rc;
     hipLaunchKernelGGL((sc_bits_kernel<IV>), dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, c.low, M, N, S, Mp, c.bits, c.partial, c.stat);
     if ((rc = check_launch("sc_bits_kernel"))) return rc;
-    hipLaunchKernelGGL(sc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count, c.stat, S);
+    hipLaunchKernelGGL(sc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count, c.stat, S, limit);
     if ((rc = check_launch("sc_sum_kernel"))) return rc;
     hipLaunchKernelGGL((sc_main_kernel<K, IV>), dim3((unsigned)(S * (Mp / kMainTile))), dim3(64 * kMainWaves), 0, st,
                        c.xT, w, c.bits, c.count, limit, B, Bp, M, Mp, N, q, outL, outU);
