@@ -49,6 +49,8 @@ _OTHER = {
     "sd_set_lp_candidate_density": ([_f], _i),
     "sd_set_bound_candidate_density": ([_f], _i),
     "sd_set_sort_candidate_density": ([_f], _i),
+    "sd_set_linf_candidate_density": ([_f], _i),
+    "sd_set_linf_candidate_depth": ([_i], _i),
     "sd_rng_word": ([_u, _u, _u, _u], _u),
     "sd_mask_threshold8": ([_f], _u),
     "sd_mask_threshold16": ([_f], _u),
@@ -67,6 +69,8 @@ def load():
         raise RuntimeError(
             "sortnet_amd: %s not found - build the HIP library first (make -C sortnet_amd/csrc); "
             "there is no fallback path" % LIB_PATH)
+    # torch first: the library must bind the HIP runtime that torch ships and has initialised, not a second copy of it
+    import torch  # noqa: F401
     lib = ctypes.CDLL(LIB_PATH)
     for name, args in SIGNATURES.items():
         fn = getattr(lib, name)
@@ -112,6 +116,23 @@ def set_sort_candidate_density(density):
     rc = lib.sd_set_sort_candidate_density(float(density))
     if rc != 0:
         raise RuntimeError("sd_set_sort_candidate_density failed: %s" % lib.sd_last_error().decode())
+
+
+def set_linf_candidate_density(density):
+    """Share of marked candidate-table entries up to which the dense l-inf forward (plain and under the factored
+    mask) works from the table (0: never; negative: built-in limit, large layers only)."""
+    lib = load()
+    rc = lib.sd_set_linf_candidate_density(float(density))
+    if rc != 0:
+        raise RuntimeError("sd_set_linf_candidate_density failed: %s" % lib.sd_last_error().decode())
+
+
+def set_linf_candidate_depth(depth):
+    """Inputs per weight row the table's bound rests on under the factored mask (0: from the keep probability)."""
+    lib = load()
+    rc = lib.sd_set_linf_candidate_depth(int(depth))
+    if rc != 0:
+        raise RuntimeError("sd_set_linf_candidate_depth failed: %s" % lib.sd_last_error().decode())
 
 
 def last_forward_kernel():

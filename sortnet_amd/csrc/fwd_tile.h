@@ -557,6 +557,7 @@ struct PolicyBase {
 
 // l-inf forward without indices (core/cuda/inf_dist_cuda.cu:17-107)
 struct LinfNograd : PolicyBase {
+    static constexpr bool GATED = true;   // one of two queued for a result when FwdArgs::gate is set
     static constexpr bool LISTS = true;
     static constexpr bool DIRECT = true;
     static constexpr bool MASKABLE = true;
@@ -604,6 +605,7 @@ __device__ __forceinline__ void store_chunk_winner(const FwdArgs& a, size_t o, f
 }
 
 struct LinfChunk : PolicyBase {
+    static constexpr bool GATED = true;   // one of two queued for a result when FwdArgs::gate is set
     static constexpr bool LISTS = true;
     static constexpr int PIPE_WAVES = 2;   // three accumulator registers per output: 2 x 8 outputs leave no room for more
     static constexpr int MIN_WAVES = 2;
@@ -633,6 +635,7 @@ struct LinfChunk : PolicyBase {
 // inside the slice needs 8 bits (at most 254 chunks per slice; 255 = none yet), so 4 x 8 outputs cost 64 + 8
 // registers instead of 96 and fit four waves per SIMD without staging registers.
 struct LinfChunkPacked : PolicyBase {
+    static constexpr bool GATED = true;   // one of two queued for a result when FwdArgs::gate is set
     static constexpr bool DIRECT = true;
     static constexpr bool MASKABLE = true;
     static constexpr bool HAS_TSTATE = true;
@@ -1177,6 +1180,7 @@ __device__ __forceinline__ uint32_t chunk_keep_bits(const FwdArgs& a, long long 
 
 template <bool PACKED>
 __global__ void __launch_bounds__(256) resolve_pos_kernel(FwdArgs a) {
+    if (gate_closed(a.gate, a.gate_limit, a.gate_above)) return;   // one of two queued for the result
     __shared__ __attribute__((aligned(16))) ResolveSlot slots[4][64];
     const long long total = (long long)a.R * a.G * a.COg;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;

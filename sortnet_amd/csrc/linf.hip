@@ -2,6 +2,7 @@
 #include "fwd_tile.h"
 #include "fwd_args.h"
 #include "bound_cols.h"
+#include "sort_cols.h"
 #include <mutex>
 #include <type_traits>
 
@@ -15,6 +16,52 @@ static float g_bound_density = -1.f;
 // (the table is paid for by the time the choice is made: the limit sits where 0.14 + 3.3 x share meets 1.04)
 constexpr float kBoundColsCap = 0.26f;
 constexpr int kHintSiteBound = 1;
+
+// The l-inf forward (plain, and under the factored mask) on dense single-group layers queues a kernel that works from
+// per-weight-row candidate tables in front of the kernels that evaluate every term; a count taken on the device
+// decides which runs.  Negative g_linf_density: built-in limit, layers of at least kMaxColsMinTerms terms, and not
+// where the tables have not paid lately (hint_build_tables); 0 never; up to 1: that share, at any size.
+static float g_linf_density = -1.f;
+static int g_linf_depth = 0;   // under the mask: inputs the bound of a weight row rests on (0 = from the keep probability)
+constexpr float kMaxColsCap = 0.10f;
+constexpr long long kMaxColsMinTerms = 1ll << 24;
+constexpr int kHintSiteLinf = 4, kHintSiteMasked = 5;
+
+// depth of the tables' bound (0 = no tables for this call)
+static int max_cols_wanted(const FwdArgs& a, int site, float keep_x, int B, int CO, int CI, int G, int HW, hipStream_t st) {
+    if (g_linf_density == 0.f || G != 1 || HW != 1 || CI % kSortColsChunk != 0 || CI > 65536 || !a.fast_x || !a.fast_w ||
+        a.ci_idx || a.co_idx) return 0;
+    int K = max_cols_depth(keep_x);
+    if (g_linf_depth > 0 && keep_x < 1.f) K = g_linf_depth;
+    if (K == 0 || g_linf_density > 0.f) return K;
+    return ((long long)B * CO * CI >= kMaxColsMinTerms && hint_build_tables(site, a.w, B, CO, CI, st)) ? K : 0;
+}
+
+static int queue_max_cols(FwdArgs& a, int K, int B, int CO, int CI, void* ws, hipStream_t st) {
+    const float cap = g_linf_density > 0.f ? g_linf_density : kMaxColsCap;
+    // depth 1: the mask keeps everything
+    int rc = max_cols_forward(a.x0, a.w, K == 1 ? nullptr : a.xmask, K == 1 ? nullptr : a.wmask, B, CO, CI, K, a.y0, a.p0,
+                              ws, cap, &a.gate, &a.gate_limit, st);
+    a.gate_above = 1;
+    return rc;
+}
+
+static void max_cols_report(const FwdArgs& a, int site, int B, int CO, int CI, hipStream_t st) {
+    if (g_linf_density < 0.f && a.gate) hint_record(site, a.w, B, CO, CI, a.gate + 1, st);
+}
+
+extern "C" int sd_set_linf_candidate_density(float density) {
+    SD_REQUIRE(density <= 1.f, "set_linf_candidate_density: %g is above 1", (double)density);
+    g_linf_density = density;
+    return SD_OK;
+}
+
+extern "C" int sd_set_linf_candidate_depth(int depth) {
+    SD_REQUIRE(depth == 0 || depth == 8 || depth == 12 || depth == 16 || depth == 20 || depth == 24,
+               "set_linf_candidate_depth: %d is not one of 0, 8, 12, 16, 20, 24", depth);
+    g_linf_depth = depth;
+    return SD_OK;
+}
 
 // One work-item per (row, chunk): the 32 keep bits of the factored mask for inputs
 // chunk*32 .. chunk*32+31 of an x row (stream 1) or a w row (stream 2).
@@ -86,8 +133,15 @@ extern "C" int sd_inf_dist_forward_nograd(const float* input, const float* weigh
     const int TB = pick_tb(a, kTb42, 2, 128);
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;
-    if (TB == 2) return launch_fwd<LinfNograd, 2, 8>(a, st);
-    return launch_fwd<LinfNograd, 4, 8>(a, st);
+    const int K = max_cols_wanted(a, kHintSiteLinf, 1.f, B, CO, CI, G, HW, st);
+    if (K) {
+        void* ws = workspace(max_cols_workspace(B, CO, CI, K), st);   // the only request of this call
+        if (!ws) return SD_ERR_HIP;
+        if ((rc = queue_max_cols(a, K, B, CO, CI, ws, st))) return rc;
+    }
+    rc = TB == 2 ? launch_fwd<LinfNograd, 2, 8>(a, st) : launch_fwd<LinfNograd, 4, 8>(a, st);
+    if (K && rc == SD_OK) max_cols_report(a, kHintSiteLinf, B, CO, CI, st);
+    return rc;
 }
 
 extern "C" int sd_inf_dist_forward(const float* input, const float* weight,
@@ -101,7 +155,17 @@ extern "C" int sd_inf_dist_forward(const float* input, const float* weight,
     SD_REQUIRE(output && pos, "inf_dist_forward: null output or pos");
     a.y0 = output; a.p0 = pos;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    return run_chunk_pos<LinfChunk>(a, w_index_ci || w_index_co, st);
+    const int K = max_cols_wanted(a, kHintSiteLinf, 1.f, B, CO, CI, G, HW, st);
+    if (!K) return run_chunk_pos<LinfChunk>(a, w_index_ci || w_index_co, st);
+    // one workspace request for both users: the split-N merge buffer first, the tables (with the counter the gates
+    // read) behind it
+    const size_t merge = (((size_t)B * CO * 8) + 255) / 256 * 256;
+    char* base = static_cast<char*>(workspace(merge + max_cols_workspace(B, CO, CI, K), st));
+    if (!base) return SD_ERR_HIP;
+    if ((rc = queue_max_cols(a, K, B, CO, CI, base + merge, st))) return rc;
+    rc = run_chunk_pos<LinfChunk>(a, false, st, base, merge);
+    if (rc == SD_OK) max_cols_report(a, kHintSiteLinf, B, CO, CI, st);
+    return rc;
 }
 
 // ---- the entry point that allocates nothing ---------------------------------------------------
@@ -181,12 +245,18 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
     // NaN terms never win the maximum, so the plain l-inf policies apply unchanged.  On the
     // vector-load path the keep bits are built once per call into the library workspace.
     size_t packed_bytes = 0;
+    int K = 0;          // depth of the candidate tables' bound (0: no tables)
+    void* tables = nullptr;
     if (a.fast_x && a.fast_w) {
         const int nchunks = (a.CIg + KT - 1) / KT;
         const long long xrows = (long long)a.R * G, wrows = (long long)CO;
         packed_bytes = pos ? (((size_t)a.R * CO * 8 + 255) / 256) * 256 : 0;
-        char* base = static_cast<char*>(workspace(packed_bytes + (size_t)(xrows + wrows) * nchunks * 4, st));
+        // one request for every user of the workspace: merge buffer, keep bits, candidate tables
+        const size_t mask_bytes = ((size_t)(xrows + wrows) * nchunks * 4 + 255) / 256 * 256;
+        K = max_cols_wanted(a, kHintSiteMasked, (float)a.t16 / 65536.f, B, CO, CI, G, HW, st);
+        char* base = static_cast<char*>(workspace(packed_bytes + mask_bytes + (K ? max_cols_workspace(B, CO, CI, K) : 0), st));
         if (!base) return SD_ERR_HIP;
+        tables = base + packed_bytes + mask_bytes;
         uint32_t* xm = reinterpret_cast<uint32_t*>(base + packed_bytes);
         uint32_t* wm = xm + xrows * nchunks;
         hipLaunchKernelGGL(build_masks_kernel, dim3((unsigned)((xrows * nchunks + 255) / 256)), dim3(256), 0, st,
@@ -196,13 +266,20 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
         if ((rc = check_launch("build_masks_kernel"))) return rc;
         a.xmask = xm; a.wmask = wm;
     }
-    if (pos) return run_chunk_pos<LinfChunk>(a, false, st);
+    if (pos) {
+        if (K && (rc = queue_max_cols(a, K, B, CO, CI, tables, st))) return rc;
+        rc = run_chunk_pos<LinfChunk>(a, false, st);
+        if (K && rc == SD_OK) max_cols_report(a, kHintSiteMasked, B, CO, CI, st);
+        return rc;
+    }
     static const int kTb42[] = {4, 2};   // 8 rows per work-item measured slower (168 registers, three waves per SIMD)
     const int TB = pick_tb(a, kTb42, 2, 128);
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;
-    if (TB == 2) return launch_fwd<LinfNograd, 2, 8>(a, st);
-    return launch_fwd<LinfNograd, 4, 8>(a, st);
+    if (K && (rc = queue_max_cols(a, K, B, CO, CI, tables, st))) return rc;
+    rc = TB == 2 ? launch_fwd<LinfNograd, 2, 8>(a, st) : launch_fwd<LinfNograd, 4, 8>(a, st);
+    if (K && rc == SD_OK) max_cols_report(a, kHintSiteMasked, B, CO, CI, st);
+    return rc;
 }
 
 extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float* inputU, const float* weight,

@@ -117,11 +117,12 @@ bool hint_build_tables(int site, const void* weight, int B, int CO, int CI, hipS
         if (e == hipSuccess) {
             h->pending = false;
             h->streak = *h->host != 0ull ? h->streak + 1 : 0;
+            // the streak is long enough (or the probe after a stretch without tables came out the same): no tables
+            // for the next kHintSkip calls, then one call probes again
+            h->skip_left = h->streak >= kHintStreak ? kHintSkip : 0;
         } else (void)hipGetLastError();   // not ready: look again at the next call
     }
-    if (h->streak < kHintStreak) return true;
     if (h->skip_left > 0) { h->skip_left--; return false; }
-    h->skip_left = kHintSkip;   // probe once, then skip again unless the tables pay now
     return true;
 }
 

@@ -28,4 +28,14 @@ int sort_cols_forward(const float* xl, const float* xu, const float* w, int B, i
                       float* outL, float* outU, void* ws, float density, const unsigned long long** gate,
                       unsigned long long* gate_limit, hipStream_t st);
 
+// l-inf distance forward (maximum and, if pos is not null, its position) from the same kind of table, optionally
+// under the factored mask (xkeep: one word per (batch row, 32 inputs), wkeep: per (weight row, 32 inputs); both or
+// neither).  K = max_cols_depth(probability that a row keeps an input): how many inputs the bound of a weight row
+// rests on (1 without a mask; 0 = the mask keeps too little for a table).  Same contract as sort_cols_forward.
+int max_cols_depth(float keep_x);
+size_t max_cols_workspace(int B, int CO, int CI, int K);
+int max_cols_forward(const float* x, const float* w, const uint32_t* xkeep, const uint32_t* wkeep, int B, int CO, int CI,
+                     int K, float* y, int* pos, void* ws, float density, const unsigned long long** gate,
+                     unsigned long long* gate_limit, hipStream_t st);
+
 }  // namespace sd

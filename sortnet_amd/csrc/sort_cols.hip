@@ -102,11 +102,15 @@ __device__ __forceinline__ float geo_sum_bits(const int (&res)[K], float q) {
 // compared with the entries of a weight row.  stat[0] collects the widths of the column ranges over all tiles and
 // columns, stat[1] the ranges of the same columns over the first 16 weight rows (added once, by the workgroups of
 // tile 0); see table_pointless().
-template <bool IV>
+// MASKED (value form only): xkeep holds one word per (batch row, 32 inputs); an input a row does not keep takes no
+// part in the ranges and is undefined in the transposed copy, so that its term never wins a comparison.  A column no
+// row of the tile keeps has neither a lower bound nor a candidate.
+template <bool IV, bool MASKED>
 __global__ void __launch_bounds__(256) sc_range_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
-                                                       const float* __restrict__ w, int B, int M, int N, int Bp,
-                                                       float* __restrict__ xr, float* __restrict__ xT,
-                                                       float* __restrict__ stat) {
+                                                       const float* __restrict__ w, const uint32_t* __restrict__ xkeep,
+                                                       int B, int M, int N, int Bp, float* __restrict__ xr,
+                                                       float* __restrict__ xT, float* __restrict__ stat) {
+    static_assert(!(IV && MASKED), "the factored mask belongs to the value form");
     __shared__ float part[4][5][64];
     __shared__ float wpart[4][2][64];
     __shared__ float tl[64][kTileB + 1];
@@ -122,10 +126,14 @@ __global__ void __launch_bounds__(256) sc_range_kernel(const float* __restrict__
         if (n < N && row < B) {
             l = xl[(size_t)row * N + n];
             u = IV ? xu[(size_t)row * N + n] : l;
-            odd += (l - l) + (u - u);
-            if (IV) repair(l, u);
-            lmin = fminf(lmin, l); lmax = fmaxf(lmax, l);
-            umin = fminf(umin, u); umax = fmaxf(umax, u);
+            bool kept = true;
+            if constexpr (MASKED) kept = (xkeep[(size_t)row * (N / kChunk) + (n >> 5)] >> (n & 31)) & 1u;
+            if (kept) {
+                odd += (l - l) + (u - u);
+                if (IV) repair(l, u);
+                lmin = fminf(lmin, l); lmax = fmaxf(lmax, l);
+                umin = fminf(umin, u); umax = fmaxf(umax, u);
+            } else l = u = __builtin_nanf("");
         }
         tl[nl][col] = l;
         if (IV) tu[nl][col] = u;
@@ -156,9 +164,12 @@ __global__ void __launch_bounds__(256) sc_range_kernel(const float* __restrict__
             // A row whose value is undefined or infinite at this input drops terms the other rows keep, so nothing
             // may be concluded from the column: its range becomes everything (no lower bound, always a candidate).
             if (!(odd == 0.f)) { lmin = umin = -__builtin_inff(); lmax = umax = __builtin_inff(); }
+            const bool empty = lmin > lmax;   // no row of the tile keeps this input
+            bw = empty ? 0.f : fmaxf(lmax - lmin, umax - umin);
+            // empty: w - max l = -inf and min u - w = -inf (no lower bound); w - min l = -inf and max u - w = -inf (no candidate)
+            if (empty) { lmin = lmax = __builtin_inff(); umin = umax = -__builtin_inff(); }
             float* o = xr + (size_t)s * 4 * N + n;
             o[0] = lmin; o[N] = lmax; o[2 * (size_t)N] = umin; o[3 * (size_t)N] = umax;
-            bw = fmaxf(lmax - lmin, umax - umin);
             if (s == 0) ww = whi - wlo;
             if (!(bw < 3.0e38f)) bw = 3.0e38f;   // infinite or undefined widths count as very wide
         }
@@ -193,10 +204,11 @@ __device__ __forceinline__ bool table_pointless(const float* stat, int S) {
 // subtraction is monotone, so this holds for the rounded terms), and K chunks of inputs whose largest such bound is
 // at least t hold K terms that are at least t in every row: the kernel keeps the K largest chunk maxima of the slice
 // (one insertion per 32 inputs), whose K-th largest over all slices bounds the K-th largest term.
-template <int K, bool IV>
+// WMASK: wkeep holds one word per (weight row, 32 inputs); an input a weight row does not keep has no term.
+template <int K, bool IV, bool WMASK>
 __global__ void __launch_bounds__(256) sc_low_kernel(const float* __restrict__ w, const float* __restrict__ xr,
-                                                     int M, int N, int S, int Mp, float* __restrict__ lists,
-                                                     const float* __restrict__ stat) {
+                                                     const uint32_t* __restrict__ wkeep, int M, int N, int S, int Mp,
+                                                     float* __restrict__ lists, const float* __restrict__ stat) {
     if (table_pointless(stat, S)) return;
     __shared__ __attribute__((aligned(16))) float wt[64][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float xs[4][4][kChunk];
@@ -235,6 +247,8 @@ __global__ void __launch_bounds__(256) sc_low_kernel(const float* __restrict__ w
                 // largest lower bound of the chunk: fmaxf drops undefined differences (an undefined weight: the term
                 // is undefined in every row), and the lists start at 0
                 float cu = 0.f, cl = 0.f;
+                uint32_t kw = ~0u;
+                if constexpr (WMASK) kw = wkeep[(size_t)(m0 + r < M ? m0 + r : M - 1) * NCH + c];
                 #pragma unroll
                 for (int n4 = 0; n4 < kChunk; n4 += 4) {
                     const float4 wv4 = *reinterpret_cast<const float4*>(&wt[r][n4]);
@@ -247,7 +261,10 @@ __global__ void __launch_bounds__(256) sc_low_kernel(const float* __restrict__ w
                     const float umin[4] = {c4.x, c4.y, c4.z, c4.w}, umax[4] = {d4.x, d4.y, d4.z, d4.w};
                     #pragma unroll
                     for (int k = 0; k < 4; k++) {
-                        cu = fmaxf(fmaxf(cu, wv[k] - lmax[k]), umin[k] - wv[k]);
+                        if constexpr (WMASK) {
+                            const float a = fmaxf(wv[k] - lmax[k], umin[k] - wv[k]);
+                            cu = fmaxf(cu, ((kw >> (n4 + k)) & 1u) ? a : 0.f);
+                        } else cu = fmaxf(fmaxf(cu, wv[k] - lmax[k]), umin[k] - wv[k]);
                         if constexpr (IV) cl = fmaxf(fmaxf(cl, lmin[k] - wv[k]), wv[k] - umax[k]);
                     }
                 }
@@ -290,9 +307,10 @@ __global__ void __launch_bounds__(256) sc_merge_kernel(const float* __restrict__
 // of the tile reaches the bound of its list and is positive (the lists start at 0 and take larger values only).
 // The words of a wavefront's 64 rows are gathered in LDS and leave row by row, so that the main kernel finds the
 // words of a weight row side by side.  The marks are counted per wavefront.
-template <bool IV>
+template <bool IV, bool WMASK>
 __global__ void __launch_bounds__(256) sc_bits_kernel(const float* __restrict__ w, const float* __restrict__ xr,
-                                                      const float* __restrict__ low, int M, int N, int S, int Mp,
+                                                      const float* __restrict__ low,
+                                                      const uint32_t* __restrict__ wkeep, int M, int N, int S, int Mp,
                                                       uint32_t* __restrict__ bits, uint32_t* __restrict__ partial,
                                                       const float* __restrict__ stat) {
     if (table_pointless(stat, S)) return;
@@ -358,6 +376,7 @@ __global__ void __launch_bounds__(256) sc_bits_kernel(const float* __restrict__ 
                     }
                 }
                 if (!valid) word = 0u;
+                if constexpr (WMASK) word &= wkeep[(size_t)(m0 + r < M ? m0 + r : M - 1) * NCH + c];
                 wd[wave][r][c - c_lo] = word;
                 marks += __builtin_popcount(word);
             }
@@ -522,20 +541,166 @@ sc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
     }
 }
 
+// l-inf distance (maximum and where it sits) from the same tables, value form, optionally under the factored mask.
+// As sc_main_kernel, with the running maximum and its position (input number, bit 31 = the difference is negative;
+// the marks are walked in ascending input order and only a larger term replaces the maximum, so the first of
+// equal terms wins as in core/cuda/inf_dist_cuda.cu:176-190) instead of the top-K lists.  `low` holds the bound the
+// marks were taken against: every unmarked input's term is below it in every row, so a maximum that reaches it is
+// the maximum over all inputs.  Under the mask a row may keep none of the inputs the bound rests on; if any row of
+// the wavefront ends below the bound, the wavefront walks the weight row again over every input it keeps (`wkeep`
+// words; all inputs without a mask), which costs that wavefront what the every-term kernel costs it.
+template <bool POS>
+__global__ void __launch_bounds__(64 * kMainWaves)
+mc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const uint32_t* __restrict__ bits,
+               const uint32_t* __restrict__ wkeep, const float* __restrict__ low,
+               const unsigned long long* __restrict__ count, unsigned long long limit, int B, int Bp, int M, int Mp,
+               int N, float* __restrict__ y, int* __restrict__ pos) {
+    if (gate_closed(count, limit, 0)) return;
+    __shared__ uint16_t list[kMainWaves][kListCap];
+    __shared__ float stage_y[kTileB][kMainTile + 1];
+    __shared__ int stage_p[POS ? kTileB : 1][kMainTile + 1];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int MB = Mp / kMainTile, NCH = N / kChunk;
+    int item = blockIdx.x;
+    if (gridDim.x % 8 == 0) item = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int mb = item % MB, s = item / MB;
+    const float* __restrict__ xcol = xT + (size_t)s * kTileB + lane;
+    uint16_t* mine = list[wave];
+    const int m = mb * kMainTile + wave;
+    if (m < M) {   // wave-uniform
+        const float* __restrict__ wrow = w + (size_t)m * N;
+        float best[2];
+        int where[2];
+        float wreg[2];
+        int nreg[2];
+        float xa[2][4], xb[2][4];
+        auto load = [&](int buf, int k0, int total) {
+            int k = k0 + (lane & 3);
+            k = k < total ? k : total - 1;
+            const int nn = (int)mine[k];
+            nreg[buf] = nn;
+            wreg[buf] = wrow[nn];
+            #pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int n = __builtin_amdgcn_readlane(nn, i);
+                xa[buf][i] = xcol[(size_t)n * Bp];
+                xb[buf][i] = xcol[(size_t)n * Bp + 64];
+            }
+        };
+        auto compute = [&](int buf, int k0, int total) {
+            #pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if (k0 + i < total) {   // wave-uniform
+                    const float wi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wreg[buf]), i));
+                    const int n = __builtin_amdgcn_readlane(nreg[buf], i);
+                    const float d0 = xa[buf][i] - wi, d1 = xb[buf][i] - wi;
+                    // an undefined difference (an input the row does not keep) never compares greater
+                    if (fabsf(d0) > best[0]) { best[0] = fabsf(d0); if (POS) where[0] = n | (d0 >= 0.f ? 0 : (int)kSign); }
+                    if (fabsf(d1) > best[1]) { best[1] = fabsf(d1); if (POS) where[1] = n | (d1 >= 0.f ? 0 : (int)kSign); }
+                }
+            }
+        };
+        auto walk = [&](int total) {
+            if (total == 0) return;
+            load(0, 0, total);
+            for (int k0 = 0; k0 < total; k0 += 8) {
+                load(1, k0 + 4, total);
+                compute(0, k0, total);
+                load(0, k0 + 8, total);
+                compute(1, k0 + 4, total);
+            }
+        };
+        // one pass over the weight row: `words` = its table words, or (second pass) the inputs it keeps
+        auto pass = [&](const uint32_t* __restrict__ words) {
+            best[0] = best[1] = kEps;
+            where[0] = where[1] = 0;
+            int cnt = 0;
+            uint32_t next = lane < NCH ? (words ? words[lane] : ~0u) : 0u;
+            for (int c0 = 0; c0 < NCH; c0 += kBatch) {
+                uint32_t word = next;
+                if (c0 + kBatch < NCH) next = c0 + kBatch + lane < NCH ? (words ? words[c0 + kBatch + lane] : ~0u) : 0u;
+                const int mine_n = __builtin_popcount(word);
+                int incl = mine_n;
+                #pragma unroll
+                for (int o = 1; o < kBatch; o <<= 1) {
+                    const int t = __shfl_up(incl, o);
+                    if (lane >= o) incl += t;
+                }
+                int off = cnt + incl - mine_n;
+                cnt += __builtin_amdgcn_readlane(incl, kBatch - 1);
+                while (word) {
+                    const int i = __builtin_ctz(word);
+                    word &= word - 1;
+                    mine[off++] = (uint16_t)(((c0 + lane) << 5) | i);
+                }
+                if (cnt > kListCap - kBatch * kChunk || c0 + kBatch >= NCH) {
+                    __builtin_amdgcn_wave_barrier();
+                    walk(cnt);
+                    cnt = 0;
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+        };
+        pass(bits + ((size_t)s * Mp + m) * NCH);
+        const float bound = low[(size_t)(s * 2) * Mp + m];
+        const int b0 = s * kTileB + lane;
+        const bool short0 = b0 < B && best[0] < bound, short1 = b0 + 64 < B && best[1] < bound;
+        if (__builtin_amdgcn_ballot_w64(short0 || short1) != 0ull) pass(wkeep ? wkeep + (size_t)m * NCH : nullptr);
+        #pragma unroll
+        for (int j = 0; j < 2; j++) {
+            stage_y[lane + 64 * j][wave] = best[j];
+            if (POS) stage_p[lane + 64 * j][wave] = where[j];
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < kTileB * kMainTile; e += 64 * kMainWaves) {
+        const int bl = e / kMainTile, mloc = e % kMainTile;
+        const int b = s * kTileB + bl, mm = mb * kMainTile + mloc;
+        if (b < B && mm < M) {
+            y[(size_t)b * M + mm] = stage_y[bl][mloc];
+            if (POS) pos[(size_t)b * M + mm] = stage_p[bl][mloc];
+        }
+    }
+}
+
+template <int K, bool WMASK>
+int run_max(const float* x, const float* w, const uint32_t* xkeep, const uint32_t* wkeep, int B, int M, int N, float* y,
+            int* pos, const Carve& c, unsigned long long limit, hipStream_t st) {
+    const int S = tiles_b(B), Bp = S * kTileB, Mp = mpad_of(M), NCH = N / kChunk, slices = slices_of(NCH);
+    int rc;
+    if ((rc = fill_zero(c.count, 8, st))) return rc;   // the count, its flag and the two sums of the probe behind them
+    if (WMASK) hipLaunchKernelGGL((sc_range_kernel<false, true>), dim3((N + 63) / 64, S), dim3(256), 0, st, x, nullptr, w, xkeep, B, M, N, Bp, c.xr, c.xT, c.stat);
+    else hipLaunchKernelGGL((sc_range_kernel<false, false>), dim3((N + 63) / 64, S), dim3(256), 0, st, x, nullptr, w, nullptr, B, M, N, Bp, c.xr, c.xT, c.stat);
+    if ((rc = check_launch("sc_range_kernel"))) return rc;
+    hipLaunchKernelGGL((sc_low_kernel<K, false, WMASK>), dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, wkeep, M, N, S, Mp, c.lists, c.stat);
+    if ((rc = check_launch("sc_low_kernel"))) return rc;
+    hipLaunchKernelGGL((sc_merge_kernel<K>), dim3((Mp + 255) / 256, S), dim3(256), 0, st, c.lists, slices, Mp, 1, c.low, c.stat);
+    if ((rc = check_launch("sc_merge_kernel"))) return rc;
+    hipLaunchKernelGGL((sc_bits_kernel<false, WMASK>), dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, c.low, wkeep, M, N, S, Mp, c.bits, c.partial, c.stat);
+    if ((rc = check_launch("sc_bits_kernel"))) return rc;
+    hipLaunchKernelGGL(sc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count, c.stat, S, limit);
+    if ((rc = check_launch("sc_sum_kernel"))) return rc;
+    const dim3 grid((unsigned)(S * (Mp / kMainTile)));
+    if (pos) hipLaunchKernelGGL((mc_main_kernel<true>), grid, dim3(64 * kMainWaves), 0, st, c.xT, w, c.bits, wkeep, c.low, c.count, limit, B, Bp, M, Mp, N, y, pos);
+    else hipLaunchKernelGGL((mc_main_kernel<false>), grid, dim3(64 * kMainWaves), 0, st, c.xT, w, c.bits, wkeep, c.low, c.count, limit, B, Bp, M, Mp, N, y, pos);
+    return check_launch("mc_main_kernel");
+}
+
 template <int K, bool IV>
 int run(const float* xl, const float* xu, const float* w, int B, int M, int N, float q, float* outL, float* outU,
         const Carve& c, unsigned long long limit, hipStream_t st) {
     const int S = tiles_b(B), Bp = S * kTileB, Mp = mpad_of(M), NCH = N / kChunk, slices = slices_of(NCH);
     int rc;
     if ((rc = fill_zero(c.count, 8, st))) return rc;   // the count and the two sums of the probe behind it
-    hipLaunchKernelGGL((sc_range_kernel<IV>), dim3((N + 63) / 64, S), dim3(256), 0, st, xl, xu, w, B, M, N, Bp, c.xr, c.xT, c.stat);
+    hipLaunchKernelGGL((sc_range_kernel<IV, false>), dim3((N + 63) / 64, S), dim3(256), 0, st, xl, xu, w, nullptr, B, M, N, Bp, c.xr, c.xT, c.stat);
     if ((rc = check_launch("sc_range_kernel"))) return rc;
-    hipLaunchKernelGGL((sc_low_kernel<K, IV>), dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, M, N, S, Mp, c.lists, c.stat);
+    hipLaunchKernelGGL((sc_low_kernel<K, IV, false>), dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, nullptr, M, N, S, Mp, c.lists, c.stat);
     if ((rc = check_launch("sc_low_kernel"))) return rc;
     const int nw = IV ? 2 : 1;
     hipLaunchKernelGGL((sc_merge_kernel<K>), dim3((Mp + 255) / 256, S * nw), dim3(256), 0, st, c.lists, slices, Mp, nw, c.low, c.stat);
     if ((rc = check_launch("sc_merge_kernel"))) return rc;
-    hipLaunchKernelGGL((sc_bits_kernel<IV>), dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, c.low, M, N, S, Mp, c.bits, c.partial, c.stat);
+    hipLaunchKernelGGL((sc_bits_kernel<IV, false>), dim3(Mp / 64, slices), dim3(256), 0, st, w, c.xr, c.low, nullptr, M, N, S, Mp, c.bits, c.partial, c.stat);
     if ((rc = check_launch("sc_bits_kernel"))) return rc;
     hipLaunchKernelGGL(sc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count, c.stat, S, limit);
     if ((rc = check_launch("sc_sum_kernel"))) return rc;
@@ -574,6 +739,40 @@ int sort_cols_forward(const float* xl, const float* xu, const float* w, int B, i
 #undef X
     }
     set_error("sort_cols_forward: K=%d outside 2..25", K);
+    return SD_ERR_ARG;
+}
+
+
+int max_cols_depth(float keep_x) {
+    if (keep_x >= 1.f) return 1;
+    // inputs the bound rests on such that a row keeps none of them less often than once in 10^6 outputs
+    const int need = (int)ceilf(logf(1e-6f) / logf(1.f - keep_x));
+    for (int k : {8, 12, 16, 20, 24}) if (need <= k) return k;
+    return 0;
+}
+
+size_t max_cols_workspace(int B, int CO, int CI, int K) { return sort_cols_workspace(B, CO, CI, K); }
+
+int max_cols_forward(const float* x, const float* w, const uint32_t* xkeep, const uint32_t* wkeep, int B, int CO, int CI,
+                     int K, float* y, int* pos, void* ws, float density, const unsigned long long** gate,
+                     unsigned long long* gate_limit, hipStream_t st) {
+    if (CI % kChunk != 0 || CI > 65536 || B < 1 || CO < 1 || (xkeep == nullptr) != (wkeep == nullptr)) {
+        set_error("max_cols_forward: shape not supported");
+        return SD_ERR_ARG;
+    }
+    const Carve c = carve(ws, B, CO, CI, K);
+    const float d = density < 0.f ? 0.f : density > 1.f ? 1.f : density;
+    const unsigned long long limit = (unsigned long long)((double)tiles_b(B) * CO * CI * d);
+    *gate = c.count;
+    *gate_limit = limit;
+    if (!xkeep) {
+        if (K == 1) return run_max<1, false>(x, w, nullptr, nullptr, B, CO, CI, y, pos, c, limit, st);
+    } else switch (K) {
+#define X(k) case k: return run_max<k, true>(x, w, xkeep, wkeep, B, CO, CI, y, pos, c, limit, st);
+        X(8) X(12) X(16) X(20) X(24)
+#undef X
+    }
+    set_error("max_cols_forward: depth %d not supported", K);
     return SD_ERR_ARG;
 }
 

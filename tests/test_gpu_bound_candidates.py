@@ -128,6 +128,26 @@ def test_bound_candidate_kernel_at_layer_size(density):
         assert torch.equal(out[dens][0], out[0.0][0]) and torch.equal(out[dens][1], out[0.0][1]), dens
 
 
+def test_bound_results_do_not_depend_on_the_table_hint(oracle, density):
+    """With the built-in limit a layer (same weights, same shape) whose tables did not pay a few times in a row is
+    given none for a while: calls before, during and after that stretch give the oracle's bits, on data of either kind."""
+    from sortnet_amd import ext
+    dev = _dev()
+    density(-1.0)
+    B, CI, CO = 140, 512, 200
+    g = torch.Generator().manual_seed(11)
+    w = (torch.randn(CO, CI, generator=g) * 0.3).contiguous().to(dev)
+    for call in range(12):
+        kind = "random" if call < 8 else "rows_alike"     # unrelated rows: every term; rows alike: the table
+        xl, xu = _intervals(B, CI, kind, 100 + call)
+        rl, ru = oracle.bound_inf_dist_forward(xl.numpy(), xu.numpy(), w.cpu().numpy(), 1, need_pos=False)
+        yl = torch.full((B, CO, 1), float("nan"), device=dev)
+        yu = torch.full((B, CO, 1), float("nan"), device=dev)
+        ext.bound_inf_dist_forward_nograd(xl.to(dev), xu.to(dev), w, yl, yu, 1)
+        torch.cuda.synchronize()   # lets the next call see which kernel ran
+        assert np.array_equal(yl.cpu().numpy(), rl) and np.array_equal(yu.cpu().numpy(), ru), call
+
+
 def test_bound_candidate_density_argument(density):
     from sortnet_amd import _lib
     with pytest.raises(RuntimeError):

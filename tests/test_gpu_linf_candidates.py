@@ -1,0 +1,137 @@
+"""GPU parity of the l-inf forward (plain and under the factored mask) when it works from candidate tables (dense
+single-group layers, CI % 32 == 0).
+
+The entry points queue a kernel that evaluates only the inputs a table marks as able to hold the maximum of a weight
+row, and the kernels that evaluate every term; a count taken on the device picks one.  Values AND positions must be
+the oracle's bits either way (core/cuda/inf_dist_cuda.cu:110-212 semantics: the first of equal terms wins, the 1e-10
+floor with position 0 when nothing exceeds it): the tests force either side (density 1 / 0) and the built-in limit,
+on batches whose rows are alike against weights of unit scale (the table marks little), on unrelated rows, on grid
+data with many exact ties, and under the mask with a shallow bound so that some outputs are recomputed from every
+input."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+@pytest.fixture
+def knobs():
+    from sortnet_amd import _lib
+
+    def set_(density, depth=0):
+        _lib.set_linf_candidate_density(density)
+        _lib.set_linf_candidate_depth(depth)
+    yield set_
+    _lib.set_linf_candidate_density(-1.0)
+    _lib.set_linf_candidate_depth(0)
+
+
+def _data(B, CI, CO, kind, seed):
+    g = torch.Generator().manual_seed(seed)
+    if kind == "rows_alike":
+        x = torch.randn(1, CI, 1, generator=g) * 0.3 + torch.randn(B, CI, 1, generator=g) * 0.05
+        w = torch.randn(CO, CI, generator=g)
+    elif kind == "images":
+        x = torch.rand(B, CI, 1, generator=g)
+        w = torch.randn(CO, CI, generator=g) * CI ** -0.5
+    elif kind == "ties":
+        x = torch.round(torch.randn(B, CI, 1, generator=g) * 0.2 * 4) / 4
+        w = torch.round(torch.randn(CO, CI, generator=g) * 4) / 4
+    else:
+        x = torch.randn(B, CI, 1, generator=g)
+        w = torch.randn(CO, CI, generator=g)
+    return x.contiguous(), w.contiguous()
+
+
+def _check_plain(oracle, x, w, tag):
+    from sortnet_amd import ext
+    dev = _dev()
+    B, CO = x.shape[0], w.shape[0]
+    ry, rpos = oracle.inf_dist_forward(x.numpy(), w.numpy(), 1)
+    y = torch.full((B, CO, 1), float("nan"), device=dev)
+    pos = torch.full((B, CO, 1), -7, device=dev, dtype=torch.int32)
+    ext.inf_dist_forward(x.to(dev), w.to(dev), y, pos, 1)
+    assert np.array_equal(y.cpu().numpy(), ry), tag
+    assert np.array_equal(pos.cpu().numpy(), rpos), tag
+    y2 = torch.full((B, CO, 1), float("nan"), device=dev)
+    ext.inf_dist_forward_nograd(x.to(dev), w.to(dev), y2, 1)
+    assert np.array_equal(y2.cpu().numpy(), ry), tag
+
+
+def _check_masked(oracle, x, w, q, seed, tag):
+    from sortnet_amd import ext
+    dev = _dev()
+    B, CO = x.shape[0], w.shape[0]
+    ry, rpos = oracle.masked_inf_dist_forward(x.numpy(), w.numpy(), q, seed, ext.MASK_FACTORED, 1)
+    y = torch.full((B, CO, 1), float("nan"), device=dev)
+    pos = torch.full((B, CO, 1), -7, device=dev, dtype=torch.int32)
+    ext.masked_inf_dist_forward(x.to(dev), w.to(dev), y, pos, 1, q, seed, ext.MASK_FACTORED)
+    assert np.array_equal(y.cpu().numpy(), ry), tag
+    assert np.array_equal(pos.cpu().numpy(), rpos), tag
+    y2 = torch.full((B, CO, 1), float("nan"), device=dev)
+    ext.masked_inf_dist_forward(x.to(dev), w.to(dev), y2, None, 1, q, seed, ext.MASK_FACTORED)
+    assert np.array_equal(y2.cpu().numpy(), ry), tag
+
+
+SHAPES = [(70, 96, 64), (33, 2048, 300), (130, 1024, 513), (1, 32, 1), (257, 320, 129), (512, 2112, 96)]
+
+
+@pytest.mark.parametrize("dens", [1.0, 0.0, -1.0])
+@pytest.mark.parametrize("B,CI,CO", SHAPES)
+def test_linf_candidate_kernels_match_oracle(oracle, knobs, dens, B, CI, CO):
+    """Ragged batch tiles and weight rows, rows of more than 64 chunks (several loads of table words per row)."""
+    knobs(dens)
+    for kind in ("rows_alike", "random", "images", "ties"):
+        x, w = _data(B, CI, CO, kind, B + CI)
+        _check_plain(oracle, x, w, "dens=%g %s" % (dens, kind))
+
+
+@pytest.mark.parametrize("dens,depth", [(1.0, 0), (1.0, 8), (0.0, 0), (-1.0, 0)])
+@pytest.mark.parametrize("B,CI,CO", SHAPES)
+def test_masked_candidate_kernels_match_oracle(oracle, knobs, dens, depth, B, CI, CO):
+    """Factored mask at q = 0.3, 0.75 and 1.  Depth 8 at q = 0.3: a row keeps none of the eight inputs the bound
+    rests on about once in 600 outputs, so many wavefronts walk their weight row a second time over every input."""
+    knobs(dens, depth)
+    for kind in ("rows_alike", "random", "ties"):
+        for q, seed in ((0.3, 5), (0.75, 77), (1.0, 3)):
+            x, w = _data(B, CI, CO, kind, B + CI + 1)
+            _check_masked(oracle, x, w, q, seed, "dens=%g depth=%d %s q=%g" % (dens, depth, kind, q))
+
+
+def test_linf_candidate_kernels_at_layer_size(knobs):
+    """B = 512, N = M = 5120, unit-scale weights against rows that are nearly alike: table kernels and every-term
+    kernels give the same values and positions, plain and masked, and the built-in limit picks the table."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, N, M = 512, 5120, 5120
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(1, N, 1, generator=g) * 0.3 + torch.randn(B, N, 1, generator=g) * 0.1).contiguous().to(dev)
+    w = torch.randn(M, N, generator=g).contiguous().to(dev)
+    out = {}
+    for dens in (0.0, 1.0, -1.0):
+        knobs(dens)
+        y, ym = torch.empty(B, M, 1, device=dev), torch.empty(B, M, 1, device=dev)
+        p = torch.empty(B, M, 1, device=dev, dtype=torch.int32)
+        pm = torch.empty_like(p)
+        ext.inf_dist_forward(x, w, y, p, 1)
+        ext.masked_inf_dist_forward(x, w, ym, pm, 1, 0.3, 9, ext.MASK_FACTORED)
+        out[dens] = (y, p, ym, pm)
+    for dens in (1.0, -1.0):
+        for a, b in zip(out[dens], out[0.0]):
+            assert torch.equal(a, b), dens
+
+
+def test_linf_candidate_arguments(knobs):
+    from sortnet_amd import _lib
+    with pytest.raises(RuntimeError):
+        _lib.set_linf_candidate_density(1.5)
+    with pytest.raises(RuntimeError):
+        _lib.set_linf_candidate_depth(5)
+    knobs(0.3, 12)
