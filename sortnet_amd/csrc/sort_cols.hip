@@ -745,8 +745,9 @@ int sort_cols_forward(const float* xl, const float* xu, const float* w, int B, i
 
 int max_cols_depth(float keep_x) {
     if (keep_x >= 1.f) return 1;
-    // inputs the bound rests on such that a row keeps none of them less often than once in 10^6 outputs
-    const int need = (int)ceilf(logf(1e-6f) / logf(1.f - keep_x));
+    // inputs the bound rests on such that a row keeps none of them less often than once in 10^4 outputs (such an
+    // output costs its wavefront a second pass over every input; more inputs lower the bound and mark more)
+    const int need = (int)ceilf(logf(1e-4f) / logf(1.f - keep_x));
     for (int k : {8, 12, 16, 20, 24}) if (need <= k) return k;
     return 0;
 }
