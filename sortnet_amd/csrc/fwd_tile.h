@@ -841,6 +841,7 @@ struct SortNograd : PolicyBase {
 
 template <int K>
 struct SortPos : PolicyBase {
+    static constexpr bool GATED = true;   // one of two queued for a result when FwdArgs::gate is set
     struct Acc { float res[K]; int idx[K]; };
     static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
         #pragma unroll

@@ -139,7 +139,7 @@ constexpr long long kSortColsMinTerms = 1ll << 24;
 
 // `site`: which entry point asks (with the built-in limit, a layer whose tables have not paid lately is not given
 // any for a while, see hint_build_tables)
-constexpr int kHintSiteSort = 2, kHintSiteBoundSort = 3;
+constexpr int kHintSiteSort = 2, kHintSiteBoundSort = 3, kHintSiteSortPos = 6;
 static bool sort_cols_ok(const FwdArgs& a, int site, int B, int CO, int CI, int G, int HW, hipStream_t st) {
     if (g_sort_density == 0.f || G != 1 || HW != 1 || CI % kSortColsChunk != 0 || !a.fast_x || !a.fast_w) return false;
     if (g_sort_density > 0.f) return true;
@@ -154,9 +154,9 @@ static void sort_cols_report(const FwdArgs& a, int site, int B, int CO, int CI, 
 // not be given memory that overlaps it, and `ws` must stay allocated until they have run (one workspace request
 // per call, carved by the caller).
 static int queue_sort_cols(FwdArgs& a, const float* xl, const float* xu, const float* w, int B, int CO, int CI, float q,
-                           int K, float* outL, float* outU, void* ws, hipStream_t st) {
+                           int K, float* outL, float* outU, int* pos, void* ws, hipStream_t st) {
     const float cap = g_sort_density > 0.f ? g_sort_density : kSortColsCap;
-    int rc = sort_cols_forward(xl, xu, w, B, CO, CI, q, K, outL, outU, ws, cap, &a.gate, &a.gate_limit, st);
+    int rc = sort_cols_forward(xl, xu, w, B, CO, CI, q, K, outL, outU, pos, ws, cap, &a.gate, &a.gate_limit, st);
     a.gate_above = 1;
     return rc;
 }
@@ -194,7 +194,7 @@ extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* we
         if (!base) return SD_ERR_HIP;
     }
     int* keys = reinterpret_cast<int*>(base + tbytes);
-    if (cols && (rc = queue_sort_cols(a, input, nullptr, weight, B, CO, CI, q, K, nullptr, output, base, st))) return rc;
+    if (cols && (rc = queue_sort_cols(a, input, nullptr, weight, B, CO, CI, q, K, nullptr, output, nullptr, base, st))) return rc;
     rc = SD_ERR_ARG;
     switch (K) {
 #define X(k) case k: if (k <= 12 && two) rc = run_two_level<(k <= 12 ? k : 2), true>(a, small, keys, st); \
@@ -220,18 +220,26 @@ extern "C" int sd_sort_neuron_forward(const float* input, const float* weight,
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 32);
     const bool two = K <= 12 && two_level_ok(a, K);
-    int* keys = nullptr;
-    if (two) {
-        keys = static_cast<int*>(workspace(two_level_bytes(a, K), st));
-        if (!keys) return SD_ERR_HIP;
+    const bool cols = sort_cols_ok(a, kHintSiteSortPos, B, CO, CI, G, HW, st);
+    // one request for both users of the workspace, as in sd_sort_neuron_forward_nograd
+    const size_t tbytes = cols ? (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256 : 0;
+    char* base = nullptr;
+    if (cols || two) {
+        base = static_cast<char*>(workspace(tbytes + (two ? two_level_bytes(a, K) : 0), st));
+        if (!base) return SD_ERR_HIP;
     }
+    int* keys = reinterpret_cast<int*>(base + tbytes);
+    if (cols && (rc = queue_sort_cols(a, input, nullptr, weight, B, CO, CI, q, K, nullptr, output, pos, base, st))) return rc;
+    rc = SD_ERR_ARG;
     switch (K) {
-#define X(k) case k: if (k <= 12 && two) return run_two_level<(k <= 12 ? k : 2), false>(a, few_tiles(a, 32, 64), keys, st); \
-                     return small ? launch_fwd<SortPos<k>, 1, 2>(a, st) : launch_fwd<SortPos<k>, 2, 2>(a, st);
+#define X(k) case k: if (k <= 12 && two) rc = run_two_level<(k <= 12 ? k : 2), false>(a, few_tiles(a, 32, 64), keys, st); \
+                     else rc = small ? launch_fwd<SortPos<k>, 1, 2>(a, st) : launch_fwd<SortPos<k>, 2, 2>(a, st); \
+                     break;
         SD_FOR_EACH_K(X)
 #undef X
     }
-    return SD_ERR_ARG;
+    if (cols && rc == SD_OK) sort_cols_report(a, kHintSiteSortPos, B, CO, CI, st);
+    return rc;
 }
 
 extern "C" int sd_bound_sort_neuron_forward(const float* inputL, const float* inputU, const float* weight,
@@ -250,7 +258,7 @@ extern "C" int sd_bound_sort_neuron_forward(const float* inputL, const float* in
     if (cols) {
         void* ws = workspace(sort_cols_workspace(B, CO, CI, K), st);   // the only request of this call
         if (!ws) return SD_ERR_HIP;
-        if ((rc = queue_sort_cols(a, inputL, inputU, weight, B, CO, CI, q, K, outputL, outputU, ws, st))) return rc;
+        if ((rc = queue_sort_cols(a, inputL, inputU, weight, B, CO, CI, q, K, outputL, outputU, nullptr, ws, st))) return rc;
     }
     rc = SD_ERR_ARG;
     switch (K) {

@@ -23,9 +23,10 @@ size_t sort_cols_workspace(int B, int CO, int CI, int K);
 // `density` of all (tile, weight row, input) triples are marked; the caller queues the kernels that evaluate every
 // term with the opposite condition on the same counter (*gate, *gate_limit); (*gate)[1] is 1 when those are to run.
 //   xu != nullptr: interval form, outL / outU receive the bounds;
-//   xu == nullptr: value form on xl, outU receives the values (outL is not used).
+//   xu == nullptr: value form on xl, outU receives the values (outL is not used) and pos, if not null, the K planes
+//   of positions (K, B, CO), largest first.
 int sort_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float q, int K,
-                      float* outL, float* outU, void* ws, float density, const unsigned long long** gate,
+                      float* outL, float* outU, int* pos, void* ws, float density, const unsigned long long** gate,
                       unsigned long long* gate_limit, hipStream_t st);
 
 // l-inf distance forward (maximum and, if pos is not null, its position) from the same kind of table, optionally

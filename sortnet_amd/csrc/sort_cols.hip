@@ -687,9 +687,126 @@ int run_max(const float* x, const float* w, const uint32_t* xkeep, const uint32_
     return check_launch("mc_main_kernel");
 }
 
+// Value form with positions (core/cuda/sort_neuron.cu:111-214): as sc_main_kernel, with the ordered insertion that
+// carries the input numbers.  The marks of a row are walked in ascending input order, and every term that is at
+// least the final K-th largest value of an output is marked, so these terms meet the list in the order and against
+// the entries they meet in the scan over all inputs: same values and same positions, ties included.  pos is
+// (K, B, M) with slot 0 = largest; the K planes leave through LDS one after the other.
+template <int K>
+__global__ void __launch_bounds__(64 * kMainWaves)
+sp_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const uint32_t* __restrict__ bits,
+               const unsigned long long* __restrict__ count, unsigned long long limit, int B, int Bp, int M, int Mp,
+               int N, float q, float* __restrict__ y, int* __restrict__ pos) {
+    if (gate_closed(count, limit, 0)) return;
+    __shared__ uint16_t list[kMainWaves][kListCap];
+    __shared__ int stage[kTileB][kMainTile + 1];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int MB = Mp / kMainTile, NCH = N / kChunk;
+    int item = blockIdx.x;
+    if (gridDim.x % 8 == 0) item = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int mb = item % MB, s = item / MB;
+    const float* __restrict__ xcol = xT + (size_t)s * kTileB + lane;
+    uint16_t* mine = list[wave];
+    const int m = mb * kMainTile + wave;
+    float res[2][K];
+    int idx[2][K];
+    #pragma unroll
+    for (int k = 0; k < K; k++) { res[0][k] = res[1][k] = 0.f; idx[0][k] = idx[1][k] = 0; }
+    if (m < M) {   // wave-uniform
+        const float* __restrict__ wrow = w + (size_t)m * N;
+        const uint32_t* __restrict__ rowbits = bits + ((size_t)s * Mp + m) * NCH;
+        float wreg[2];
+        int nreg[2];
+        float xa[2][4], xb[2][4];
+        auto load = [&](int buf, int k0, int total) {
+            int k = k0 + (lane & 3);
+            k = k < total ? k : total - 1;
+            const int nn = (int)mine[k];
+            nreg[buf] = nn;
+            wreg[buf] = wrow[nn];
+            #pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int n = __builtin_amdgcn_readlane(nn, i);
+                xa[buf][i] = xcol[(size_t)n * Bp];
+                xb[buf][i] = xcol[(size_t)n * Bp + 64];
+            }
+        };
+        auto compute = [&](int buf, int k0, int total) {
+            #pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if (k0 + i < total) {   // wave-uniform
+                    const float wi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wreg[buf]), i));
+                    const int n = __builtin_amdgcn_readlane(nreg[buf], i);
+                    const float d0 = xa[buf][i] - wi, d1 = xb[buf][i] - wi;
+                    if (fabsf(d0) > res[0][0]) topk_insert<K>(res[0], idx[0], fabsf(d0), n | (d0 >= 0.f ? 0 : (int)kSign));
+                    if (fabsf(d1) > res[1][0]) topk_insert<K>(res[1], idx[1], fabsf(d1), n | (d1 >= 0.f ? 0 : (int)kSign));
+                }
+            }
+        };
+        auto walk = [&](int total) {
+            if (total == 0) return;
+            load(0, 0, total);
+            for (int k0 = 0; k0 < total; k0 += 8) {
+                load(1, k0 + 4, total);
+                compute(0, k0, total);
+                load(0, k0 + 8, total);
+                compute(1, k0 + 4, total);
+            }
+        };
+        int cnt = 0;
+        uint32_t next = lane < NCH ? rowbits[lane] : 0u;
+        for (int c0 = 0; c0 < NCH; c0 += kBatch) {
+            uint32_t word = next;
+            if (c0 + kBatch < NCH) next = c0 + kBatch + lane < NCH ? rowbits[c0 + kBatch + lane] : 0u;
+            const int mine_n = __builtin_popcount(word);
+            int incl = mine_n;
+            #pragma unroll
+            for (int o = 1; o < kBatch; o <<= 1) {
+                const int t = __shfl_up(incl, o);
+                if (lane >= o) incl += t;
+            }
+            int off = cnt + incl - mine_n;
+            cnt += __builtin_amdgcn_readlane(incl, kBatch - 1);
+            while (word) {
+                const int i = __builtin_ctz(word);
+                word &= word - 1;
+                mine[off++] = (uint16_t)(((c0 + lane) << 5) | i);
+            }
+            if (cnt > kListCap - kBatch * kChunk || c0 + kBatch >= NCH) {
+                __builtin_amdgcn_wave_barrier();
+                walk(cnt);
+                cnt = 0;
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+    }
+    const size_t plane = (size_t)B * M;
+    // the values, then the K planes of positions (slot 0 = largest = res[K-1])
+    #pragma unroll
+    for (int round = 0; round <= K; round++) {
+        if (m < M) {
+            #pragma unroll
+            for (int j = 0; j < 2; j++)
+                stage[lane + 64 * j][wave] = round == 0 ? __builtin_bit_cast(int, geo_sum<K>(res[j], q)) : idx[j][K - round];
+        }
+        __syncthreads();
+        for (int e = tid; e < kTileB * kMainTile; e += 64 * kMainWaves) {
+            const int bl = e / kMainTile, mloc = e % kMainTile;
+            const int b = s * kTileB + bl, mm = mb * kMainTile + mloc;
+            if (b < B && mm < M) {
+                const size_t o = (size_t)b * M + mm;
+                if (round == 0) y[o] = __builtin_bit_cast(float, stage[bl][mloc]);
+                else pos[(size_t)(round - 1) * plane + o] = stage[bl][mloc];
+            }
+        }
+        __syncthreads();
+    }
+}
+
 template <int K, bool IV>
 int run(const float* xl, const float* xu, const float* w, int B, int M, int N, float q, float* outL, float* outU,
-        const Carve& c, unsigned long long limit, hipStream_t st) {
+        int* pos, const Carve& c, unsigned long long limit, hipStream_t st) {
     const int S = tiles_b(B), Bp = S * kTileB, Mp = mpad_of(M), NCH = N / kChunk, slices = slices_of(NCH);
     int rc;
     if ((rc = fill_zero(c.count, 8, st))) return rc;   // the count and the two sums of the probe behind it
@@ -704,6 +821,13 @@ int run(const float* xl, const float* xu, const float* w, int B, int M, int N, f
     if ((rc = check_launch("sc_bits_kernel"))) return rc;
     hipLaunchKernelGGL(sc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)(Mp / 64) * slices * 4, c.count, c.stat, S, limit);
     if ((rc = check_launch("sc_sum_kernel"))) return rc;
+    if constexpr (!IV) {
+        if (pos) {
+            hipLaunchKernelGGL((sp_main_kernel<K>), dim3((unsigned)(S * (Mp / kMainTile))), dim3(64 * kMainWaves), 0, st,
+                               c.xT, w, c.bits, c.count, limit, B, Bp, M, Mp, N, q, outU, pos);
+            return check_launch("sp_main_kernel");
+        }
+    }
     hipLaunchKernelGGL((sc_main_kernel<K, IV>), dim3((unsigned)(S * (Mp / kMainTile))), dim3(64 * kMainWaves), 0, st,
                        c.xT, w, c.bits, c.count, limit, B, Bp, M, Mp, N, q, outL, outU);
     return check_launch("sc_main_kernel");
@@ -721,7 +845,7 @@ size_t sort_cols_workspace(int B, int CO, int CI, int K) {
     X(18) X(19) X(20) X(21) X(22) X(23) X(24) X(25)
 
 int sort_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float q, int K,
-                      float* outL, float* outU, void* ws, float density, const unsigned long long** gate,
+                      float* outL, float* outU, int* pos, void* ws, float density, const unsigned long long** gate,
                       unsigned long long* gate_limit, hipStream_t st) {
     if (CI % kChunk != 0 || CI > 65536 || B < 1 || CO < 1) {
         set_error("sort_cols_forward: shape not supported");
@@ -733,8 +857,8 @@ int sort_cols_forward(const float* xl, const float* xu, const float* w, int B, i
     *gate = c.count;
     *gate_limit = limit;
     switch (K) {
-#define X(k) case k: return xu ? run<k, true>(xl, xu, w, B, CO, CI, q, outL, outU, c, limit, st) \
-                               : run<k, false>(xl, nullptr, w, B, CO, CI, q, outL, outU, c, limit, st);
+#define X(k) case k: return xu ? run<k, true>(xl, xu, w, B, CO, CI, q, outL, outU, nullptr, c, limit, st) \
+                               : run<k, false>(xl, nullptr, w, B, CO, CI, q, outL, outU, pos, c, limit, st);
         SD_SORT_COLS_K(X)
 #undef X
     }

@@ -1,4 +1,4 @@
-"""GPU parity of the sort neuron (values only) and its interval bounds when they work from candidate tables (dense
+"""GPU parity of the sort neuron (values, values with positions) and its interval bounds when they work from candidate tables (dense
 single-group layers, CI % 32 == 0).
 
 Both entry points queue a kernel that evaluates only the inputs a table marks as able to be among the K largest
@@ -60,17 +60,21 @@ def _run(x, xl, xu, w, q, K):
     y, yl, yu = (torch.full((B, CO, 1), float("nan"), device=dev) for _ in range(3))
     ext.sort_neuron_forward_nograd(x.to(dev), w.to(dev), y, 1, q, K)
     ext.bound_sort_neuron_forward(xl.to(dev), xu.to(dev), w.to(dev), yl, yu, 1, q, K)
-    return y.cpu().numpy(), yl.cpu().numpy(), yu.cpu().numpy()
+    yp = torch.full((B, CO, 1), float("nan"), device=dev)
+    pos = torch.full((K, B, CO, 1), -7, device=dev, dtype=torch.int32)
+    ext.sort_neuron_forward(x.to(dev), w.to(dev), yp, pos, 1, q, K)
+    return y.cpu().numpy(), yl.cpu().numpy(), yu.cpu().numpy(), yp.cpu().numpy(), pos.cpu().numpy()
 
 
 def _check(oracle, density, dens, x, xl, xu, w, q, K, tag):
     """Against the oracle at the sort neuron's bar (rel 1e-5), and bit for bit against the every-term kernels."""
-    ry = oracle.sort_neuron_forward(x.numpy(), w.numpy(), q, K, need_pos=False)
+    ry, rpos = oracle.sort_neuron_forward(x.numpy(), w.numpy(), q, K)
     rl, ru = oracle.bound_sort_neuron_forward(xl.numpy(), xu.numpy(), w.numpy(), q, K)
     density(dens)
     got = _run(x, xl, xu, w, q, K)
-    for g, r in zip(got, (ry, rl, ru)):
+    for g, r in zip(got[:4], (ry, rl, ru, ry)):
         np.testing.assert_allclose(g, r, rtol=RTOL, err_msg=tag)
+    assert np.array_equal(got[4], rpos), tag   # positions: exact, ties included
     if dens != 0.0:
         density(0.0)
         for g, e in zip(got, _run(x, xl, xu, w, q, K)):
@@ -109,10 +113,12 @@ def test_sort_candidate_kernels_at_layer_size(density):
     out = {}
     for dens in (0.0, 1.0, -1.0):
         density(dens)
-        y, yl, yu = (torch.empty(B, M, 1, device=dev) for _ in range(3))
+        y, yl, yu, yp = (torch.empty(B, M, 1, device=dev) for _ in range(4))
+        pos = torch.empty(K, B, M, 1, device=dev, dtype=torch.int32)
         ext.sort_neuron_forward_nograd(x.contiguous(), w, y, 1, q, K)
         ext.bound_sort_neuron_forward(xl, xu, w, yl, yu, 1, q, K)
-        out[dens] = (y, yl, yu)
+        ext.sort_neuron_forward(x.contiguous(), w, yp, pos, 1, q, K)
+        out[dens] = (y, yl, yu, yp, pos)
     for dens in (1.0, -1.0):
         for a, b in zip(out[dens], out[0.0]):
             assert torch.equal(a, b), dens
