@@ -71,10 +71,10 @@ int sd_set_lp_candidate_density(float density);
  * that evaluates every term; both give the same bits.  Built-in limit 0.26.  No reference counterpart
  * (core/cuda/bound_inf_dist_cuda.cu evaluates every term). */
 int sd_set_bound_candidate_density(float density);
-/* The same for sd_sort_neuron_forward_nograd and sd_bound_sort_neuron_forward on dense single-group layers (CI a
+/* The same for sd_sort_neuron_forward[_nograd] and sd_bound_sort_neuron_forward on dense single-group layers (CI a
  * multiple of 32): a kernel that works from a table of the inputs that can be among the K largest terms of a weight
- * row over a tile of 128 batch rows, and the kernels that evaluate every term; both give the same bits.  Built-in
- * limit 0.10, and the table is only built for layers of at least 2^24 terms; a positive `density` applies at any
+ * row over a tile of 128 batch rows, and the kernels that evaluate every term; both give the same bits (positions
+ * included).  Built-in limit 0.10, and the table is only built for layers of at least 2^24 terms; a positive `density` applies at any
  * size.  No reference counterpart (core/cuda/sort_neuron.cu evaluates every term). */
 int sd_set_sort_candidate_density(float density);
 /* The same for sd_inf_dist_forward[_nograd] (no index lists) and sd_masked_inf_dist_forward (factored mask) on dense

@@ -1,6 +1,7 @@
 // Sort neuron and its interval bounds from per-weight-row candidate tables (see sort_cols.h).
 #include "sort_cols.h"
 #include <type_traits>
+#include <utility>
 #include "fwd_tile.h"
 
 namespace sd {
@@ -455,7 +456,7 @@ sc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
         int cnt = 0;   // marks in the list
         float wreg[2];
         X xa[2][4], xb[2][4];
-        auto load = [&](int buf, int k0, int total) {
+        auto load = [&](int buf, int k0, int total) __attribute__((always_inline)) {
             int k = k0 + (lane & 3);
             k = k < total ? k : total - 1;
             const int nn = (int)mine[k];
@@ -467,7 +468,7 @@ sc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
                 xb[buf][i] = xcol[(size_t)n * Bp + 64];
             }
         };
-        auto compute = [&](int buf, int k0, int total) {
+        auto compute = [&](int buf, int k0, int total) __attribute__((always_inline)) {
             #pragma unroll
             for (int i = 0; i < 4; i++) {
                 if (k0 + i < total) {   // wave-uniform
@@ -487,7 +488,7 @@ sc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
             }
         };
         // walks the list, the loads of a group in flight while the group before it is used
-        auto walk = [&](int total) {
+        auto walk = [&](int total) __attribute__((always_inline)) {
             if (total == 0) return;
             load(0, 0, total);
             for (int k0 = 0; k0 < total; k0 += 8) {
@@ -575,7 +576,7 @@ mc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
         float wreg[2];
         int nreg[2];
         float xa[2][4], xb[2][4];
-        auto load = [&](int buf, int k0, int total) {
+        auto load = [&](int buf, int k0, int total) __attribute__((always_inline)) {
             int k = k0 + (lane & 3);
             k = k < total ? k : total - 1;
             const int nn = (int)mine[k];
@@ -588,7 +589,7 @@ mc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
                 xb[buf][i] = xcol[(size_t)n * Bp + 64];
             }
         };
-        auto compute = [&](int buf, int k0, int total) {
+        auto compute = [&](int buf, int k0, int total) __attribute__((always_inline)) {
             #pragma unroll
             for (int i = 0; i < 4; i++) {
                 if (k0 + i < total) {   // wave-uniform
@@ -601,7 +602,7 @@ mc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
                 }
             }
         };
-        auto walk = [&](int total) {
+        auto walk = [&](int total) __attribute__((always_inline)) {
             if (total == 0) return;
             load(0, 0, total);
             for (int k0 = 0; k0 < total; k0 += 8) {
@@ -612,7 +613,7 @@ mc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
             }
         };
         // one pass over the weight row: `words` = its table words, or (second pass) the inputs it keeps
-        auto pass = [&](const uint32_t* __restrict__ words) {
+        auto pass = [&](const uint32_t* __restrict__ words) __attribute__((always_inline)) {
             best[0] = best[1] = kEps;
             where[0] = where[1] = 0;
             int cnt = 0;
@@ -687,6 +688,11 @@ int run_max(const float* x, const float* w, const uint32_t* xkeep, const uint32_
     return check_launch("mc_main_kernel");
 }
 
+template <class F, int... R>
+__device__ __forceinline__ void static_for(F&& f, std::integer_sequence<int, R...>) {
+    (f(std::integral_constant<int, R>{}), ...);
+}
+
 // Value form with positions (core/cuda/sort_neuron.cu:111-214): as sc_main_kernel, with the ordered insertion that
 // carries the input numbers.  The marks of a row are walked in ascending input order, and every term that is at
 // least the final K-th largest value of an output is marked, so these terms meet the list in the order and against
@@ -719,7 +725,7 @@ sp_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
         float wreg[2];
         int nreg[2];
         float xa[2][4], xb[2][4];
-        auto load = [&](int buf, int k0, int total) {
+        auto load = [&](int buf, int k0, int total) __attribute__((always_inline)) {
             int k = k0 + (lane & 3);
             k = k < total ? k : total - 1;
             const int nn = (int)mine[k];
@@ -732,7 +738,7 @@ sp_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
                 xb[buf][i] = xcol[(size_t)n * Bp + 64];
             }
         };
-        auto compute = [&](int buf, int k0, int total) {
+        auto compute = [&](int buf, int k0, int total) __attribute__((always_inline)) {
             #pragma unroll
             for (int i = 0; i < 4; i++) {
                 if (k0 + i < total) {   // wave-uniform
@@ -744,7 +750,7 @@ sp_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
                 }
             }
         };
-        auto walk = [&](int total) {
+        auto walk = [&](int total) __attribute__((always_inline)) {
             if (total == 0) return;
             load(0, 0, total);
             for (int k0 = 0; k0 < total; k0 += 8) {
@@ -782,13 +788,16 @@ sp_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
         }
     }
     const size_t plane = (size_t)B * M;
-    // the values, then the K planes of positions (slot 0 = largest = res[K-1])
-    #pragma unroll
-    for (int round = 0; round <= K; round++) {
+    // the values, then the K planes of positions (slot 0 = largest = res[K-1]); the rounds are expanded at compile
+    // time so that the lists are only ever indexed with constants and stay in registers
+    static_for([&](auto R) __attribute__((always_inline)) {
+        constexpr int round = decltype(R)::value;
         if (m < M) {
             #pragma unroll
-            for (int j = 0; j < 2; j++)
-                stage[lane + 64 * j][wave] = round == 0 ? __builtin_bit_cast(int, geo_sum<K>(res[j], q)) : idx[j][K - round];
+            for (int j = 0; j < 2; j++) {
+                if constexpr (round == 0) stage[lane + 64 * j][wave] = __builtin_bit_cast(int, geo_sum<K>(res[j], q));
+                else stage[lane + 64 * j][wave] = idx[j][K - round];
+            }
         }
         __syncthreads();
         for (int e = tid; e < kTileB * kMainTile; e += 64 * kMainWaves) {
@@ -796,12 +805,12 @@ sp_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
             const int b = s * kTileB + bl, mm = mb * kMainTile + mloc;
             if (b < B && mm < M) {
                 const size_t o = (size_t)b * M + mm;
-                if (round == 0) y[o] = __builtin_bit_cast(float, stage[bl][mloc]);
+                if constexpr (round == 0) y[o] = __builtin_bit_cast(float, stage[bl][mloc]);
                 else pos[(size_t)(round - 1) * plane + o] = stage[bl][mloc];
             }
         }
         __syncthreads();
-    }
+    }, std::make_integer_sequence<int, K + 1>{});
 }
 
 template <int K, bool IV>
