@@ -24,6 +24,10 @@ def main():
     ap.add_argument("--ops", default="linf,mask,bwd,bound,sort,lp,shift,idx")
     ap.add_argument("--reps", type=int, default=5)
     ap.add_argument("--keep", type=float, default=0.3, help="keep probability of the index-list rows")
+    ap.add_argument("--data", choices=["config", "unit"], default="config",
+                    help="config: inputs ~ U[0,1], weights ~ N(0, 1/N) (the benchmark configurations); unit: weights ~ "
+                         "N(0, 1) as the reference initialises them against batch rows that are alike (centred "
+                         "activations): the regime of the candidate-table kernels")
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
     import torch
@@ -31,8 +35,12 @@ def main():
     dev = torch.device("cuda:0")
     B, N, M = args.shape
     g = torch.Generator().manual_seed(0)
-    x = torch.rand(B, N, 1, generator=g).to(dev)
-    w = (torch.randn(M, N, generator=g) * N ** -0.5).to(dev)
+    if args.data == "unit":
+        x = (torch.randn(1, N, 1, generator=g) * 0.3 + torch.randn(B, N, 1, generator=g) * 0.1).contiguous().to(dev)
+        w = torch.randn(M, N, generator=g).to(dev)
+    else:
+        x = torch.rand(B, N, 1, generator=g).to(dev)
+        w = (torch.randn(M, N, generator=g) * N ** -0.5).to(dev)
     gy = torch.randn(B, M, 1, generator=g).to(dev)
     xn = torch.randn(B, N, 1, generator=g).to(dev)
     xl, xu = (x - 2 / 255).contiguous(), (x + 2 / 255).contiguous()
