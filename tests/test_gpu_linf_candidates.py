@@ -80,7 +80,7 @@ def _check_masked(oracle, x, w, q, seed, tag):
     assert np.array_equal(y2.cpu().numpy(), ry), tag
 
 
-SHAPES = [(70, 96, 64), (33, 2048, 300), (130, 1024, 513), (1, 32, 1), (257, 320, 129), (512, 2112, 96)]
+SHAPES = [(70, 96, 64), (33, 2048, 300), (130, 1024, 513), (1, 32, 1), (257, 320, 129), (700, 160, 72), (512, 2112, 96)]
 
 
 @pytest.mark.parametrize("dens", [1.0, 0.0, -1.0])

@@ -82,7 +82,7 @@ def _check(oracle, density, dens, x, xl, xu, w, q, K, tag):
 
 
 @pytest.mark.parametrize("dens", [1.0, 0.0, -1.0])
-@pytest.mark.parametrize("B,CI,CO", [(70, 96, 64), (33, 2048, 300), (130, 1024, 513), (1, 32, 1), (257, 320, 129),
+@pytest.mark.parametrize("B,CI,CO", [(70, 96, 64), (33, 2048, 300), (130, 1024, 513), (1, 32, 1), (257, 320, 129), (700, 160, 72),
                                      (512, 1088, 96)])
 def test_sort_candidate_kernels_match_oracle(oracle, density, dens, B, CI, CO):
     """Ragged batch tiles (B not a multiple of 128) and weight rows (CO not a multiple of 32 / 64 / 128), rows of
