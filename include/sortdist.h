@@ -71,6 +71,12 @@ int sd_set_lp_candidate_density(float density);
  * that evaluates every term; both give the same bits.  Built-in limit 0.26.  No reference counterpart
  * (core/cuda/bound_inf_dist_cuda.cu evaluates every term). */
 int sd_set_bound_candidate_density(float density);
+/* Which table kernel serves sd_bound_inf_dist_forward_nograd: 1 = the one that stages tiles of inputs and weights
+ * through LDS (marked shares of a few per cent and more), 2 = the one that walks a weight row's marks over a
+ * transposed copy of the inputs (marked shares below about 1 %: weights of unit scale against batch rows that are
+ * alike), 0 (default) = 1 until a layer has reported that few marks three calls in a row, then 2 for 31 calls.  Same
+ * bits whichever runs. */
+int sd_set_bound_candidate_form(int form);
 /* The same for sd_sort_neuron_forward[_nograd] and sd_bound_sort_neuron_forward on dense single-group layers (CI a
  * multiple of 32): a kernel that works from a table of the inputs that can be among the K largest terms of a weight
  * row over a tile of 128 batch rows, and the kernels that evaluate every term; both give the same bits (positions

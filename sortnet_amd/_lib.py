@@ -48,6 +48,7 @@ _OTHER = {
     "sd_last_forward_kernel": ([], ctypes.c_char_p),
     "sd_set_lp_candidate_density": ([_f], _i),
     "sd_set_bound_candidate_density": ([_f], _i),
+    "sd_set_bound_candidate_form": ([_i], _i),
     "sd_set_sort_candidate_density": ([_f], _i),
     "sd_set_linf_candidate_density": ([_f], _i),
     "sd_set_linf_candidate_depth": ([_i], _i),
@@ -107,6 +108,14 @@ def set_bound_candidate_density(density):
     rc = lib.sd_set_bound_candidate_density(float(density))
     if rc != 0:
         raise RuntimeError("sd_set_bound_candidate_density failed: %s" % lib.sd_last_error().decode())
+
+
+def set_bound_candidate_form(form):
+    """Table kernel of the dense interval forward: 0 chosen per layer, 1 staged tiles, 2 walk over transposed inputs."""
+    lib = load()
+    rc = lib.sd_set_bound_candidate_form(int(form))
+    if rc != 0:
+        raise RuntimeError("sd_set_bound_candidate_form failed: %s" % lib.sd_last_error().decode())
 
 
 def set_sort_candidate_density(density):

@@ -528,7 +528,8 @@ __global__ void __launch_bounds__(256) table_kernel(const float* __restrict__ xl
 }
 
 // count[0] = marks of the table per weight row, count[1] = of the table per batch row (the one that was not built
-// counts as full), count[2] = 1 when neither is below its limit, which is what the every-term kernel waits for
+// counts as full), count[2] = 1 when neither is below its limit, which is what the every-term kernel waits for,
+// count[3] = 1 when the per-weight-row marks are below a sixteenth of their limit (for the caller's choice of kernel)
 __global__ void __launch_bounds__(1024) sum_tables_kernel(const uint32_t* __restrict__ partial, size_t n_col,
                                                           size_t n_row, unsigned long long* __restrict__ count,
                                                           const float* __restrict__ stat, int S,
@@ -549,6 +550,8 @@ __global__ void __launch_bounds__(1024) sum_tables_kernel(const uint32_t* __rest
         count[0] = c;
         count[1] = r;
         count[2] = (c > limit_col && r > limit_row) ? 1ull : 0ull;
+        // so few marks per weight row that staging tiles through LDS is most of the main kernel's time
+        count[3] = c <= limit_col / 16 ? 1ull : 0ull;
     }
 }
 

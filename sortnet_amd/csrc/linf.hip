@@ -15,7 +15,9 @@ static float g_bound_density = -1.f;
 // cycles per marked (tile, weight row, input)) and the table 0.08 ms, against 1.04 ms for every term
 // (the table is paid for by the time the choice is made: the limit sits where 0.14 + 3.3 x share meets 1.04)
 constexpr float kBoundColsCap = 0.26f;
-constexpr int kHintSiteBound = 1;
+constexpr int kHintSiteBound = 1, kHintSiteBoundSparse = 8;
+constexpr float kBoundSparseCap = 0.03f;   // marked share up to which the kernel without LDS staging runs
+static int g_bound_form = 0;              // 0: chosen per layer, 1: staged tiles, 2: transposed-row walk
 
 // The l-inf forward (plain, and under the factored mask) on dense single-group layers queues a kernel that works from
 // per-weight-row candidate tables in front of the kernels that evaluate every term; a count taken on the device
@@ -303,6 +305,26 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
     // with the built-in limit, a layer whose tables have not paid lately is not given any for a while
     const bool hinted = cols && g_bound_density < 0.f;
     if (hinted && !hint_build_tables(kHintSiteBound, weight, B, CO, CI, st)) cols = false;
+    // Very few marks (weights of unit scale against rows that are alike: below 1 %): the staged kernel would spend its
+    // time moving tiles through LDS, and the kernel that walks a weight row's marks over a transposed copy of the
+    // inputs serves better.  Chosen by hand (sd_set_bound_candidate_form) or, with the built-in limit, for a layer
+    // whose last three staged calls reported that few marks ("not building" the staged tables, in the hint's terms).
+    bool sparse = cols && g_bound_form == 2 && CI <= 65536;
+    if (cols && g_bound_form == 0 && hinted && CI <= 65536)
+        sparse = !hint_build_tables(kHintSiteBoundSparse, weight, B, CO, CI, st);
+    if (sparse) {
+        void* ws = workspace(sort_cols_workspace(B, CO, CI, 1), st);   // the only request of this call
+        if (!ws) return SD_ERR_HIP;
+        if (a.nsplit > 1) {   // the every-term kernel, should it run, merges its slices into zeros
+            if ((rc = fill_zero(outputL, (size_t)B * CO * HW, st))) return rc;
+            if ((rc = fill_zero(outputU, (size_t)B * CO * HW, st))) return rc;
+        }
+        if ((rc = sort_cols_forward(inputL, inputU, weight, B, CO, CI, 0.f, 1, outputL, outputU, nullptr, ws,
+                                    g_bound_density > 0.f ? g_bound_density : kBoundSparseCap, &a.gate, &a.gate_limit, st)))
+            return rc;
+        a.gate_above = 1;
+        return TB == 2 ? launch_fwd<BoundNogradGated, 2, 8>(a, st) : launch_fwd<BoundNogradGated, 4, 8>(a, st);
+    }
     if (a.nsplit > 1 || cols) {
         if ((rc = fill_zero(outputL, (size_t)B * CO * HW, st))) return rc;
         if ((rc = fill_zero(outputU, (size_t)B * CO * HW, st))) return rc;
@@ -314,7 +336,10 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
             return rc;
         a.gate_above = 1;
         rc = TB == 2 ? launch_fwd<BoundNogradGated, 2, 8>(a, st) : launch_fwd<BoundNogradGated, 4, 8>(a, st);
-        if (hinted && rc == SD_OK) hint_record(kHintSiteBound, weight, B, CO, CI, a.gate, st);   // the gate is 1 when every term ran
+        if (hinted && rc == SD_OK) {
+            hint_record(kHintSiteBound, weight, B, CO, CI, a.gate, st);   // the gate is 1 when every term ran
+            if (g_bound_form == 0) hint_record(kHintSiteBoundSparse, weight, B, CO, CI, a.gate + 1, st);   // 1: very few marks
+        }
         return rc;
     }
     if (TB == 2) return launch_fwd<BoundNograd, 2, 8>(a, st);
@@ -324,6 +349,12 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
 extern "C" int sd_set_bound_candidate_density(float density) {
     SD_REQUIRE(density <= 1.f, "set_bound_candidate_density: %g is above 1", (double)density);
     g_bound_density = density;
+    return SD_OK;
+}
+
+extern "C" int sd_set_bound_candidate_form(int form) {
+    SD_REQUIRE(form >= 0 && form <= 2, "set_bound_candidate_form: %d is not 0 (automatic), 1 (staged tiles) or 2 (row walk)", form);
+    g_bound_form = form;
     return SD_OK;
 }
 

@@ -22,7 +22,8 @@ size_t sort_cols_workspace(int B, int CO, int CI, int K);
 // Builds the table, counts its marks on the device and queues the table kernel so that it runs only when at most
 // `density` of all (tile, weight row, input) triples are marked; the caller queues the kernels that evaluate every
 // term with the opposite condition on the same counter (*gate, *gate_limit); (*gate)[1] is 1 when those are to run.
-//   xu != nullptr: interval form, outL / outU receive the bounds;
+//   xu != nullptr: interval form, outL / outU receive the bounds; with K = 1 these are the interval bounds of the
+//   l-inf distance (maxima with the 1e-10 floor, q unused), for layers whose marks are too few to stage tiles for;
 //   xu == nullptr: value form on xl, outU receives the values (outL is not used) and pos, if not null, the K planes
 //   of positions (K, B, CO), largest first.
 int sort_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float q, int K,

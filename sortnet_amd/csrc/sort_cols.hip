@@ -418,7 +418,9 @@ __global__ void __launch_bounds__(1024) sc_sum_kernel(const uint32_t* __restrict
 // loads of the next four in flight): per mark one weight (a wave-uniform load), one transposed row of inputs (two
 // coalesced loads) and the insertions into the top-K lists, which are the single-pass kernel's (branch-free medians; same terms, same lists).  The
 // results of the workgroup leave through LDS, 128 bytes wide.
-template <int K, bool IV>
+// MAXFORM (K = 1, interval form): the lists are the running maxima of the interval bounds of the l-inf distance
+// (core/cuda/bound_inf_dist_cuda.cu:15-118), which leave as max(1e-10, .) instead of through the geometric sum.
+template <int K, bool IV, bool MAXFORM = false>
 __global__ void __launch_bounds__(64 * kMainWaves)
 sc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const uint32_t* __restrict__ bits,
                const unsigned long long* __restrict__ count, unsigned long long limit, int B, int Bp, int M, int Mp,
@@ -473,7 +475,16 @@ sc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
             for (int i = 0; i < 4; i++) {
                 if (k0 + i < total) {   // wave-uniform
                     const float wi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wreg[buf]), i));
-                    if constexpr (IV) {
+                    if constexpr (IV && MAXFORM) {
+                        // a term with an undefined operand is dropped (min / max keep the defined one, as the
+                        // reference's do; the final max with 0 drops a term that is undefined altogether)
+                        const float a1 = wi - xa[buf][i].x, a2 = xa[buf][i].y - wi;
+                        const float b1 = wi - xb[buf][i].x, b2 = xb[buf][i].y - wi;
+                        insert_bits<K>(lo[0], fmaxf(-fminf(a1, a2), 0.f));
+                        insert_bits<K>(hi[0], fmaxf(fmaxf(a1, a2), 0.f));
+                        insert_bits<K>(lo[1], fmaxf(-fminf(b1, b2), 0.f));
+                        insert_bits<K>(hi[1], fmaxf(fmaxf(b1, b2), 0.f));
+                    } else if constexpr (IV) {
                         const float a1 = wi - xa[buf][i].x, a2 = xa[buf][i].y - wi;
                         const float b1 = wi - xb[buf][i].x, b2 = xb[buf][i].y - wi;
                         insert_bits<K>(lo[0], -fminf(a1, a2));
@@ -527,8 +538,14 @@ sc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
         }
         #pragma unroll
         for (int j = 0; j < 2; j++) {
-            stage[0][lane + 64 * j][ml] = geo_sum_bits<K>(hi[j], q);
-            if constexpr (IV) stage[1][lane + 64 * j][ml] = geo_sum_bits<K>(lo[j], q);
+            if constexpr (MAXFORM) {
+                static_assert(!MAXFORM || (K == 1 && IV), "the maximum form is the interval form with one entry");
+                stage[0][lane + 64 * j][ml] = fmaxf(__builtin_bit_cast(float, hi[j][0]), kEps);
+                stage[1][lane + 64 * j][ml] = fmaxf(__builtin_bit_cast(float, lo[j][0]), kEps);
+            } else {
+                stage[0][lane + 64 * j][ml] = geo_sum_bits<K>(hi[j], q);
+                if constexpr (IV) stage[1][lane + 64 * j][ml] = geo_sum_bits<K>(lo[j], q);
+            }
         }
     }
     __syncthreads();
@@ -813,7 +830,7 @@ sp_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
     }, std::make_integer_sequence<int, K + 1>{});
 }
 
-template <int K, bool IV>
+template <int K, bool IV, bool MAXFORM = false>
 int run(const float* xl, const float* xu, const float* w, int B, int M, int N, float q, float* outL, float* outU,
         int* pos, const Carve& c, unsigned long long limit, hipStream_t st) {
     const int S = tiles_b(B), Bp = S * kTileB, Mp = mpad_of(M), NCH = N / kChunk, slices = slices_of(NCH);
@@ -837,7 +854,7 @@ int run(const float* xl, const float* xu, const float* w, int B, int M, int N, f
             return check_launch("sp_main_kernel");
         }
     }
-    hipLaunchKernelGGL((sc_main_kernel<K, IV>), dim3((unsigned)(S * (Mp / kMainTile))), dim3(64 * kMainWaves), 0, st,
+    hipLaunchKernelGGL((sc_main_kernel<K, IV, MAXFORM>), dim3((unsigned)(S * (Mp / kMainTile))), dim3(64 * kMainWaves), 0, st,
                        c.xT, w, c.bits, c.count, limit, B, Bp, M, Mp, N, q, outL, outU);
     return check_launch("sc_main_kernel");
 }
@@ -865,6 +882,7 @@ int sort_cols_forward(const float* xl, const float* xu, const float* w, int B, i
     const unsigned long long limit = (unsigned long long)((double)tiles_b(B) * CO * CI * d);
     *gate = c.count;
     *gate_limit = limit;
+    if (K == 1 && xu) return run<1, true, true>(xl, xu, w, B, CO, CI, q, outL, outU, nullptr, c, limit, st);
     switch (K) {
 #define X(k) case k: return xu ? run<k, true>(xl, xu, w, B, CO, CI, q, outL, outU, nullptr, c, limit, st) \
                                : run<k, false>(xl, nullptr, w, B, CO, CI, q, outL, outU, pos, c, limit, st);

@@ -24,10 +24,12 @@ def _dev():
 def density():
     from sortnet_amd import _lib
 
-    def set_(d):
+    def set_(d, form=0):
         _lib.set_bound_candidate_density(d)
+        _lib.set_bound_candidate_form(form)
     yield set_
     _lib.set_bound_candidate_density(-1.0)
+    _lib.set_bound_candidate_form(0)
 
 
 def _intervals(B, CI, kind, seed):
@@ -46,15 +48,15 @@ def _intervals(B, CI, kind, seed):
     return xl, xu
 
 
-@pytest.mark.parametrize("dens", [1.0, 0.0, -1.0])
+@pytest.mark.parametrize("dens,form", [(1.0, 1), (1.0, 2), (0.0, 0), (-1.0, 0), (-1.0, 2)])
 @pytest.mark.parametrize("B,CI,CO", [(70, 96, 64), (33, 2048, 300), (130, 1024, 513), (1, 32, 1), (257, 320, 129),
-                                     (512, 512, 640)])
-def test_bound_candidate_kernel_matches_oracle(oracle, density, dens, B, CI, CO):
+                                     (512, 512, 640), (700, 160, 72)])
+def test_bound_candidate_kernel_matches_oracle(oracle, density, dens, form, B, CI, CO):
     """Ragged batch tiles (B not a multiple of 128) and weight tiles (CO not a multiple of 128), one and several of
-    each, input ranges cut in slices or not."""
+    each, input ranges cut in slices or not; both table kernels (staged tiles, walk over transposed inputs)."""
     from sortnet_amd import ext
     dev = _dev()
-    density(dens)
+    density(dens, form)
     for kind in ("rows_alike", "random", "inverted", "images"):
         for wscale in (0.02, 1.0):
             xl, xu = _intervals(B, CI, kind, B + CI)
@@ -64,21 +66,21 @@ def test_bound_candidate_kernel_matches_oracle(oracle, density, dens, B, CI, CO)
             yl = torch.full((B, CO, 1), float("nan"), device=dev)
             yu = torch.full((B, CO, 1), float("nan"), device=dev)
             ext.bound_inf_dist_forward_nograd(xl.to(dev), xu.to(dev), w.to(dev), yl, yu, 1)
-            tag = "dens=%g %s wscale=%g" % (dens, kind, wscale)
+            tag = "dens=%g form=%d %s wscale=%g" % (dens, form, kind, wscale)
             assert np.array_equal(yl.cpu().numpy(), rl), tag
             assert np.array_equal(yu.cpu().numpy(), ru), tag
 
 
-@pytest.mark.parametrize("dens", [1.0, 0.0])
+@pytest.mark.parametrize("dens,form", [(1.0, 1), (1.0, 2), (0.0, 0)])
 @pytest.mark.parametrize("kind", ["rows_alike", "images"])
-def test_bound_candidate_kernel_undefined_and_infinite_entries(oracle, density, dens, kind):
+def test_bound_candidate_kernel_undefined_and_infinite_entries(oracle, density, dens, form, kind):
     """A term with an undefined operand is dropped by the reference's strict compares (an interval with one
     undefined end keeps the other end's term), so a row that holds NaN where its neighbours hold their maximum has
     a smaller result than they do: the tables must not conclude anything from such a column.  Infinite ends and
     weights likewise.  Both orientations of the table (rows alike / images) and the every-term kernel."""
     from sortnet_amd import ext
     dev = _dev()
-    density(dens)
+    density(dens, form)
     B, CI, CO = 200, 256, 150
     xl, xu = _intervals(B, CI, kind, 5)
     g = torch.Generator().manual_seed(6)
@@ -119,13 +121,13 @@ def test_bound_candidate_kernel_at_layer_size(density):
     xl, xu = (x - r).contiguous().to(dev), (x + r).contiguous().to(dev)
     w = (torch.randn(M, N, generator=g) * N ** -0.5).contiguous().to(dev)
     out = {}
-    for dens in (0.0, 1.0, -1.0):
-        density(dens)
+    for dens, form in ((0.0, 0), (1.0, 1), (-1.0, 0), (1.0, 2)):
+        density(dens, form)
         yl, yu = torch.empty(B, M, 1, device=dev), torch.empty(B, M, 1, device=dev)
         ext.bound_inf_dist_forward_nograd(xl, xu, w, yl, yu, 1)
-        out[dens] = (yl, yu)
-    for dens in (1.0, -1.0):
-        assert torch.equal(out[dens][0], out[0.0][0]) and torch.equal(out[dens][1], out[0.0][1]), dens
+        out[(dens, form)] = (yl, yu)
+    for key in ((1.0, 1), (-1.0, 0), (1.0, 2)):
+        assert torch.equal(out[key][0], out[(0.0, 0)][0]) and torch.equal(out[key][1], out[(0.0, 0)][1]), key
 
 
 def test_bound_results_do_not_depend_on_the_table_hint(oracle, density):
