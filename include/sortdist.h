@@ -86,7 +86,7 @@ int sd_set_sort_candidate_density(float density);
 /* The same for sd_inf_dist_forward[_nograd] (no index lists) and sd_masked_inf_dist_forward (factored mask) on dense
  * single-group layers (CI a multiple of 32, at most 65536): a kernel that works from a table of the inputs that can hold
  * the maximum of a weight row over a tile of 128 batch rows, and the kernels that evaluate every term; same values and
- * positions either way.  Built-in limit 0.10, layers of at least 2^24 terms.  Under the mask the table's bound rests on
+ * positions either way.  Built-in limit 0.10, layers of at least 2^31 terms.  Under the mask the table's bound rests on
  * `depth` inputs per weight row, chosen so that a batch row keeps none of them less than once in 10^4 outputs (such an
  * output is recomputed from every input); sd_set_linf_candidate_depth overrides the choice (0 = automatic; 8, 12, 16,
  * 20 or 24).  No reference counterpart (core/cuda/inf_dist_cuda.cu evaluates every term). */

@@ -26,7 +26,7 @@ static int g_bound_form = 0;              // 0: chosen per layer, 1: staged tile
 static float g_linf_density = -1.f;
 static int g_linf_depth = 0;   // under the mask: inputs the bound of a weight row rests on (0 = from the keep probability)
 constexpr float kMaxColsCap = 0.10f;
-constexpr long long kMaxColsMinTerms = 1ll << 24;
+constexpr long long kMaxColsMinTerms = 1ll << 31;   // below, the tables cost more than evaluating every term
 constexpr int kHintSiteLinf = 4, kHintSiteMasked = 5;
 
 // depth of the tables' bound (0 = no tables for this call)

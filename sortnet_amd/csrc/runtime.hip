@@ -72,12 +72,13 @@ void* workspace(size_t bytes, hipStream_t stream) {
 }
 
 namespace {
+constexpr int kHintRing = 4;   // outcomes of a layer that may be on their way to the host at once
 struct HintSlot {
     int dev, site, B, CO, CI;
     const void* weight;         // the layer: same shapes with other weights are other layers
-    unsigned long long* host;   // pinned: the flag of the last recorded call
-    hipEvent_t ev;
-    bool pending;               // a copy is queued and not yet looked at
+    unsigned long long* host;   // pinned: kHintRing flags
+    hipEvent_t ev[kHintRing];   // recorded behind the copy of flag i
+    int head, queued;           // oldest outcome not yet looked at, and how many are queued
     int streak, skip_left;
 };
 std::mutex g_hint_mu;
@@ -95,13 +96,16 @@ HintSlot* hint_slot(int site, const void* weight, int B, int CO, int CI, bool cr
     for (HintSlot& h : g_hints)
         if (h.dev == dev && h.site == site && h.weight == weight && h.B == B && h.CO == CO && h.CI == CI) return &h;
     if (!create || g_hints.size() >= 256) return nullptr;
-    HintSlot h{dev, site, B, CO, CI, weight, nullptr, nullptr, false, 0, 0};
-    if (hipHostMalloc(reinterpret_cast<void**>(&h.host), sizeof(unsigned long long), hipHostMallocDefault) != hipSuccess ||
-        hipEventCreateWithFlags(&h.ev, hipEventDisableTiming) != hipSuccess) {
+    HintSlot h{};
+    h.dev = dev; h.site = site; h.B = B; h.CO = CO; h.CI = CI; h.weight = weight;
+    if (hipHostMalloc(reinterpret_cast<void**>(&h.host), kHintRing * sizeof(unsigned long long), hipHostMallocDefault) != hipSuccess) {
         (void)hipGetLastError();
         return nullptr;
     }
-    *h.host = 0;
+    for (int i = 0; i < kHintRing; i++) {
+        h.host[i] = 0;
+        if (hipEventCreateWithFlags(&h.ev[i], hipEventDisableTiming) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    }
     g_hints.push_back(h);
     return &g_hints.back();
 }
@@ -112,15 +116,15 @@ bool hint_build_tables(int site, const void* weight, int B, int CO, int CI, hipS
     std::lock_guard<std::mutex> lock(g_hint_mu);
     HintSlot* h = hint_slot(site, weight, B, CO, CI, false);
     if (!h) return true;
-    if (h->pending) {
-        const hipError_t e = hipEventQuery(h->ev);
-        if (e == hipSuccess) {
-            h->pending = false;
-            h->streak = *h->host != 0ull ? h->streak + 1 : 0;
-            // the streak is long enough (or the probe after a stretch without tables came out the same): no tables
-            // for the next kHintSkip calls, then one call probes again
-            h->skip_left = h->streak >= kHintStreak ? kHintSkip : 0;
-        } else (void)hipGetLastError();   // not ready: look again at the next call
+    // outcomes that have arrived, oldest first (the host may run several calls ahead of the device)
+    while (h->queued > 0) {
+        if (hipEventQuery(h->ev[h->head]) != hipSuccess) { (void)hipGetLastError(); break; }   // not ready: next call
+        h->streak = h->host[h->head] != 0ull ? h->streak + 1 : 0;
+        // the streak is long enough (or the probe after a stretch without tables came out the same): no tables
+        // for the next kHintSkip calls, then one call probes again
+        h->skip_left = h->streak >= kHintStreak ? kHintSkip : 0;
+        h->head = (h->head + 1) % kHintRing;
+        h->queued--;
     }
     if (h->skip_left > 0) { h->skip_left--; return false; }
     return true;
@@ -131,13 +135,14 @@ void hint_record(int site, const void* weight, int B, int CO, int CI, const unsi
     if (capturing(stream)) return;
     std::lock_guard<std::mutex> lock(g_hint_mu);
     HintSlot* h = hint_slot(site, weight, B, CO, CI, true);
-    if (!h || h->pending) return;
-    if (hipMemcpyAsync(h->host, every_term_ran, sizeof(unsigned long long), hipMemcpyDeviceToHost, stream) != hipSuccess ||
-        hipEventRecord(h->ev, stream) != hipSuccess) {
+    if (!h || h->queued == kHintRing) return;
+    const int i = (h->head + h->queued) % kHintRing;
+    if (hipMemcpyAsync(h->host + i, every_term_ran, sizeof(unsigned long long), hipMemcpyDeviceToHost, stream) != hipSuccess ||
+        hipEventRecord(h->ev[i], stream) != hipSuccess) {
         (void)hipGetLastError();
         return;
     }
-    h->pending = true;
+    h->queued++;
 }
 
 __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t* __restrict__ p, size_t n) {
