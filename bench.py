@@ -409,16 +409,17 @@ def main():
         sec = {}
         short, warm = max(3, args.steps // 4), 2
 
-        def masked_entry(mask, q, **kw):
-            r = run_masked(args, mask, q, short, warm, **kw)
-            return {"ms_per_step": r["ms_per_step"], "samples_per_s": r["samples_per_s"], "steps": short,
+        def masked_entry(mask, q, steps=short, warmup=warm, **kw):
+            r = run_masked(args, mask, q, steps, warmup, **kw)
+            return {"ms_per_step": r["ms_per_step"], "samples_per_s": r["samples_per_s"], "steps": steps,
                     "phase_ms": r["phase_ms"]}
 
         other = "term" if args.mask == "factored" else "factored"
         sec[other + "_mask"] = dict(masked_entry(other, args.q), workload=workload_text(args, other, args.q))
         sec["q1"] = dict(masked_entry(args.mask, 1.0), workload=workload_text(args, args.mask, 1.0))
         # the same step from the reference's own initialisation (weights of unit scale, core/models/norm_dist.py:30)
-        sec["unit_weights"] = dict(masked_entry(args.mask, args.q, weight_std=1.0),
+        # (enough steps for the layers to have settled on their kernels: a layer reports three calls before it switches)
+        sec["unit_weights"] = dict(masked_entry(args.mask, args.q, steps=max(short, 12), warmup=4, weight_std=1.0),
                                    workload=workload_text(args, args.mask, args.q).replace("N(0, 1/fan_in)", "N(0, 1)")
                                    + " as the reference initialises them")
         # the reference's own training form at the keep probability of its published commands (0.7-0.85)
