@@ -9,7 +9,8 @@ constexpr int kChunk = kColsChunk;   // inputs per table word
 constexpr int kTileB = 128;          // batch rows of a tile: 64 lanes x 2
 constexpr int kTileW = 128;          // weight rows of a workgroup of the main kernel: 16 wavefronts x 8
 constexpr int kLowSlices = 8;        // slices of the input range in the two table kernels
-constexpr int kSegChunks = 64;       // chunks whose table words the main kernel keeps in LDS at a time
+constexpr int kSegChunks = 64;       // chunks whose table words the per-batch-row main kernel keeps in LDS at a time
+constexpr int kStage = 64;           // inputs of one LDS stage of the per-weight-row main kernel (two table words)
 
 inline size_t align256(size_t b) { return (b + 255) / 256 * 256; }
 inline int tiles_b(int B) { return (B + kTileB - 1) / kTileB; }
@@ -23,12 +24,13 @@ struct Carve {
     unsigned long long* count;   // [0] marks of the per-weight-row table, [1] of the per-batch-row table, [2] every-term kernel's turn
     uint32_t* bits;   // [S][NCH][Mp] (or [T][NCH][Bp]): bit i of a word = input 32 c + i may hold a maximum of that row in that tile
     uint32_t* partial;   // marks per wavefront of the table kernel
+    float* xt;        // [S][N][64][4] per batch tile and input: (l, l', u, u') of the tile's rows i and i + 64, repaired
 };
 
 inline int bpad_of(int B) { return (B + kTileB - 1) / kTileB * kTileB; }
 inline size_t maxz(size_t a, size_t b) { return a > b ? a : b; }
 
-size_t carve_sizes(int B, int M, int N, size_t (&sz)[6]) {
+size_t carve_sizes(int B, int M, int N, size_t (&sz)[7]) {
     const size_t S = tiles_b(B), Mp = mpad_of(M), Bp = bpad_of(B), T = Mp / kTileW, NCH = N / kChunk;
     sz[0] = align256(S * 4 * N * 4);                               // xr
     sz[1] = align256(T * 2 * N * 4);                               // wr
@@ -36,11 +38,12 @@ size_t carve_sizes(int B, int M, int N, size_t (&sz)[6]) {
     sz[3] = 256;                                                   // count
     sz[4] = align256(maxz(S * NCH * Mp, T * NCH * Bp) * 4);        // bits
     sz[5] = align256(maxz(Mp / 64, Bp / 64 * ((T + 3) / 4)) * kLowSlices * 4 * 4);   // partial
-    return sz[0] + sz[1] + sz[2] + sz[3] + sz[4] + sz[5];
+    sz[6] = align256(S * N * 1024);                                // xt
+    return sz[0] + sz[1] + sz[2] + sz[3] + sz[4] + sz[5] + sz[6];
 }
 
 Carve carve(void* ws, int B, int M, int N) {
-    size_t sz[6];
+    size_t sz[7];
     carve_sizes(B, M, N, sz);
     const size_t S = tiles_b(B), Mp = mpad_of(M), Bp = bpad_of(B), T = Mp / kTileW;
     char* p = static_cast<char*>(ws);
@@ -52,7 +55,8 @@ Carve carve(void* ws, int B, int M, int N) {
     p += sz[2];
     c.count = reinterpret_cast<unsigned long long*>(p); p += sz[3];
     c.bits = reinterpret_cast<uint32_t*>(p); p += sz[4];
-    c.partial = reinterpret_cast<uint32_t*>(p);
+    c.partial = reinterpret_cast<uint32_t*>(p); p += sz[5];
+    c.xt = reinterpret_cast<float*>(p);
     return c;
 }
 
@@ -239,118 +243,154 @@ __device__ __forceinline__ void col_table_body(const float* __restrict__ w, cons
 // ---- main kernel --------------------------------------------------------------------------
 // A workgroup of 16 wavefronts owns 128 batch rows x 128 weight rows and a slice of the inputs.  Lane l holds the
 // batch rows l and l + 64; wavefront v the weight rows 8 v .. 8 v + 7: 32 running minima / maxima per lane.  The
-// inputs go by in chunks of 32: the l, u and weight tiles (128 x 32 each) of the next-but-one chunk are in flight
-// while the current one is used from LDS (always issued, so that the number of loads in flight is the same on every
-// path; a chunk nobody marks re-reads one hot line).  In LDS an input's operands lie together: (l, l', u, u') of a
-// lane's two rows as one 16-byte word, the 128 weights of the input in a row, so that a marked (weight row, input)
-// pair costs a wavefront two LDS reads (its own word and the weight as a broadcast) and eight vector instructions,
-// the terms of the every-term kernel.  The results leave through an
-// LDS transpose (coalesced along the weight rows) and merge over the slices by atomic maximum.
-constexpr int kMainTileFloats = kChunk * (4 * 64 + 4 + kTileW + 4);   // l/u tile + weight tile of one chunk, either orientation
-constexpr int kMainWords = kSegChunks * kTileW;
+// inputs go by in stages of 64.  The (l, l', u, u') words of a lane's two rows come from a copy that xt_kernel has
+// laid out per tile and input the way they lie in LDS (repaired, 1 KB per input), so staging is four 16-byte copies
+// per work-item, fetched while the previous stage is used.  A wavefront's weights never enter LDS: lane n of register
+// r holds w[row r][input n of the stage], and a marked input's weight is read from its lane.  The two table words of
+// a (stage, weight row) are scalar loads.  A marked (weight row, input) pair then costs one 16-byte LDS read, one
+// lane read and the eight vector instructions of the terms; the operands of a row's next mark are fetched while the
+// current one is used.  The results leave through an LDS transpose (coalesced along the weight rows) and merge over
+// the slices by atomic maximum.
+constexpr int kStageFloats = kStage * 256;   // (l, l', u, u') of 64 lanes per input
+constexpr int kMainTileFloats = kChunk * (2 * kTileB + 4 + 2 * 64 + 4);   // per-batch-row main kernel: l/u tile + weight tile of one chunk
+constexpr int kMainWords = kSegChunks * kTileB;                            // and its table words
+constexpr int kLdsWords = 2 * kMainTileFloats + kMainWords > 2 * kStageFloats ? 2 * kMainTileFloats + kMainWords
+                                                                              : 2 * kStageFloats;
 
-__device__ __forceinline__ void bound_cols_body(const float* __restrict__ xl, const float* __restrict__ xu,
-                                                const float* __restrict__ w, const uint32_t* __restrict__ bits, int B,
-                                                int M, int Mp, int N, int nsplit, float* __restrict__ yL,
-                                                float* __restrict__ yU, float* smem, uint32_t* wb) {
+// (l, l', u, u') of the batch rows i and i + 64 of every tile, per input, repaired: the layout the main kernel keeps
+// in LDS, so that it stages a tile with 16-byte copies.  16 inputs per workgroup.
+__global__ void __launch_bounds__(256) xt_kernel(const float* __restrict__ xl, const float* __restrict__ xu, int B, int N,
+                                                 const unsigned long long* __restrict__ count,
+                                                 unsigned long long limit_col, float* __restrict__ xT) {
+    if (count[0] > limit_col) return;
+    __shared__ __attribute__((aligned(16))) float t[16 * 256];
+    const int n0 = blockIdx.x * 16, s = blockIdx.y;
+    const int row = threadIdx.x >> 1, half = threadIdx.x & 1;
+    const int b = s * kTileB + row < B ? s * kTileB + row : B - 1;
+    const float* pl = xl + (size_t)b * N + n0 + 8 * half;
+    const float* pu = xu + (size_t)b * N + n0 + 8 * half;
+    float4 l0 = *reinterpret_cast<const float4*>(pl), l1 = *reinterpret_cast<const float4*>(pl + 4);
+    float4 u0 = *reinterpret_cast<const float4*>(pu), u1 = *reinterpret_cast<const float4*>(pu + 4);
+    repair(l0.x, u0.x); repair(l0.y, u0.y); repair(l0.z, u0.z); repair(l0.w, u0.w);
+    repair(l1.x, u1.x); repair(l1.y, u1.y); repair(l1.z, u1.z); repair(l1.w, u1.w);
+    const float l[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
+    const float u[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+    float* d = t + (8 * half) * 256 + 4 * (row & 63) + (row >> 6);
+    #pragma unroll
+    for (int k = 0; k < 8; k++) { d[k * 256] = l[k]; d[k * 256 + 2] = u[k]; }
+    __syncthreads();
+    float4* dst = reinterpret_cast<float4*>(xT + ((size_t)s * N + n0) * 256);
+    const float4* src = reinterpret_cast<const float4*>(t);
+    #pragma unroll
+    for (int k = 0; k < 4; k++) dst[threadIdx.x + 256 * k] = src[threadIdx.x + 256 * k];
+}
+
+__device__ __forceinline__ void bound_cols_body(const float* __restrict__ xT, const float* __restrict__ w,
+                                                const uint32_t* __restrict__ bits, int B, int M, int Mp, int N,
+                                                int nsplit, float* __restrict__ yL, float* __restrict__ yU, float* smem) {
     constexpr int TW = 8;
-    constexpr int XROW = 4 * 64 + 4;     // floats per input in the l/u tile: 64 lanes x (l, l', u, u'), skewed by 4 banks
-    constexpr int WROW = kTileW + 4;     // floats per input in the weight tile
-    constexpr int kTileFloats = kChunk * (XROW + WROW);
-    static_assert(2 * kTileFloats >= kTileB * (kTileW + 1), "the transpose of the results fits where the tiles were");
-    static_assert(kTileFloats == kMainTileFloats, "LDS of the shared kernel");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int TM = (M + kTileW - 1) / kTileW, SB = (B + kTileB - 1) / kTileB, NCH = N / kChunk;
+    const int NST = (NCH + 1) / 2;
     const int mt = blockIdx.x % TM, s = (blockIdx.x / TM) % SB, split = blockIdx.x / (TM * SB);
     const int m0 = mt * kTileW, b0 = s * kTileB;
-    const int per = (NCH + nsplit - 1) / nsplit;
-    const int c_lo = split * per, c_hi = c_lo + per < NCH ? c_lo + per : NCH;
-    auto xt = [&](int buf) { return smem + buf * kTileFloats; };
-    auto wt = [&](int buf) { return smem + buf * kTileFloats + kChunk * XROW; };
+    const int per = (NST + nsplit - 1) / nsplit;
+    const int st_lo = split * per, st_hi = st_lo + per < NST ? st_lo + per : NST;
 
     float lo[TW][2], hi[TW][2];
     #pragma unroll
     for (int r = 0; r < TW; r++) { lo[r][0] = lo[r][1] = -kEps; hi[r][0] = hi[r][1] = kEps; }
 
-    // word of (chunk c, weight row m0 + i): bw[c * Mp + i]; rows past the last one, up to the padded count, hold zero.
-    // The words of up to kSegChunks chunks are copied to LDS ahead of the loop over them, so that no global load
-    // sits between two chunks.
-    const uint32_t* __restrict__ bw = bits + (size_t)s * NCH * Mp + m0;
-    int seg_lo = c_lo;
-    auto marked = [&](int c) {
-        const uint32_t* q = wb + (c - seg_lo) * kTileW;
-        return __builtin_amdgcn_ballot_w64((q[lane] | q[lane + 64]) != 0u) != 0ull;
-    };
-    const int frow = tid >> 3, fq = tid & 7;
-    const int fb = b0 + frow < B ? b0 + frow : B - 1, fm = m0 + frow < M ? m0 + frow : M - 1;
-    auto fetch = [&](int c, bool need, float4& l4, float4& u4, float4& w4) {
-        const size_t off = (size_t)c * kChunk + 4 * fq;
-        l4 = *reinterpret_cast<const float4*>(need ? xl + (size_t)fb * N + off : xl);
-        u4 = *reinterpret_cast<const float4*>(need ? xu + (size_t)fb * N + off : xu);
-        w4 = *reinterpret_cast<const float4*>(need ? w + (size_t)fm * N + off : w);
-    };
-    auto stash = [&](int buf, float4 l4, float4 u4, const float4& w4) {
-        repair(l4.x, u4.x); repair(l4.y, u4.y); repair(l4.z, u4.z); repair(l4.w, u4.w);
-        // row frow belongs to lane frow % 64, slot frow / 64 of (l, l', u, u')
-        float* dx = xt(buf) + (4 * fq) * XROW + 4 * (frow & 63) + (frow >> 6);
-        dx[0] = l4.x; dx[2] = u4.x;
-        dx[XROW] = l4.y; dx[XROW + 2] = u4.y;
-        dx[2 * XROW] = l4.z; dx[2 * XROW + 2] = u4.z;
-        dx[3 * XROW] = l4.w; dx[3 * XROW + 2] = u4.w;
-        float* dw = wt(buf) + (4 * fq) * WROW + frow;
-        dw[0] = w4.x; dw[WROW] = w4.y; dw[2 * WROW] = w4.z; dw[3 * WROW] = w4.w;
-    };
-    // The scalar unit is shared by the wavefronts of a compute unit, so the walk spends as few scalar instructions
-    // per marked input as it can: one loop per weight row over that row's own marks (find-first-set, clear, branch)
-    // instead of a walk over the union with a test per row.
-    auto compute = [&](int buf, int c) {
-        const float* X = xt(buf) + 4 * lane, *W = wt(buf) + wave * TW;
-        const uint4* rowwords = reinterpret_cast<const uint4*>(wb + (c - seg_lo) * kTileW + wave * TW);
-        const uint4 q0 = rowwords[0], q1 = rowwords[1];
-        const uint32_t words[TW] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    if (st_lo < st_hi) {
+        const float* __restrict__ xsrc = xT + (size_t)s * N * 256;
+        const size_t xlast = (size_t)N * 256 - 4;                       // the tile's last 16-byte word
+        const int mrow = m0 + wave * TW;
+        const uint32_t* __restrict__ bw = bits + (size_t)s * NCH * Mp + mrow;   // words of chunk c: bw[c * Mp + r]
+        size_t wrow[TW];
         #pragma unroll
-        for (int r = 0; r < TW; r++) {
-            uint32_t bm = __builtin_amdgcn_readfirstlane(words[r]);
-            while (bm) {
-                const int n = __builtin_ctz(bm);
-                bm &= bm - 1;
-                const float4 x = *reinterpret_cast<const float4*>(X + n * XROW);   // l, l', u, u' of the lane's two rows
-                const float wv = W[n * WROW + r];
-                const float a1 = wv - x.x, a2 = x.z - wv, b1 = wv - x.y, b2 = x.w - wv;
-                lo[r][0] = fminf(fminf(lo[r][0], a1), a2);
-                hi[r][0] = fmaxf(fmaxf(hi[r][0], a1), a2);
-                lo[r][1] = fminf(fminf(lo[r][1], b1), b2);
-                hi[r][1] = fmaxf(fmaxf(hi[r][1], b1), b2);
-            }
-        }
-    };
+        for (int r = 0; r < TW; r++) wrow[r] = (size_t)(mrow + r < M ? mrow + r : M - 1) * N;
 
-    for (; seg_lo < c_hi; seg_lo += kSegChunks) {
-        const int seg_hi = seg_lo + kSegChunks < c_hi ? seg_lo + kSegChunks : c_hi;
-        __syncthreads();   // the previous segment's words and tiles are no longer read
-        for (int e = tid; e < (seg_hi - seg_lo) * kTileW; e += 1024)
-            wb[e] = bw[(size_t)(seg_lo + (e >> 7)) * Mp + (e & (kTileW - 1))];
+        auto load_x = [&](int st, float4 (&v)[4]) __attribute__((always_inline)) {
+            #pragma unroll
+            for (int k = 0; k < 4; k++) {
+                size_t off = (size_t)st * kStageFloats + 4 * (size_t)(tid + 1024 * k);
+                if (off > xlast) off = xlast;                            // half stage at the end of the inputs
+                v[k] = *reinterpret_cast<const float4*>(xsrc + off);
+            }
+        };
+        auto store_x = [&](int buf, const float4 (&v)[4]) __attribute__((always_inline)) {
+            float4* d = reinterpret_cast<float4*>(smem + buf * kStageFloats);
+            #pragma unroll
+            for (int k = 0; k < 4; k++) d[tid + 1024 * k] = v[k];
+        };
+        auto load_w = [&](int st, float (&v)[TW]) __attribute__((always_inline)) {
+            const int n = st * kStage + lane < N ? st * kStage + lane : N - 1;
+            #pragma unroll
+            for (int r = 0; r < TW; r++) v[r] = w[wrow[r] + n];
+        };
+        auto load_words = [&](int st, uint32_t (&a)[TW], uint32_t (&b)[TW]) __attribute__((always_inline)) {
+            const int c0 = 2 * st, c1 = 2 * st + 1 < NCH ? 2 * st + 1 : 2 * st;
+            const uint32_t keep = 2 * st + 1 < NCH ? 0xffffffffu : 0u;
+            #pragma unroll
+            for (int r = 0; r < TW; r++) {
+                a[r] = bw[(size_t)c0 * Mp + r];
+                b[r] = bw[(size_t)c1 * Mp + r] & keep;
+            }
+        };
+        auto term = [&](float (&l2)[2], float (&h2)[2], const float4& x, float wv) __attribute__((always_inline)) {
+            const float a1 = wv - x.x, a2 = x.z - wv, b1 = wv - x.y, b2 = x.w - wv;
+            l2[0] = fminf(fminf(l2[0], a1), a2);
+            h2[0] = fmaxf(fmaxf(h2[0], a1), a2);
+            l2[1] = fminf(fminf(l2[1], b1), b2);
+            h2[1] = fmaxf(fmaxf(h2[1], b1), b2);
+        };
+        // a weight row's marks of the stage, in order; the operands of the next mark are on their way while the
+        // current one is used
+        auto compute = [&](int buf, const float (&wv)[TW], const uint32_t (&wa)[TW], const uint32_t (&wb2)[TW])
+                           __attribute__((always_inline)) {
+            const float* X = smem + buf * kStageFloats + 4 * lane;
+            #pragma unroll
+            for (int r = 0; r < TW; r++) {
+                unsigned long long bm = ((unsigned long long)wb2[r] << 32) | (unsigned long long)wa[r];
+                if (bm) {
+                    int n = __builtin_ctzll(bm);
+                    bm &= bm - 1;
+                    float4 xa = *reinterpret_cast<const float4*>(X + n * 256), xb;
+                    float va = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv[r]), n)), vb;
+                    while (true) {
+                        if (!bm) { term(lo[r], hi[r], xa, va); break; }
+                        n = __builtin_ctzll(bm);
+                        bm &= bm - 1;
+                        xb = *reinterpret_cast<const float4*>(X + n * 256);
+                        vb = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv[r]), n));
+                        term(lo[r], hi[r], xa, va);
+                        if (!bm) { term(lo[r], hi[r], xb, vb); break; }
+                        n = __builtin_ctzll(bm);
+                        bm &= bm - 1;
+                        xa = *reinterpret_cast<const float4*>(X + n * 256);
+                        va = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv[r]), n));
+                        term(lo[r], hi[r], xb, vb);
+                    }
+                }
+            }
+        };
+
+        float4 xs[4];
+        float wc[TW], wn[TW];
+        uint32_t a0[TW], a1[TW], n0[TW], n1[TW];
+        load_x(st_lo, xs); load_w(st_lo, wc); load_words(st_lo, a0, a1);
+        store_x(0, xs);
         __syncthreads();
-        float4 la, ua, wa, lb, ub, wc;
-        bool n0 = marked(seg_lo), n1 = seg_lo + 1 < seg_hi ? marked(seg_lo + 1) : false;
-        fetch(seg_lo, n0, la, ua, wa);
-        fetch(seg_lo + 1 < seg_hi ? seg_lo + 1 : seg_lo, n1, lb, ub, wc);
-        if (n0) stash(0, la, ua, wa);
-        __syncthreads();
-        for (int c = seg_lo; c < seg_hi; c += 2) {
-            const bool n2 = c + 2 < seg_hi ? marked(c + 2) : false;
-            fetch(c + 2 < seg_hi ? c + 2 : c, n2, la, ua, wa);
-            if (n0) compute(0, c);
-            if (n1) stash(1, lb, ub, wc);
+        for (int st = st_lo; st < st_hi; st++) {
+            const int buf = (st - st_lo) & 1;
+            const int nx = st + 1 < st_hi ? st + 1 : st;   // the last stage is fetched once more rather than behind a test
+            load_x(nx, xs); load_w(nx, wn); load_words(nx, n0, n1);
+            compute(buf, wc, a0, a1);
+            store_x(buf ^ 1, xs);
+            #pragma unroll
+            for (int r = 0; r < TW; r++) { wc[r] = wn[r]; a0[r] = n0[r]; a1[r] = n1[r]; }
             __syncthreads();
-            if (c + 1 >= seg_hi) break;
-            const bool n3 = c + 3 < seg_hi ? marked(c + 3) : false;
-            fetch(c + 3 < seg_hi ? c + 3 : c, n3, lb, ub, wc);
-            if (n1) compute(1, c + 1);
-            if (n2) stash(0, la, ua, wa);
-            __syncthreads();
-            n0 = n2; n1 = n3;
         }
     }
 
@@ -555,9 +595,13 @@ __global__ void __launch_bounds__(1024) sum_tables_kernel(const uint32_t* __rest
     }
 }
 
-// Main kernel of this orientation: the kernel above with the roles exchanged.  Lane l holds the weight rows l and
-// l + 64 of the tile ((w, w') of an input as one 8-byte word), wavefront v the batch rows 8 v .. 8 v + 7, whose
-// (l, u) of an input are one 8-byte broadcast; the results are written along the weight rows as they are.
+// Main kernel of this orientation, same tile with the roles exchanged: lane l holds the weight rows l and l + 64
+// of the tile, wavefront v the batch rows 8 v .. 8 v + 7.  The inputs go by in chunks of 32; the l, u and weight
+// tiles (128 x 32 each) of the next-but-one chunk are in flight while the current one is used from LDS, where an
+// input's (w, w') of a lane is one 8-byte word and the (l, u) of a batch row one 8-byte broadcast.  The table words
+// of 64 chunks at a time are copied to LDS ahead of the loop over them; a chunk nobody marks is not staged.  One
+// loop per batch row over that row's own marks (find-first-set, clear, branch); the results are written along the
+// weight rows as they are.
 __device__ __forceinline__ void bound_rows_body(const float* __restrict__ xl, const float* __restrict__ xu,
                                                 const float* __restrict__ w, const uint32_t* __restrict__ bits, int B,
                                                 int Bp, int M, int N, int nsplit, float* __restrict__ yL,
@@ -678,19 +722,21 @@ __device__ __forceinline__ void bound_rows_body(const float* __restrict__ xl, co
 // One launch for both orientations (same grid, same LDS): whichever table is below its limit is used
 __global__ void __launch_bounds__(1024, 1)
 bound_table_kernel(const float* __restrict__ xl, const float* __restrict__ xu, const float* __restrict__ w,
-                   const uint32_t* __restrict__ bits, const unsigned long long* __restrict__ count,
-                   unsigned long long limit_col, unsigned long long limit_row, int B, int Bp, int M, int Mp, int N,
-                   int nsplit, float* __restrict__ yL, float* __restrict__ yU) {
-    __shared__ __attribute__((aligned(16))) float smem[2 * kMainTileFloats];
-    __shared__ __attribute__((aligned(16))) uint32_t wb[kMainWords];
-    if (count[0] <= limit_col) bound_cols_body(xl, xu, w, bits, B, M, Mp, N, nsplit, yL, yU, smem, wb);
-    else if (count[1] <= limit_row) bound_rows_body(xl, xu, w, bits, B, Bp, M, N, nsplit, yL, yU, smem, wb);
+                   const float* __restrict__ xT, const uint32_t* __restrict__ bits,
+                   const unsigned long long* __restrict__ count, unsigned long long limit_col,
+                   unsigned long long limit_row, int B, int Bp, int M, int Mp, int N, int nsplit,
+                   float* __restrict__ yL, float* __restrict__ yU) {
+    __shared__ __attribute__((aligned(16))) float lds[kLdsWords];
+    if (count[0] <= limit_col) bound_cols_body(xT, w, bits, B, M, Mp, N, nsplit, yL, yU, lds);
+    else if (count[1] <= limit_row)
+        bound_rows_body(xl, xu, w, bits, B, Bp, M, N, nsplit, yL, yU, lds,
+                        reinterpret_cast<uint32_t*>(lds + 2 * kMainTileFloats));
 }
 
 }  // namespace
 
 size_t bound_cols_workspace(int B, int CO, int CI) {
-    size_t sz[6];
+    size_t sz[7];
     return carve_sizes(B, CO, CI, sz);
 }
 
@@ -727,13 +773,20 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
     *gate = c.count + 2;
     *gate_limit = 0ull;
     // a few workgroups per compute unit over the run: the work of a workgroup follows the marks of its rows
-    const long long wgs = (long long)T * S;
-    int nsplit = (int)((2ll * num_cus() + wgs - 1) / wgs);
-    if (nsplit > NCH / 8) nsplit = NCH / 8;
-    if (nsplit > 16) nsplit = 16;
-    if (nsplit < 1) nsplit = 1;
-    hipLaunchKernelGGL(bound_table_kernel, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.bits, c.count,
-                       limit_col, limit_row, B, Bp, CO, Mp, CI, nsplit, outL, outU);
+    hipLaunchKernelGGL(xt_kernel, dim3(CI / 16, S), dim3(256), 0, st, xl, xu, B, CI, c.count, limit_col, c.xt);
+    if ((rc = check_launch("xt_kernel"))) return rc;
+    // Slices of the input range.  A workgroup takes a whole compute unit and stays for its whole run, so the launch
+    // proceeds in rounds of num_cus() workgroups and 2.5 rounds cost three: the count with the least time by that
+    // model, each further slice priced at 4 % (its share of the merge), is taken.
+    const long long wgs = (long long)T * S, cus = num_cus();
+    int nsplit = 1;
+    double best = 0.0;
+    for (int n = 1; n <= 16 && (n == 1 || n <= NCH / 8); n++) {
+        const double cost = (double)((wgs * n + cus - 1) / cus) / n * (1.0 + 0.04 * n);
+        if (n == 1 || cost < best) { best = cost; nsplit = n; }
+    }
+    hipLaunchKernelGGL(bound_table_kernel, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.xt, c.bits,
+                       c.count, limit_col, limit_row, B, Bp, CO, Mp, CI, nsplit, outL, outU);
     return check_launch("bound_table_kernel");
 }
 
