@@ -19,12 +19,13 @@ constexpr int kColsChunk = 32;
 size_t bound_cols_workspace(int B, int CO, int CI);
 
 // Builds the table, counts its marks on the device and queues the table kernel so that it runs only when at most
-// `density` of all (tile, weight row, input) triples are marked; the caller queues the kernel that evaluates every
+// `density` of all (tile, weight row, input) triples are marked (`density_rows` of all (tile of weight rows, batch
+// row, input) triples where the table is built per batch row); the caller queues the kernel that evaluates every
 // term with the opposite condition on the same counter (*gate, *gate_limit).  outL / outU must be zero-filled:
 // the slices of the input range merge by atomic maximum.  (*gate)[1] (the word behind the gate) is 1 when the marks
 // per weight row are so few (below a sixteenth of the limit) that a kernel without LDS staging would serve better.
 int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float* outL,
-                       float* outU, void* ws, float density, const unsigned long long** gate,
+                       float* outU, void* ws, float density, float density_rows, const unsigned long long** gate,
                        unsigned long long* gate_limit, hipStream_t st);
 
 }  // namespace sd

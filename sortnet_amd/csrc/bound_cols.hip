@@ -741,7 +741,7 @@ size_t bound_cols_workspace(int B, int CO, int CI) {
 }
 
 int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float* outL,
-                       float* outU, void* ws, float density, const unsigned long long** gate,
+                       float* outU, void* ws, float density, float density_rows, const unsigned long long** gate,
                        unsigned long long* gate_limit, hipStream_t st) {
     if (CI % kChunk != 0 || B < 1 || CO < 1) { set_error("bound_cols_forward: shape not supported"); return SD_ERR_ARG; }
     const Carve c = carve(ws, B, CO, CI);
@@ -753,8 +753,9 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
     if ((rc = check_launch("col_range_kernel"))) return rc;
     const int slices = NCH < kLowSlices ? NCH : kLowSlices;
     const float d = density < 0.f ? 0.f : density > 1.f ? 1.f : density;
+    const float dr = density_rows < 0.f ? 0.f : density_rows > 1.f ? 1.f : density_rows;
     const unsigned long long limit_col = (unsigned long long)((double)S * CO * CI * d);
-    const unsigned long long limit_row = (unsigned long long)((double)T * B * CI * d);
+    const unsigned long long limit_row = (unsigned long long)((double)T * B * CI * dr);
     // ranges of W per tile of weight rows: only when the probe picks the tables per batch row
     hipLaunchKernelGGL(row_range_kernel, dim3((CI + 63) / 64, T), dim3(256), 0, st, w, CO, CI, S, c.wr, c.stat);
     if ((rc = check_launch("row_range_kernel"))) return rc;

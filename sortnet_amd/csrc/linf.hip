@@ -11,10 +11,11 @@ using namespace sd;
 // largest share of marked (tile, weight row, input) triples at which the candidate-table kernel of the interval
 // forward runs instead of the kernel that evaluates every term (sd_set_bound_candidate_density); negative: built-in
 static float g_bound_density = -1.f;
-// measured at B = 512, M = N = 5120: the table kernel takes 0.14 + 3.3 x share ms (140 us of staging, then about 75 SIMD
-// cycles per marked (tile, weight row, input)) and the table 0.08 ms, against 1.04 ms for every term
-// (the table is paid for by the time the choice is made: the limit sits where 0.14 + 3.3 x share meets 1.04)
-constexpr float kBoundColsCap = 0.26f;
+// measured at B = 512, M = N = 5120: the table kernel takes 0.09 + 2.6 x share ms (about 60 SIMD cycles per marked
+// (tile, weight row, input)) after 0.10 ms for the tables, against 1.03-1.09 ms for every term; the kernel of the
+// tables per batch row 0.14 + 3.3 x share ms.  The tables are paid for by the time the choice is made, so the limits
+// sit a little below where the table kernel alone meets the every-term kernel.
+constexpr float kBoundColsCap = 0.30f, kBoundRowsCap = 0.26f;
 constexpr int kHintSiteBound = 1, kHintSiteBoundSparse = 8;
 constexpr float kBoundSparseCap = 0.03f;   // marked share up to which the kernel without LDS staging runs
 static int g_bound_form = 0;              // 0: chosen per layer, 1: staged tiles, 2: transposed-row walk
@@ -332,7 +333,8 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
     if (cols) {
         void* ws = workspace(bound_cols_workspace(B, CO, CI), st);
         if (!ws) return SD_ERR_HIP;
-        if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, outputL, outputU, ws, cap, &a.gate, &a.gate_limit, st)))
+        if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, outputL, outputU, ws, cap,
+                                     g_bound_density >= 0.f ? g_bound_density : kBoundRowsCap, &a.gate, &a.gate_limit, st)))
             return rc;
         a.gate_above = 1;
         rc = TB == 2 ? launch_fwd<BoundNogradGated, 2, 8>(a, st) : launch_fwd<BoundNogradGated, 4, 8>(a, st);
