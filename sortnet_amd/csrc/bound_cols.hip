@@ -24,13 +24,14 @@ struct Carve {
     unsigned long long* count;   // [0] marks of the per-weight-row table, [1] of the per-batch-row table, [2] every-term kernel's turn
     uint32_t* bits;   // [S][NCH][Mp] (or [T][NCH][Bp]): bit i of a word = input 32 c + i may hold a maximum of that row in that tile
     uint32_t* partial;   // marks per wavefront of the table kernel
+    uint32_t* order;  // [S][Mp] per batch tile and block of 128 weight rows: the row (0..127) at each place of the block
     float* xt;        // [S][N][64][4] per batch tile and input: (l, l', u, u') of the tile's rows i and i + 64, repaired
 };
 
 inline int bpad_of(int B) { return (B + kTileB - 1) / kTileB * kTileB; }
 inline size_t maxz(size_t a, size_t b) { return a > b ? a : b; }
 
-size_t carve_sizes(int B, int M, int N, size_t (&sz)[7]) {
+size_t carve_sizes(int B, int M, int N, size_t (&sz)[8]) {
     const size_t S = tiles_b(B), Mp = mpad_of(M), Bp = bpad_of(B), T = Mp / kTileW, NCH = N / kChunk;
     sz[0] = align256(S * 4 * N * 4);                               // xr
     sz[1] = align256(T * 2 * N * 4);                               // wr
@@ -39,11 +40,12 @@ size_t carve_sizes(int B, int M, int N, size_t (&sz)[7]) {
     sz[4] = align256(maxz(S * NCH * Mp, T * NCH * Bp) * 4);        // bits
     sz[5] = align256(maxz(Mp / 64, Bp / 64 * ((T + 3) / 4)) * kLowSlices * 4 * 4);   // partial
     sz[6] = align256(S * N * 1024);                                // xt
-    return sz[0] + sz[1] + sz[2] + sz[3] + sz[4] + sz[5] + sz[6];
+    sz[7] = align256(S * Mp * 4);                                  // order
+    return sz[0] + sz[1] + sz[2] + sz[3] + sz[4] + sz[5] + sz[6] + sz[7];
 }
 
 Carve carve(void* ws, int B, int M, int N) {
-    size_t sz[7];
+    size_t sz[8];
     carve_sizes(B, M, N, sz);
     const size_t S = tiles_b(B), Mp = mpad_of(M), Bp = bpad_of(B), T = Mp / kTileW;
     char* p = static_cast<char*>(ws);
@@ -56,7 +58,8 @@ Carve carve(void* ws, int B, int M, int N) {
     c.count = reinterpret_cast<unsigned long long*>(p); p += sz[3];
     c.bits = reinterpret_cast<uint32_t*>(p); p += sz[4];
     c.partial = reinterpret_cast<uint32_t*>(p); p += sz[5];
-    c.xt = reinterpret_cast<float*>(p);
+    c.xt = reinterpret_cast<float*>(p); p += sz[6];
+    c.order = reinterpret_cast<uint32_t*>(p);
     return c;
 }
 
@@ -149,14 +152,22 @@ __device__ __forceinline__ bool rows_decide(const float* stat, int S) {
 //         atomic maximum of the bit patterns (all values >= 1e-10 > 0 on zero-filled memory);
 //   else: one table word per (tile, chunk, weight row): bit n set when the largest the term can be reaches the
 //         lower bound of the upper or of the lower result; the marks are counted.
+// Within a block of 128 weight rows the words are not stored in the order of the rows.  The main kernel gives each
+// of its 16 wavefronts eight places of a block and a workgroup ends with its slowest wavefront, while the marks of a
+// row vary several-fold around their mean (with consecutive rows the fullest wavefront carries 1.2-1.35 times the
+// mean).  A row's lower bounds tell how many marks it will get (the smaller of the two ranks the rows of a block
+// nearly as their mark counts do), so the rows are ranked by it, smallest (most marks) first, and dealt back and
+// forth: ranks 0..15 to wavefronts 0..15, ranks 16..31 to wavefronts 15..0, and so on.  order[] names the row at
+// each place.
 template <bool LOW>
 __device__ __forceinline__ void col_table_body(const float* __restrict__ w, const float* __restrict__ xr,
                                                int M, int N, int S, int Mp, float* __restrict__ low,
                                                uint32_t* __restrict__ bits, uint32_t* __restrict__ partial,
-                                               int bx, int by, int gx, int gy) {
+                                               uint32_t* __restrict__ order, int bx, int by, int gx, int gy) {
     // row stride 36 words: 16-byte rows, and the 128-bit reads of 16 consecutive lanes fall on disjoint banks
     __shared__ __attribute__((aligned(16))) float wt[64][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float xs[4][4][kChunk];   // column ranges of the four batch tiles of this pass, current chunk
+    __shared__ float keys[LOW ? 1 : 4][LOW ? 1 : kTileW];            // per batch tile of this pass: what the rows of the block are ranked by
     const int tid = threadIdx.x, r = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int m0 = bx * 64, NCH = N / kChunk;
@@ -172,9 +183,27 @@ __device__ __forceinline__ void col_table_body(const float* __restrict__ w, cons
         const int s = sb + wave;
         const bool active = s < S;
         float LU = kEps, LL = kEps;
+        int wordrow = m0 + r;   // where this row's words go: its place within its block of 128
         if (!LOW && active) {
             LU = fmaxf(kEps, low[(size_t)(s * 2) * Mp + m0 + r]);
             LL = fmaxf(kEps, low[(size_t)(s * 2 + 1) * Mp + m0 + r]);
+            const int mb = m0 & ~(kTileW - 1), mine = m0 - mb + r;
+            #pragma unroll
+            for (int j = r; j < kTileW; j += 64) {
+                const float a = fmaxf(kEps, low[(size_t)(s * 2) * Mp + mb + j]);
+                const float b = fmaxf(kEps, low[(size_t)(s * 2 + 1) * Mp + mb + j]);
+                keys[wave][j] = mb + j < M ? fminf(a, b) : __builtin_inff();   // rows past the last one have no marks
+            }
+            __builtin_amdgcn_wave_barrier();   // LDS operations of one wavefront complete in order
+            const float key = keys[wave][mine];
+            int rank = 0;
+            for (int j = 0; j < kTileW; j++) {
+                const float other = keys[wave][j];
+                rank += (other < key || (other == key && j < mine)) ? 1 : 0;
+            }
+            const int k = rank >> 4, j = rank & 15;
+            wordrow = mb + ((k & 1) ? 15 - j : j) * 8 + k;
+            if (by == 0) order[(size_t)s * Mp + wordrow] = (uint32_t)mine;
         }
         // the weights and ranges of the next chunk are fetched while the current one is used
         float4 pa, pb;
@@ -221,7 +250,7 @@ __device__ __forceinline__ void col_table_body(const float* __restrict__ w, cons
                 }
                 if (!LOW) {
                     if (!valid) word = 0u;
-                    bits[((size_t)s * NCH + c) * Mp + m0 + r] = word;
+                    bits[((size_t)s * NCH + c) * Mp + wordrow] = word;
                     marks += __builtin_popcount(word);
                 }
             }
@@ -286,8 +315,9 @@ __global__ void __launch_bounds__(256) xt_kernel(const float* __restrict__ xl, c
 }
 
 __device__ __forceinline__ void bound_cols_body(const float* __restrict__ xT, const float* __restrict__ w,
-                                                const uint32_t* __restrict__ bits, int B, int M, int Mp, int N,
-                                                int nsplit, float* __restrict__ yL, float* __restrict__ yU, float* smem) {
+                                                const uint32_t* __restrict__ bits, const uint32_t* __restrict__ order,
+                                                int B, int M, int Mp, int N, int nsplit, float* __restrict__ yL,
+                                                float* __restrict__ yU, float* smem) {
     constexpr int TW = 8;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -302,14 +332,18 @@ __device__ __forceinline__ void bound_cols_body(const float* __restrict__ xT, co
     #pragma unroll
     for (int r = 0; r < TW; r++) { lo[r][0] = lo[r][1] = -kEps; hi[r][0] = hi[r][1] = kEps; }
 
+    // the rows at this wavefront's eight places of the block (wave-uniform)
+    int row[TW];
+    #pragma unroll
+    for (int r = 0; r < TW; r++) row[r] = (int)order[(size_t)s * Mp + m0 + wave * TW + r];
+
     if (st_lo < st_hi) {
         const float* __restrict__ xsrc = xT + (size_t)s * N * 256;
         const size_t xlast = (size_t)N * 256 - 4;                       // the tile's last 16-byte word
-        const int mrow = m0 + wave * TW;
-        const uint32_t* __restrict__ bw = bits + (size_t)s * NCH * Mp + mrow;   // words of chunk c: bw[c * Mp + r]
+        const uint32_t* __restrict__ bw = bits + (size_t)s * NCH * Mp + m0 + wave * TW;   // words of chunk c: bw[c * Mp + r]
         size_t wrow[TW];
         #pragma unroll
-        for (int r = 0; r < TW; r++) wrow[r] = (size_t)(mrow + r < M ? mrow + r : M - 1) * N;
+        for (int r = 0; r < TW; r++) wrow[r] = (size_t)(m0 + row[r] < M ? m0 + row[r] : M - 1) * N;
 
         auto load_x = [&](int st, float4 (&v)[4]) __attribute__((always_inline)) {
             #pragma unroll
@@ -403,7 +437,7 @@ __device__ __forceinline__ void bound_cols_body(const float* __restrict__ xT, co
         for (int r = 0; r < TW; r++) {
             #pragma unroll
             for (int j = 0; j < 2; j++)
-                tr[(lane + 64 * j) * (kTileW + 1) + wave * TW + r] = which == 0 ? -lo[r][j] : hi[r][j];
+                tr[(lane + 64 * j) * (kTileW + 1) + row[r]] = which == 0 ? -lo[r][j] : hi[r][j];
         }
         __syncthreads();
         float* y = which == 0 ? yL : yU;
@@ -554,7 +588,7 @@ __global__ void __launch_bounds__(256) table_kernel(const float* __restrict__ xl
                                                     const float* __restrict__ wr, int B, int M, int N, int S, int T,
                                                     int Mp, int Bp, int slices, float* __restrict__ low,
                                                     uint32_t* __restrict__ bits, uint32_t* __restrict__ partial,
-                                                    const float* __restrict__ stat) {
+                                                    uint32_t* __restrict__ order, const float* __restrict__ stat) {
     const int id = blockIdx.x;
     if (rows_decide(stat, S)) {
         const int gx = Bp / 64, gy = slices, gz = (T + 3) / 4;
@@ -563,7 +597,7 @@ __global__ void __launch_bounds__(256) table_kernel(const float* __restrict__ xl
     } else {
         const int gx = Mp / 64, gy = slices;
         if (id >= gx * gy) return;
-        col_table_body<LOW>(w, xr, M, N, S, Mp, low, bits, partial, id % gx, id / gx, gx, gy);
+        col_table_body<LOW>(w, xr, M, N, S, Mp, low, bits, partial, order, id % gx, id / gx, gx, gy);
     }
 }
 
@@ -722,12 +756,12 @@ __device__ __forceinline__ void bound_rows_body(const float* __restrict__ xl, co
 // One launch for both orientations (same grid, same LDS): whichever table is below its limit is used
 __global__ void __launch_bounds__(1024, 1)
 bound_table_kernel(const float* __restrict__ xl, const float* __restrict__ xu, const float* __restrict__ w,
-                   const float* __restrict__ xT, const uint32_t* __restrict__ bits,
+                   const float* __restrict__ xT, const uint32_t* __restrict__ bits, const uint32_t* __restrict__ order,
                    const unsigned long long* __restrict__ count, unsigned long long limit_col,
                    unsigned long long limit_row, int B, int Bp, int M, int Mp, int N, int nsplit,
                    float* __restrict__ yL, float* __restrict__ yU) {
     __shared__ __attribute__((aligned(16))) float lds[kLdsWords];
-    if (count[0] <= limit_col) bound_cols_body(xT, w, bits, B, M, Mp, N, nsplit, yL, yU, lds);
+    if (count[0] <= limit_col) bound_cols_body(xT, w, bits, order, B, M, Mp, N, nsplit, yL, yU, lds);
     else if (count[1] <= limit_row)
         bound_rows_body(xl, xu, w, bits, B, Bp, M, N, nsplit, yL, yU, lds,
                         reinterpret_cast<uint32_t*>(lds + 2 * kMainTileFloats));
@@ -736,7 +770,7 @@ bound_table_kernel(const float* __restrict__ xl, const float* __restrict__ xu, c
 }  // namespace
 
 size_t bound_cols_workspace(int B, int CO, int CI) {
-    size_t sz[7];
+    size_t sz[8];
     return carve_sizes(B, CO, CI, sz);
 }
 
@@ -762,10 +796,10 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
     const int wg_col = (Mp / 64) * slices, wg_row = (Bp / 64) * slices * ((T + 3) / 4);
     const int wg_tab = wg_col > wg_row ? wg_col : wg_row;
     hipLaunchKernelGGL(table_kernel<true>, dim3(wg_tab), dim3(256), 0, st, xl, xu, w, c.xr, c.wr, B, CO, CI, S, T, Mp, Bp,
-                       slices, c.low, c.bits, c.partial, c.stat);
+                       slices, c.low, c.bits, c.partial, c.order, c.stat);
     if ((rc = check_launch("table_kernel<low>"))) return rc;
     hipLaunchKernelGGL(table_kernel<false>, dim3(wg_tab), dim3(256), 0, st, xl, xu, w, c.xr, c.wr, B, CO, CI, S, T, Mp, Bp,
-                       slices, c.low, c.bits, c.partial, c.stat);
+                       slices, c.low, c.bits, c.partial, c.order, c.stat);
     if ((rc = check_launch("table_kernel<bits>"))) return rc;
     hipLaunchKernelGGL(sum_tables_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)wg_col * 4, (size_t)wg_row * 4,
                        c.count, c.stat, S, limit_col, limit_row);
@@ -787,7 +821,7 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
         if (n == 1 || cost < best) { best = cost; nsplit = n; }
     }
     hipLaunchKernelGGL(bound_table_kernel, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.xt, c.bits,
-                       c.count, limit_col, limit_row, B, Bp, CO, Mp, CI, nsplit, outL, outU);
+                       c.order, c.count, limit_col, limit_row, B, Bp, CO, Mp, CI, nsplit, outL, outU);
     return check_launch("bound_table_kernel");
 }
 
