@@ -1179,7 +1179,9 @@ __device__ __forceinline__ uint32_t chunk_keep_bits(const FwdArgs& a, long long 
     return 0xffffffffu;
 }
 
-template <bool PACKED>
+// LISTS: the layer has kept-input index lists.  Without them an input's column is its number, and no load stands
+// between the two operand loads of one output and those of the next, so that a wavefront has them all in flight.
+template <bool PACKED, bool LISTS>
 __global__ void __launch_bounds__(256) resolve_pos_kernel(FwdArgs a) {
     if (gate_closed(a.gate, a.gate_limit, a.gate_above)) return;   // one of two queued for the result
     __shared__ __attribute__((aligned(16))) ResolveSlot slots[4][64];
@@ -1229,7 +1231,7 @@ __global__ void __launch_bounds__(256) resolve_pos_kernel(FwdArgs a) {
             int n = (q.cid < 0 ? 0 : q.cid) * KT + l;
             cand[u] = n < a.CIg && ((q.keep >> l) & 1u) != 0u;
             if (n >= a.CIg) n = 0;
-            const int col = a.ci_idx ? a.ci_idx[q.coff + n] : n;
+            const int col = LISTS ? a.ci_idx[q.coff + n] : n;
             d[u] = a.x0[(size_t)q.xoff + (size_t)n * a.HW] - a.w[q.woff + col];
             best[u] = q.best;
         }
@@ -1328,8 +1330,13 @@ inline int launch_resolve_bound(const FwdArgs& a, hipStream_t stream) {
 inline int launch_resolve(const FwdArgs& a, hipStream_t stream) {
     long long total = (long long)a.R * a.G * a.COg;
     dim3 grid((unsigned)((total + 255) / 256));
-    if (a.nsplit > 1) hipLaunchKernelGGL((resolve_pos_kernel<true>), grid, dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL((resolve_pos_kernel<false>), grid, dim3(256), 0, stream, a);
+    if (a.ci_idx) {
+        if (a.nsplit > 1) hipLaunchKernelGGL((resolve_pos_kernel<true, true>), grid, dim3(256), 0, stream, a);
+        else hipLaunchKernelGGL((resolve_pos_kernel<false, true>), grid, dim3(256), 0, stream, a);
+    } else {
+        if (a.nsplit > 1) hipLaunchKernelGGL((resolve_pos_kernel<true, false>), grid, dim3(256), 0, stream, a);
+        else hipLaunchKernelGGL((resolve_pos_kernel<false, false>), grid, dim3(256), 0, stream, a);
+    }
     return check_launch("resolve_pos_kernel");
 }
 
