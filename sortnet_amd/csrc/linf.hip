@@ -16,6 +16,10 @@ static float g_bound_density = -1.f;
 // tables per batch row 0.14 + 3.3 x share ms.  The tables are paid for by the time the choice is made, so the limits
 // sit a little below where the table kernel alone meets the every-term kernel.
 constexpr float kBoundColsCap = 0.30f, kBoundRowsCap = 0.26f;
+// With the built-in limits, layers below this many terms go without tables: building them and starting the table
+// kernel takes about 0.19 ms, which is what the every-term kernel needs for 2.4 G terms (512 x 10 x 5120: 0.06 ms
+// for every term against 0.10 ms from tables).
+constexpr long long kBoundColsMinTerms = 1ll << 31;
 constexpr int kHintSiteBound = 1, kHintSiteBoundSparse = 8;
 constexpr float kBoundSparseCap = 0.03f;   // marked share up to which the kernel without LDS staging runs
 static int g_bound_form = 0;              // 0: chosen per layer, 1: staged tiles, 2: transposed-row walk
@@ -302,7 +306,8 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
     // dense single-group layers: a kernel that works from per-weight-row candidate tables is queued in front of the
     // one that evaluates every term, and a count taken on the device decides which of the two runs
     const float cap = g_bound_density >= 0.f ? g_bound_density : kBoundColsCap;
-    bool cols = cap > 0.f && G == 1 && HW == 1 && CI % kColsChunk == 0 && a.fast_x && a.fast_w;
+    bool cols = cap > 0.f && G == 1 && HW == 1 && CI % kColsChunk == 0 && a.fast_x && a.fast_w &&
+                (g_bound_density >= 0.f || (long long)B * CO * CI >= kBoundColsMinTerms);
     // with the built-in limit, a layer whose tables have not paid lately is not given any for a while
     const bool hinted = cols && g_bound_density < 0.f;
     if (hinted && !hint_build_tables(kHintSiteBound, weight, B, CO, CI, st)) cols = false;

@@ -131,23 +131,33 @@ def test_bound_candidate_kernel_at_layer_size(density):
 
 
 def test_bound_results_do_not_depend_on_the_table_hint(oracle, density):
-    """With the built-in limit a layer (same weights, same shape) whose tables did not pay a few times in a row is
-    given none for a while: calls before, during and after that stretch give the oracle's bits, on data of either kind."""
+    """With the built-in limits (layers of at least 2^31 terms) a layer (same weights, same shape) whose tables did not
+    pay a few times in a row is given none for a while: calls before, during and after that stretch give the bits of
+    the every-term kernel on all rows and of the oracle on the first rows, on data of either kind."""
     from sortnet_amd import ext
     dev = _dev()
-    density(-1.0)
-    B, CI, CO = 140, 512, 200
+    B, CI, CO = 512, 2048, 2048
     g = torch.Generator().manual_seed(11)
     w = (torch.randn(CO, CI, generator=g) * 0.3).contiguous().to(dev)
+    calls = []
+    density(-1.0)
     for call in range(12):
         kind = "random" if call < 8 else "rows_alike"     # unrelated rows: every term; rows alike: the table
         xl, xu = _intervals(B, CI, kind, 100 + call)
-        rl, ru = oracle.bound_inf_dist_forward(xl.numpy(), xu.numpy(), w.cpu().numpy(), 1, need_pos=False)
+        xl, xu = xl.to(dev), xu.to(dev)
         yl = torch.full((B, CO, 1), float("nan"), device=dev)
         yu = torch.full((B, CO, 1), float("nan"), device=dev)
-        ext.bound_inf_dist_forward_nograd(xl.to(dev), xu.to(dev), w, yl, yu, 1)
+        ext.bound_inf_dist_forward_nograd(xl, xu, w, yl, yu, 1)
         torch.cuda.synchronize()   # lets the next call see which kernel ran
-        assert np.array_equal(yl.cpu().numpy(), rl) and np.array_equal(yu.cpu().numpy(), ru), call
+        calls.append((xl, xu, yl, yu))
+    density(0.0)
+    for call, (xl, xu, yl, yu) in enumerate(calls):
+        el, eu = torch.empty_like(yl), torch.empty_like(yu)
+        ext.bound_inf_dist_forward_nograd(xl, xu, w, el, eu, 1)
+        assert torch.equal(yl, el) and torch.equal(yu, eu), call
+        rl, ru = oracle.bound_inf_dist_forward(xl[:8].cpu().numpy(), xu[:8].cpu().numpy(), w.cpu().numpy(), 1,
+                                               need_pos=False)
+        assert np.array_equal(yl[:8].cpu().numpy(), rl) and np.array_equal(yu[:8].cpu().numpy(), ru), call
 
 
 def test_bound_candidate_density_argument(density):
@@ -159,7 +169,7 @@ def test_bound_candidate_density_argument(density):
 
 def test_bound_candidate_kernel_long_slices(density):
     """Enough output tiles that the input range is not cut (B = 2048, CO = 4096) and more than 64 chunks of inputs
-    (CI = 2112): the table kernel stages its mark words in two segments.  Same bits as the every-term kernel."""
+    (CI = 2112: 33 stages of 64 inputs in one slice).  Same bits as the every-term kernel."""
     from sortnet_amd import ext
     dev = _dev()
     B, CI, CO = 2048, 2112, 4096
