@@ -155,13 +155,19 @@ __global__ void __launch_bounds__(256) bound_bwd_rows_kernel(BwdArgs a) {
 // grad_weight needs neither a zero-fill pass nor global atomics.  Work-item = (row j = tid % WR, batch rows
 // tid / WR + i * 256 / WR): the WR positions of one batch row are adjacent in memory when HW == 1.
 // MODE 0: l-inf, 1: sort neuron (K slots, geometric coefficients), 2: interval bounds (two positions).
+// A workgroup reads WR adjacent entries of every row of pos and grad_output, so one 64-byte piece of those rows is
+// shared by 16 / WR workgroups.  Workgroups go to the chip's eight dies in turn, each
+// with a cache of its own: eight consecutive row blocks are given to one die, next to each other in launch order, so
+// that a piece is fetched from memory by one die, once, instead of by all eight.
 constexpr int kMaxWRowsLds = 15360;   // floats of LDS the weight-row histograms of one workgroup may take
 
 template <int MODE>
 __global__ void __launch_bounds__(256) wrows_bwd_kernel(BwdArgs a, int WR) {
     extern __shared__ float hist[];             // [WR][CIg]
     const int CO = a.G * a.COg;
-    const int c0 = blockIdx.x * WR;
+    const int die = blockIdx.x & 7, k = blockIdx.x >> 3;
+    const int c0 = ((((k >> 3) * 8 + die) << 3) + (k & 7)) * WR;
+    if (c0 >= CO) return;                       // the grid is rounded up to 64 row blocks
     const int nrows = CO - c0 < WR ? CO - c0 : WR;
     for (int n = threadIdx.x; n < WR * a.CIg; n += 256) hist[n] = 0.f;
     __syncthreads();
@@ -204,7 +210,8 @@ static bool launch_wrows(const BwdArgs& a, hipStream_t st) {
     int WR = 1;
     while (WR < 8 && 2 * WR * a.CIg <= kMaxWRowsLds) WR *= 2;
     const int CO = a.G * a.COg;
-    hipLaunchKernelGGL((wrows_bwd_kernel<MODE>), dim3((unsigned)((CO + WR - 1) / WR)), dim3(256),
+    const int blocks = (CO + WR - 1) / WR;
+    hipLaunchKernelGGL((wrows_bwd_kernel<MODE>), dim3((unsigned)((blocks + 63) / 64 * 64)), dim3(256),
                        (size_t)WR * a.CIg * sizeof(float), st, a, WR);
     return true;
 }
