@@ -35,7 +35,8 @@ def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=8,
+                    help="untimed steps; a layer's table hints settle within its first seven calls")
     ap.add_argument("--batch", type=int, default=512)
     ap.add_argument("--width", type=int, default=5120)
     ap.add_argument("--depth", type=int, default=6, help="distance layers incl. the class layer (reference: depth=6)")
@@ -407,7 +408,7 @@ def main():
 
     if not args.no_secondary:
         sec = {}
-        short, warm = max(3, args.steps // 4), 2
+        short, warm = max(3, args.steps // 4), 8   # a layer's table hints settle within its first seven calls
 
         def masked_entry(mask, q, steps=short, warmup=warm, **kw):
             r = run_masked(args, mask, q, steps, warmup, **kw)
@@ -419,7 +420,7 @@ def main():
         sec["q1"] = dict(masked_entry(args.mask, 1.0), workload=workload_text(args, args.mask, 1.0))
         # the same step from the reference's own initialisation (weights of unit scale, core/models/norm_dist.py:30)
         # (enough steps for the layers to have settled on their kernels: a layer reports three calls before it switches)
-        sec["unit_weights"] = dict(masked_entry(args.mask, args.q, steps=max(short, 12), warmup=4, weight_std=1.0),
+        sec["unit_weights"] = dict(masked_entry(args.mask, args.q, steps=max(short, 12), warmup=8, weight_std=1.0),
                                    workload=workload_text(args, args.mask, args.q).replace("N(0, 1/fan_in)", "N(0, 1)")
                                    + " as the reference initialises them")
         # the reference's own training form at the keep probability of its published commands (0.7-0.85)
