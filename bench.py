@@ -26,8 +26,9 @@ if ROOT not in sys.path:
 
 FP32_VECTOR_PEAK_TFLOPS = 157.3     # MI355X published fp32 vector peak
 VALU_LANE_RATE = 78.64e12           # 256 CUs x 4 SIMD x 16 lanes x 2 issue ports x 2.4 GHz lane-instructions/s
-# HBM bytes of one 512x5120x5120 interval-bound launch come from the committed counter summary (two rocprofv3
-# --pmc runs, FETCH_SIZE and WRITE_SIZE, scaled by a plain copy of known size): the line "traffic_bytes_per_launch"
+# HBM bytes of one 512x5120x5120 launch come from the committed counter summary (two rocprofv3 --pmc runs,
+# FETCH_SIZE and WRITE_SIZE, scaled by a plain copy of known size): the lines "traffic_bytes_per_launch" (interval
+# forward, every term) and "traffic_bytes_per_launch_masked_forward" (l-inf forward under the factored mask)
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_headline_hbm_traffic.txt")
 
 
@@ -199,12 +200,13 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     ibp_events = []
     ibp_kernel = [None]          # the tile kernel the library dispatched for the width x width interval layers
     probe = []                   # operands of the last width x width interval layer of the last step
-    dense_events = []
+    dense_ms = []                # every-term interval kernel, per launch
+    fwd_ms, fwd_kernel = [], [None]   # masked l-inf forward tile kernel, per launch
 
-    def step(i, timed):
+    def step(i, timed, after_layer=None):
         marks = [ev() for _ in range(5)]
         marks[0].record()
-        dist = model.forward(x, step_seed=i)
+        dist = model.forward(x, step_seed=i, after_layer=after_layer)
         logits, worst = margins(dist, targets, eps)
         loss = hinge_loss(worst)
         marks[1].record()
@@ -258,18 +260,37 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
         ylo = torch.empty(lo.size(0), w.size(0), 1, device=dev)
         yup = torch.empty_like(ylo)
         _lib.set_bound_candidate_density(0.0)
+        _lib.time_forward_kernels(True)      # events around the tile kernel's own launch, on the stream it is queued on
         try:
             with torch.no_grad():
                 for k in range(2 + max(8, steps)):
-                    e0, e1 = ev(), ev()
-                    e0.record()
                     ext.bound_inf_dist_forward_nograd(lo, up, w, ylo, yup, 1)
-                    e1.record()
-                    if k >= 2:
-                        dense_events.append((e0, e1))
+                    ms = _lib.last_forward_kernel_ms()
+                    if k >= 2 and ms is not None:
+                        dense_ms.append(ms)
             ibp_kernel[0] = _lib.last_forward_kernel()
         finally:
             _lib.set_bound_candidate_density(-1.0)
+            _lib.time_forward_kernels(False)
+        torch.cuda.synchronize()
+
+    if time_ibp and q < 1.0:
+        # The kernel with the largest share of the step: the masked l-inf forward with chunk tracking of a
+        # width x width layer.  A few more steps, with the library's events around the tile kernel's launch switched
+        # on and read back after every such layer (which makes the host wait: these steps are not part of `value`).
+        def read_timer(i, w):
+            if i > 0 and tuple(w.shape) == (width, width):
+                ms = _lib.last_forward_kernel_ms()
+                if ms is not None:
+                    fwd_ms.append(ms)
+                    fwd_kernel[0] = _lib.last_forward_kernel()
+
+        _lib.time_forward_kernels(True)
+        try:
+            for k in range(max(4, steps // 4)):
+                step(warmup + steps + k, False, after_layer=read_timer)
+        finally:
+            _lib.time_forward_kernels(False)
         torch.cuda.synchronize()
 
     if calib_copy:
@@ -285,7 +306,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
         "ms_per_step": elapsed * 1e3 / steps, "samples_per_s": batch / (elapsed / steps), "steps": steps,
         "phase_ms": phase_ms, "terms_per_step": model.terms_per_sample() * batch,
         "ibp_launch_ms": [a.elapsed_time(b) for a, b in ibp_events], "ibp_kernel": ibp_kernel[0],
-        "ibp_every_term_ms": [a.elapsed_time(b) for a, b in dense_events],
+        "ibp_every_term_ms": dense_ms, "fwd_kernel_ms": fwd_ms, "fwd_kernel": fwd_kernel[0],
         "loss": float(loss.detach()), "certified_frac": float((cert.max(dim=1)[0] < 0).float().mean()),
     }
     del model, opt
@@ -293,10 +314,10 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     return res
 
 
-def committed_traffic():
-    """traffic_bytes_per_launch of the committed counter summary, or None."""
+def committed_traffic(key):
+    """The figure `key` of the committed counter summary, or None."""
     try:
-        m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(TRAFFIC_PROFILE).read(), re.M)
+        m = re.search(r"^%s:\s*([0-9.eE+]+)" % key, open(TRAFFIC_PROFILE).read(), re.M)
         return float(m.group(1)) if m else None
     except OSError:
         return None
@@ -367,18 +388,19 @@ def main():
     step_s = head["ms_per_step"] * 1e-3
     step_flops = head["terms_per_step"] * (2 + 6)         # forward 2 flops/term, interval bounds 6 flops/term
     layer_terms = args.batch * args.width * args.width
-    launches, dense = head["ibp_launch_ms"], head["ibp_every_term_ms"]
+    launches, dense, fwd = head["ibp_launch_ms"], head["ibp_every_term_ms"], head["fwd_kernel_ms"]
     step_ms = sum(launches) / max(len(launches), 1)
     ibp_ms = sum(dense) / max(len(dense), 1)
-    achieved = 6.0 * layer_terms / (ibp_ms * 1e-3) / 1e12 if dense else None
-    roofline = {
-        "bound": "valu",
+    fwd_ms = sum(fwd) / max(len(fwd), 1)
+    at_size = (args.batch, args.width) == (512, 5120)
+    factored = args.mask == "factored"
+    interval = {
         "kernel": "sd::%s, policy BoundNograd (interval-bound forward, every term, %dx%dx%d)" % (head["ibp_kernel"], args.batch, args.width, args.width),
-        "achieved": achieved, "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
-        "frac": achieved / FP32_VECTOR_PEAK_TFLOPS if achieved else None,
-        "traffic": committed_traffic() if (args.batch, args.width) == (512, 5120) else None,
+        "achieved": 6.0 * layer_terms / (ibp_ms * 1e-3) / 1e12 if dense else None, "unit": "TFLOP/s",
+        "frac": 6.0 * layer_terms / (ibp_ms * 1e-3) / 1e12 / FP32_VECTOR_PEAK_TFLOPS if dense else None,
+        "traffic": committed_traffic("traffic_bytes_per_launch") if at_size else None,
         "algorithmic_bytes": 4.0 * (args.width * args.width + 4 * args.batch * args.width),
-        "avg_launch_ms": ibp_ms, "launches_timed": len(dense),
+        "avg_launch_ms": ibp_ms if dense else None, "launches_timed": len(dense),
         "valu_issue_frac": 4.0 * layer_terms / (ibp_ms * 1e-3) / VALU_LANE_RATE if dense else None,
         "in_step": {
             "avg_call_ms": step_ms if launches else None, "calls_timed": len(launches),
@@ -388,11 +410,37 @@ def main():
                     "count taken on the device picks the table kernel or the every-term kernel; terms that cannot "
                     "hold a maximum are never formed, so this rate is not bounded by the vector peak",
         },
-        "note": "tropical (sub/min/max) contraction on the fp32 vector ALUs, not MFMA; 6 flops per term in 4 VALU "
-                "instructions; a register-only stream of this mix reaches 72 T lane-instructions/s on this part "
-                "(floor 56 fs/term = 69% of peak) and the part sustains ~2.0 of its 2.4 GHz under this kernel; timed "
-                "after the steps on the operands of their last width x width layer with the candidate table switched off",
+        "note": "6 flops per term in 4 VALU instructions; a register-only stream of this mix reaches 72 T "
+                "lane-instructions/s on this part (floor 56 fs/term = 69% of peak) and the part sustains ~2.0 of its "
+                "2.4 GHz under this kernel; the step itself takes this entry point's results from candidate tables "
+                "(in_step), so these launches are queued after the steps, on the operands of their last width x width "
+                "layer with the table switched off",
     }
+    if fwd:
+        achieved = 2.0 * layer_terms / (fwd_ms * 1e-3) / 1e12
+        roofline = {
+            "bound": "valu",
+            "kernel": "sd::%s, policy %s (l-inf forward under the %s mask with the winning chunk tracked for the "
+                      "positions, every term, %dx%dx%d)" % (head["fwd_kernel"], "LinfChunkPacked" if factored else "MaskedTermChunk",
+                                                            args.mask, args.batch, args.width, args.width),
+            "achieved": achieved, "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": achieved / FP32_VECTOR_PEAK_TFLOPS,
+            "traffic": committed_traffic("traffic_bytes_per_launch_masked_forward") if at_size and factored else None,
+            "algorithmic_bytes": 4.0 * (args.width * args.width + 3 * args.batch * args.width),
+            "avg_launch_ms": fwd_ms, "launches_timed": len(fwd),
+            "valu_issue_frac": 1.5 * layer_terms / (fwd_ms * 1e-3) / VALU_LANE_RATE if factored else None,
+            "note": ("the kernel with the largest share of the step (four launches, about 30 %); tropical (sub/max) "
+                     "contraction on the fp32 vector ALUs, not MFMA: 2 flops per term in 1.5 VALU instructions (one "
+                     "subtraction, half a three-operand maximum), so a register-only stream at the part's 72 T "
+                     "lane-instructions/s would give 61 % of the peak; " if factored else
+                     "the kernel with the largest share of the step; 2 flops per term, and the keep decision of every "
+                     "term comes from a counter hash that costs more than the term; ") +
+                    "timed by events around the kernel's own launch (sd_time_forward_kernels) in a few further steps "
+                    "after the timed ones, every width x width layer",
+            "interval_every_term": interval,
+        }
+    else:   # q = 1: no masked layers; the interval kernel is the one to report
+        roofline = dict(interval, bound="valu", peak=FP32_VECTOR_PEAK_TFLOPS)
     out = {
         "metric": "train samples/s (fwd+bwd+IBP) 5x5120 SortNet-MLP, B=512; % FP32 VALU peak",
         "value": head["samples_per_s"], "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -59,6 +59,13 @@ const char* sd_last_error(void);
  * "fwd_kernel_direct<4,8>" (global -> LDS loads), "fwd_kernel_pipe<4,8>" (register-staged), "fwd_kernel_lists<2,8>"
  * (gather loads), "fwd_kernel<2,4>" (general): for tests and benchmarks that must know which path they measured. */
 const char* sd_last_forward_kernel(void);
+/* For benchmarks that must report a tile kernel's own duration rather than an entry point's (which also queues fill,
+ * table and resolve kernels): after sd_time_forward_kernels(1) every forward entry point called by this thread records
+ * an event on its stream before and after the launch of its forward tile kernel, and sd_last_forward_kernel_ms() waits
+ * for the later one and returns the milliseconds between them (-1 when there is none).  Off by default; nothing is
+ * recorded on a stream that is being captured. */
+int sd_time_forward_kernels(int on);
+float sd_last_forward_kernel_ms(void);
 /* Dense single-group l-p calls at general p queue two kernels for the same result: one that evaluates every term
  * and one that works from a table of the inputs that can hold a term that counts (per output-channel tile and batch
  * row).  The share of marked table entries, counted on the device, decides which of the two runs: the table kernel

@@ -46,6 +46,8 @@ _OTHER = {
     "sd_version": ([], _i),
     "sd_last_error": ([], ctypes.c_char_p),
     "sd_last_forward_kernel": ([], ctypes.c_char_p),
+    "sd_time_forward_kernels": ([_i], _i),
+    "sd_last_forward_kernel_ms": ([], ctypes.c_float),
     "sd_set_lp_candidate_density": ([_f], _i),
     "sd_set_bound_candidate_density": ([_f], _i),
     "sd_set_bound_candidate_form": ([_i], _i),
@@ -147,3 +149,14 @@ def set_linf_candidate_depth(depth):
 def last_forward_kernel():
     """Name and register tile of the forward tile kernel that this thread's last forward call dispatched."""
     return load().sd_last_forward_kernel().decode()
+
+
+def time_forward_kernels(on):
+    """Switches the events around this thread's forward tile kernel launches on or off."""
+    load().sd_time_forward_kernels(1 if on else 0)
+
+
+def last_forward_kernel_ms():
+    """Duration of the forward tile kernel this thread launched last with timing on (waits for it), or None."""
+    ms = load().sd_last_forward_kernel_ms()
+    return None if ms < 0 else ms

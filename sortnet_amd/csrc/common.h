@@ -73,6 +73,9 @@ void set_error(const char* fmt, ...);
 int check_launch(const char* what);
 // records which forward tile kernel the calling thread dispatched last (sd_last_forward_kernel)
 void note_forward_kernel(const char* kind, int tb, int tm);
+// With sd_time_forward_kernels(1): an event on `stream` before and after a forward tile kernel's launch, for
+// sd_last_forward_kernel_ms.  Nothing while the stream is being captured.
+void forward_kernel_timer(hipStream_t stream, bool after);
 
 #define SD_REQUIRE(cond, ...)                                   \
     do {                                                        \

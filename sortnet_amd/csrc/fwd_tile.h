@@ -508,7 +508,7 @@ namespace sd {
 
 // host-side launcher; the caller has validated shapes
 template <class P, int TB, int TM>
-int launch_fwd(const FwdArgs& a, hipStream_t stream) {
+int launch_fwd_kernel(const FwdArgs& a, hipStream_t stream) {
     // exact dense tiles of the policies that opt in go through the LDS-direct kernel
     if constexpr (P::DIRECT && TB % 4 == 0 && TM % 4 == 0) {
         if (direct_ok<TB, TM, P::MASKABLE>(a)) return launch_fwd_direct<P, TB, TM>(a, stream);
@@ -529,6 +529,14 @@ int launch_fwd(const FwdArgs& a, hipStream_t stream) {
     note_forward_kernel("fwd_kernel", TB, TM);
     hipLaunchKernelGGL((fwd_kernel<P, TB, TM>), grid, dim3(256), 0, stream, a);
     return check_launch("fwd_kernel");
+}
+
+template <class P, int TB, int TM>
+int launch_fwd(const FwdArgs& a, hipStream_t stream) {
+    forward_kernel_timer(stream, false);
+    const int rc = launch_fwd_kernel<P, TB, TM>(a, stream);
+    forward_kernel_timer(stream, true);
+    return rc;
 }
 
 // -------------------------------------------------------------------------------------------

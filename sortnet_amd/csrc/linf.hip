@@ -121,7 +121,11 @@ static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st, void* mer
         if (!a.packed0) return SD_ERR_HIP;
         if ((rc = fill_zero(a.packed0, n * 2, st))) return rc;
     }
-    if (packed_direct) rc = launch_fwd_direct<LinfChunkPacked, 4, 8>(a, st);
+    if (packed_direct) {
+        forward_kernel_timer(st, false);
+        rc = launch_fwd_direct<LinfChunkPacked, 4, 8>(a, st);
+        forward_kernel_timer(st, true);
+    }
     else if (TB == 2) rc = gather ? launch_fwd<P, 2, 8>(a, st) : launch_fwd<P, 2, P::WIDE_TM>(a, st);
     else rc = launch_fwd<P, P::WIDE_TB, P::WIDE_TM>(a, st);
     if (rc) return rc;

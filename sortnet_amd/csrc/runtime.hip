@@ -30,6 +30,26 @@ void note_forward_kernel(const char* kind, int tb, int tm) {
     snprintf(g_fwd_kernel, sizeof(g_fwd_kernel), "%s<%d,%d>", kind, tb, tm);
 }
 
+// sd_time_forward_kernels / sd_last_forward_kernel_ms: two events per thread, created on first use
+static thread_local bool g_time_kernels = false, g_timed = false, g_time_ev_made = false;
+static thread_local hipEvent_t g_time_ev[2];
+
+void forward_kernel_timer(hipStream_t stream, bool after) {
+    if (!g_time_kernels) return;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) { (void)hipGetLastError(); return; }
+    if (cap != hipStreamCaptureStatusNone) return;
+    if (!g_time_ev_made) {
+        if (hipEventCreate(&g_time_ev[0]) != hipSuccess || hipEventCreate(&g_time_ev[1]) != hipSuccess) {
+            (void)hipGetLastError();
+            return;
+        }
+        g_time_ev_made = true;
+    }
+    if (hipEventRecord(g_time_ev[after ? 1 : 0], stream) != hipSuccess) { (void)hipGetLastError(); return; }
+    g_timed = after;
+}
+
 int num_cus() {
     static int cached[64] = {0};
     int dev = 0;
@@ -178,6 +198,19 @@ int sd_version(void) { return 100; }
 const char* sd_last_error(void) { return sd::g_err; }
 
 const char* sd_last_forward_kernel(void) { return sd::g_fwd_kernel; }
+
+int sd_time_forward_kernels(int on) { sd::g_time_kernels = on != 0; sd::g_timed = false; return SD_OK; }
+
+float sd_last_forward_kernel_ms(void) {
+    if (!sd::g_timed) return -1.f;
+    float ms = -1.f;
+    if (hipEventSynchronize(sd::g_time_ev[1]) != hipSuccess ||
+        hipEventElapsedTime(&ms, sd::g_time_ev[0], sd::g_time_ev[1]) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1.f;
+    }
+    return ms;
+}
 
 uint32_t sd_rng_word(uint32_t seed, uint32_t stream_id, uint32_t row, uint32_t col) {
     return sd::rng_word(sd::rng_row_key(seed, stream_id, row), col);

@@ -37,9 +37,10 @@ class DistanceMLP:
     def terms_per_sample(self):
         return sum(w.numel() for w in self.weights)
 
-    def forward(self, x, step_seed, trace=None):
+    def forward(self, x, step_seed, trace=None, after_layer=None):
         """Training forward: x (B, in_features) -> distances to the class prototypes (B, classes).
-        `trace`, a list, receives per layer (input, raw distances, batch mean or None) for inspection."""
+        `trace`, a list, receives per layer (input, raw distances, batch mean or None) for inspection;
+        `after_layer(i, weight)` is called right after layer i's distance op has been queued."""
         h = x.unsqueeze(-1)
         for i, w in enumerate(self.weights):
             h_in = h
@@ -47,6 +48,8 @@ class DistanceMLP:
                 h = F.norm_dist(h, w, float("inf"))
             else:
                 h = F.masked_inf_dist(h, w, self.q, seed=step_seed * 64 + i, mode=self.mask_mode)
+            if after_layer is not None:
+                after_layer(i, w)
             y, mean = h, None
             if i < self.num_layers - 1:
                 h, mean = F.mean_shift(h, self.running_mean[i], self.momentum)
