@@ -18,7 +18,10 @@ def test_more_than_one_gpu_is_refused():
 def test_traffic_figure_comes_from_the_committed_profile():
     sys.path.insert(0, ROOT)
     import bench
-    t = bench.committed_traffic()
+    t = bench.committed_traffic("traffic_bytes_per_launch")
     assert t is not None and 1.4e8 < t < 2e9          # above the 147 MB of algorithmic traffic, below absurd
+    t = bench.committed_traffic("traffic_bytes_per_launch_masked_forward")
+    assert t is not None and 1.3e8 < t < 2e9          # above the 136 MB of algorithmic traffic
+    assert bench.committed_traffic("no_such_figure") is None
     text = open(bench.TRAFFIC_PROFILE).read()
     assert "FETCH_SIZE" in text and "WRITE_SIZE" in text and "rocprofv3" in text
