@@ -103,5 +103,7 @@ void hint_record(int site, const void* weight, int B, int CO, int CI, const unsi
 
 // zero-fill n floats on `stream` with a kernel (graph-capture friendly, no memset node)
 int fill_zero(void* ptr, size_t n_words, hipStream_t stream);
+// the same for two buffers with one launch
+int fill_zero2(void* a, size_t na_words, void* b, size_t nb_words, hipStream_t stream);
 
 }  // namespace sd

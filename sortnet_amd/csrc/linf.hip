@@ -326,8 +326,7 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
         void* ws = workspace(sort_cols_workspace(B, CO, CI, 1), st);   // the only request of this call
         if (!ws) return SD_ERR_HIP;
         if (a.nsplit > 1) {   // the every-term kernel, should it run, merges its slices into zeros
-            if ((rc = fill_zero(outputL, (size_t)B * CO * HW, st))) return rc;
-            if ((rc = fill_zero(outputU, (size_t)B * CO * HW, st))) return rc;
+            if ((rc = fill_zero2(outputL, (size_t)B * CO * HW, outputU, (size_t)B * CO * HW, st))) return rc;
         }
         if ((rc = sort_cols_forward(inputL, inputU, weight, B, CO, CI, 0.f, 1, outputL, outputU, nullptr, ws,
                                     g_bound_density > 0.f ? g_bound_density : kBoundSparseCap, &a.gate, &a.gate_limit, st)))
@@ -336,8 +335,7 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
         return TB == 2 ? launch_fwd<BoundNogradGated, 2, 8>(a, st) : launch_fwd<BoundNogradGated, 4, 8>(a, st);
     }
     if (a.nsplit > 1 || cols) {
-        if ((rc = fill_zero(outputL, (size_t)B * CO * HW, st))) return rc;
-        if ((rc = fill_zero(outputU, (size_t)B * CO * HW, st))) return rc;
+        if ((rc = fill_zero2(outputL, (size_t)B * CO * HW, outputU, (size_t)B * CO * HW, st))) return rc;
     }
     if (cols) {
         void* ws = workspace(bound_cols_workspace(B, CO, CI), st);

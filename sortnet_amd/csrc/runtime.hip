@@ -174,6 +174,29 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t* __restrict__ p
     for (size_t k = n4 * 4 + i; k < n; k += stride) p[k] = 0u;
 }
 
+__global__ void __launch_bounds__(256) fill_zero2_kernel(uint4* __restrict__ a, size_t na4, uint4* __restrict__ b,
+                                                         size_t nb4) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, stride = (size_t)gridDim.x * 256;
+    for (size_t k = i; k < na4; k += stride) a[k] = make_uint4(0u, 0u, 0u, 0u);
+    for (size_t k = i; k < nb4; k += stride) b[k] = make_uint4(0u, 0u, 0u, 0u);
+}
+
+int fill_zero2(void* a, size_t na_words, void* b, size_t nb_words, hipStream_t stream) {
+    if (na_words % 4 != 0 || nb_words % 4 != 0 || reinterpret_cast<uintptr_t>(a) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(b) % 16 != 0) {   // not two runs of whole 16-byte words: one launch each
+        int rc = fill_zero(a, na_words, stream);
+        return rc ? rc : fill_zero(b, nb_words, stream);
+    }
+    const size_t n4 = (na_words > nb_words ? na_words : nb_words) / 4;
+    if (n4 == 0) return SD_OK;
+    size_t blocks = (n4 + 255) / 256;
+    const size_t cap = (size_t)num_cus() * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(fill_zero2_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, reinterpret_cast<uint4*>(a),
+                       na_words / 4, reinterpret_cast<uint4*>(b), nb_words / 4);
+    return check_launch("fill_zero2");
+}
+
 int fill_zero(void* ptr, size_t n_words, hipStream_t stream) {
     if (n_words == 0) return SD_OK;
     if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) {
