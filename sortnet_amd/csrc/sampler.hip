@@ -47,8 +47,11 @@ __device__ __forceinline__ int block_exclusive_scan(int mine, int* wave_total) {
 // The `count` smallest 48-bit keys (word << 16 | channel) are the keys whose word is below the count-th smallest
 // word w, plus the lowest channels among the keys whose word equals w.
 //
-// CACHED (C <= 256 * kCached): the words stay in registers; w is found by bisection over the 32-bit word range
-// with one ballot and population count per register slot, and ties on w are ranked by the ordered scan.
+// CACHED (C <= 256 * kCached): the words stay in registers; w is found by a radix selection over the 32-bit word
+// range (three LDS histograms: bits 31..20, 19..8, 7..0, each followed by a scan that names the bin holding the
+// count-th smallest word among those that match the bins chosen so far), and ties on w are ranked by the ordered
+// scan.  (A bisection over the word range, 32 rounds of counting with a barrier each, took 60 us and more for 16
+// sub-batches of 5120 channels: the kernel occupies 16 compute units and every round is latency.)
 // Otherwise the words are recomputed and the threshold is found by bisection over the whole 48-bit key range.
 constexpr int kCached = 32;
 
@@ -56,6 +59,8 @@ template <bool CACHED>
 __global__ void __launch_bounds__(256) sample_index_lists_kernel(uint32_t seed, int C, int count, int* __restrict__ out) {
     __shared__ int part[2][4];
     __shared__ int wave_total[4];
+    __shared__ int hist[CACHED ? 4096 : 1];
+    __shared__ int sel[2];
     const int tid = threadIdx.x;
     const uint32_t rowkey = rng_row_key(seed, 4u, blockIdx.x);
     const int per = (C + 255) / 256;
@@ -65,16 +70,35 @@ __global__ void __launch_bounds__(256) sample_index_lists_kernel(uint32_t seed, 
         uint32_t word[kCached];
         #pragma unroll
         for (int i = 0; i < kCached; i++) word[i] = rng_word(rowkey, (uint32_t)(c0 + i));
-        // smallest w with #{word <= w} >= count
-        uint32_t lo = 0u, hi = 0xffffffffu;
-        for (int it = 0; it < 32; it++) {
-            const uint32_t mid = lo + ((hi - lo) >> 1);
-            int cnt = 0;
+        // smallest w with #{word <= w} >= count: its bits from the top, `remaining` = its rank among the words
+        // that share the bits found so far
+        uint32_t w = 0u;
+        int remaining = count;
+        #pragma unroll
+        for (int level = 0; level < 3; level++) {
+            const int shift = level == 0 ? 20 : level == 1 ? 8 : 0;
+            const int nbins = level == 2 ? 256 : 4096, own = nbins / 256;
+            for (int k = tid; k < nbins; k += 256) hist[k] = 0;
+            __syncthreads();
             #pragma unroll
-            for (int i = 0; i < kCached; i++) cnt += __popcll(__ballot(c0 + i < c1 && word[i] <= mid));
-            if (block_sum_uniform(cnt, part, it & 1) >= count) hi = mid; else lo = mid + 1u;
+            for (int i = 0; i < kCached; i++) {
+                const bool match = level == 0 || (level == 1 ? (word[i] >> 20) == (w >> 20) : (word[i] >> 8) == (w >> 8));
+                if (c0 + i < c1 && match) atomicAdd(&hist[(word[i] >> shift) & (uint32_t)(nbins - 1)], 1);
+            }
+            __syncthreads();
+            int local = 0;
+            for (int k = 0; k < own; k++) local += hist[tid * own + k];
+            int running = block_exclusive_scan(local, wave_total);
+            for (int k = 0; k < own; k++) {
+                const int h = hist[tid * own + k];
+                if (running < remaining && running + h >= remaining) { sel[0] = tid * own + k; sel[1] = running; }
+                running += h;
+            }
+            __syncthreads();
+            w |= (uint32_t)sel[0] << shift;
+            remaining -= sel[1];
+            __syncthreads();   // sel, hist and wave_total are rewritten by the next level
         }
-        const uint32_t w = hi;
         int below = 0, ties = 0;
         #pragma unroll
         for (int i = 0; i < kCached; i++) {

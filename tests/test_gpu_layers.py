@@ -37,6 +37,17 @@ def test_sampler_matches_oracle(oracle, S, G, C, q):
         assert not np.array_equal(idx[0], idx[1])    # sub-batches get different subsets
 
 
+@pytest.mark.parametrize("C,count", [(5120, 1), (5120, 5120), (5120, 5119), (8192, 4096), (257, 128), (1, 1), (300, 299)])
+def test_sampler_counts_at_the_ends(oracle, C, count):
+    """Counts the probability does not produce (one channel, all but one, all), many seeds: the selection of the
+    count-th smallest word has to name the right bin at every level of its histograms."""
+    from sortnet_amd import ext
+    dev = _dev()
+    for seed in range(20, 28):
+        idx = ext.sample_index_lists(seed, 3, 1, C, count, dev).cpu().numpy()
+        assert np.array_equal(idx, oracle.sample_index_lists(seed, 3, 1, C, count)), seed
+
+
 def test_plain_stack_value_and_bounds(oracle):
     from sortnet_amd.layers import NormDist, BoundSequential, DropoutRegistry
     dev = _dev()
