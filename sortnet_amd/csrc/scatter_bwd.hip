@@ -202,10 +202,77 @@ __global__ void __launch_bounds__(256) wrows_bwd_kernel(BwdArgs a, int WR) {
     for (int n = threadIdx.x; n < nrows * a.CIg; n += 256) out[n] = hist[n];
 }
 
+// The same for the l-inf layer with index lists (core/cuda/inf_dist_cuda.cu:214-275 scatters with global atomics into a
+// zero-filled grad_weight).  A weight row r receives from sub-batch s only when r is in that sub-batch's list of kept
+// outputs, from the output at r's place in the list: row_place_kernel writes the place of every weight row per
+// (sub-batch, group), -1 for rows not kept, so that a workgroup can again own WR weight rows, collect them in LDS over
+// all samples (the position is a place in the sub-batch's list of kept inputs, whose entry is the column) and write
+// them out once, rows nobody kept as zeros.
+__global__ void __launch_bounds__(256) row_place_kernel(const int* __restrict__ co_idx, int COg, int W_COg,
+                                                        int* __restrict__ place) {
+    const int sg = blockIdx.x;                      // sub-batch * G + group
+    int* p = place + (size_t)sg * W_COg;
+    for (int r = threadIdx.x; r < W_COg; r += 256) p[r] = -1;
+    __syncthreads();                                // the fills of this workgroup are ordered before its entries
+    for (int m = threadIdx.x; m < COg; m += 256) {
+        const int r = co_idx[(size_t)sg * COg + m];
+        if (r >= 0 && r < W_COg) p[r] = m;
+    }
+}
+
+__global__ void __launch_bounds__(256) wrows_lists_bwd_kernel(BwdArgs a, int WR, const int* __restrict__ place) {
+    extern __shared__ float hist[];             // [WR][W_CIg]
+    const int rows_total = a.G * a.W_COg;
+    const int die = blockIdx.x & 7, k = blockIdx.x >> 3;
+    const int c0 = ((((k >> 3) * 8 + die) << 3) + (k & 7)) * WR;      // as in wrows_bwd_kernel
+    if (c0 >= rows_total) return;
+    const int nrows = rows_total - c0 < WR ? rows_total - c0 : WR;
+    for (int n = threadIdx.x; n < WR * a.W_CIg; n += 256) hist[n] = 0.f;
+    __syncthreads();
+    const int j = threadIdx.x % WR, rstep = 256 / WR;
+    const int R = a.B * a.HW;
+    if (j < nrows) {
+        const int g = (c0 + j) / a.W_COg, rr = (c0 + j) - g * a.W_COg;
+        float* h = hist + (size_t)j * a.W_CIg;
+        for (int r = threadIdx.x / WR; r < R; r += rstep) {
+            int b = r, hw = 0;
+            if (a.HW > 1) { b = r / a.HW; hw = r - b * a.HW; }
+            const int sg = (b / kSubBatch) * a.G + g;
+            const int m = place ? place[(size_t)sg * a.W_COg + rr] : rr;
+            if (m < 0) continue;
+            const size_t o = ((size_t)(b * a.G + g) * a.COg + m) * a.HW + hw;
+            const float grad = a.g0[o];
+            const int pr = a.p0[o];
+            const int n = pr & 0x7fffffff;
+            if (n >= a.CIg) continue;                // a position outside the list: not followed into LDS
+            const int col = a.ci_idx ? a.ci_idx[(size_t)sg * a.CIg + n] : n;
+            if ((unsigned)col < (unsigned)a.W_CIg) atomicAdd(&h[col], pr >= 0 ? -grad : grad);
+        }
+    }
+    __syncthreads();
+    float* out = a.gw + (size_t)c0 * a.W_CIg;
+    for (int n = threadIdx.x; n < nrows * a.W_CIg; n += 256) out[n] = hist[n];
+}
+
 // launches wrows_bwd_kernel when the layer is dense and a row fits; returns false when the caller has to
 // take the zero-fill + atomics path for grad_weight
 template <int MODE>
 static bool launch_wrows(const BwdArgs& a, hipStream_t st) {
+    if ((a.ci_idx || a.co_idx) && MODE == 0 && a.W_CIg <= kMaxWRowsLds) {
+        int* place = nullptr;
+        if (a.co_idx) {
+            const int SG = (a.B + kSubBatch - 1) / kSubBatch * a.G;
+            place = static_cast<int*>(workspace((size_t)SG * a.W_COg * sizeof(int), st));   // the only request of the call
+            if (!place) return false;
+            hipLaunchKernelGGL(row_place_kernel, dim3((unsigned)SG), dim3(256), 0, st, a.co_idx, a.COg, a.W_COg, place);
+        }
+        int WR = 1;
+        while (WR < 8 && 2 * WR * a.W_CIg <= kMaxWRowsLds) WR *= 2;
+        const int blocks = (a.G * a.W_COg + WR - 1) / WR;
+        hipLaunchKernelGGL(wrows_lists_bwd_kernel, dim3((unsigned)((blocks + 63) / 64 * 64)), dim3(256),
+                           (size_t)WR * a.W_CIg * sizeof(float), st, a, WR, place);
+        return true;
+    }
     if (a.ci_idx || a.co_idx || a.CIg > kMaxWRowsLds) return false;
     int WR = 1;
     while (WR < 8 && 2 * WR * a.CIg <= kMaxWRowsLds) WR *= 2;

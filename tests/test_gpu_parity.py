@@ -152,6 +152,40 @@ def test_inf_dist_index_lists(oracle, B, CI, CO, G, ci_n, co_n):
     ext.inf_dist_forward(xd, wd, y4, p4, G, cid, None)
     r4, rp4 = oracle.inf_dist_forward(x.numpy(), w.numpy(), G, True, ci, None)
     assert np.array_equal(y4.cpu().numpy(), r4) and np.array_equal(p4.cpu().numpy(), rp4)
+    # their backward passes: weight rows nobody kept come back as zeros, rows kept by some sub-batches only from those
+    rgx3, rgw3 = oracle.inf_dist_backward(gy.numpy(), rp3, xfull.shape, w.shape, G, True, None, co)
+    gx3, gw3 = torch.empty(B, CI, 1, device=dev), torch.full_like(wd, float("nan"))
+    ext.inf_dist_backward_input_weight(gd, p3, gx3, gw3, G, None, cod)
+    _close(gx3, rgx3)
+    _close(gw3, rgw3)
+    gy4 = _gen((B, CO, 1), 10)
+    rgx4, rgw4 = oracle.inf_dist_backward(gy4.numpy(), rp4, x.shape, w.shape, G, True, ci, None)
+    gx4, gw4 = torch.empty_like(xd), torch.full_like(wd, float("nan"))
+    ext.inf_dist_backward_input_weight(gy4.to(dev), p4, gx4, gw4, G, cid, None)
+    _close(gx4, rgx4)
+    _close(gw4, rgw4)
+
+
+def test_inf_dist_index_lists_with_spatial_positions(oracle):
+    """Index lists on a layer with HW = 3 and two groups: forward bits and both gradients."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, CI, CO, G, HW, ci_n, co_n = 40, 64, 48, 2, 3, 12, 8
+    ci, co = _index_lists(B, CI, CO, ci_n, co_n, G, 25)
+    w = _gen((CO, CI // G), 26, scale=0.3)
+    x, gy = _gen((B, ci_n * G, HW), 27, "rand"), _gen((B, co_n * G, HW), 28)
+    ry, rpos = oracle.inf_dist_forward(x.numpy(), w.numpy(), G, True, ci, co)
+    xd, wd, gd = x.to(dev), w.to(dev), gy.to(dev)
+    cid, cod = torch.from_numpy(ci).to(dev), torch.from_numpy(co).to(dev)
+    y = torch.empty(B, co_n * G, HW, device=dev)
+    pos = torch.empty(B, co_n * G, HW, device=dev, dtype=torch.int32)
+    ext.inf_dist_forward(xd, wd, y, pos, G, cid, cod)
+    assert np.array_equal(y.cpu().numpy(), ry) and np.array_equal(pos.cpu().numpy(), rpos)
+    rgx, rgw = oracle.inf_dist_backward(gy.numpy(), rpos, x.shape, w.shape, G, True, ci, co)
+    gx, gw = torch.empty_like(xd), torch.full_like(wd, float("nan"))
+    ext.inf_dist_backward_input_weight(gd, pos, gx, gw, G, cid, cod)
+    _close(gx, rgx)
+    _close(gw, rgw)
 
 
 @pytest.mark.parametrize("mode", [0, 1])
