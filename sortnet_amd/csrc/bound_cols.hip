@@ -314,10 +314,18 @@ __global__ void __launch_bounds__(256) xt_kernel(const float* __restrict__ xl, c
     for (int k = 0; k < 4; k++) dst[threadIdx.x + 256 * k] = src[threadIdx.x + 256 * k];
 }
 
+// POS: for the forward that also returns positions.  Every output then carries, next to its running minimum / maximum,
+// the number (within the slice, 8 bits) of the 32-input chunk whose mark last raised it - the marks of a row go by in
+// the order of the inputs and only a strictly better term replaces, so this is the chunk of the first input that
+// attains the result, as the every-term kernel's chunk tracking finds it - and the slices merge as that kernel's do:
+// 64-bit atomic maximum of (value bits << 32 | ~chunk) into packedL / packedU, from which resolve_bound_kernel takes
+// values and positions.  Outputs that no term raised above the 1e-10 start write nothing.
+template <bool POS>
 __device__ __forceinline__ void bound_cols_body(const float* __restrict__ xT, const float* __restrict__ w,
                                                 const uint32_t* __restrict__ bits, const uint32_t* __restrict__ order,
                                                 int B, int M, int Mp, int N, int nsplit, float* __restrict__ yL,
-                                                float* __restrict__ yU, float* smem) {
+                                                float* __restrict__ yU, unsigned long long* __restrict__ packedL,
+                                                unsigned long long* __restrict__ packedU, float* smem) {
     constexpr int TW = 8;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -329,8 +337,9 @@ __device__ __forceinline__ void bound_cols_body(const float* __restrict__ xT, co
     const int st_lo = split * per, st_hi = st_lo + per < NST ? st_lo + per : NST;
 
     float lo[TW][2], hi[TW][2];
+    uint32_t cw[TW];   // POS: chunk numbers of (lower, lower', upper, upper') of a weight row, one byte each, 255 = none
     #pragma unroll
-    for (int r = 0; r < TW; r++) { lo[r][0] = lo[r][1] = -kEps; hi[r][0] = hi[r][1] = kEps; }
+    for (int r = 0; r < TW; r++) { lo[r][0] = lo[r][1] = -kEps; hi[r][0] = hi[r][1] = kEps; cw[r] = 0xffffffffu; }
 
     // the rows at this wavefront's eight places of the block (wave-uniform)
     int row[TW];
@@ -372,18 +381,33 @@ __device__ __forceinline__ void bound_cols_body(const float* __restrict__ xT, co
                 b[r] = bw[(size_t)c1 * Mp + r] & keep;
             }
         };
-        auto term = [&](float (&l2)[2], float (&h2)[2], const float4& x, float wv) __attribute__((always_inline)) {
+        // kl4: the chunk number of the mark within the slice in all four bytes
+        auto term = [&](float (&l2)[2], float (&h2)[2], uint32_t& c4, const float4& x, float wv, uint32_t kl4)
+                        __attribute__((always_inline)) {
             const float a1 = wv - x.x, a2 = x.z - wv, b1 = wv - x.y, b2 = x.w - wv;
-            l2[0] = fminf(fminf(l2[0], a1), a2);
-            h2[0] = fmaxf(fmaxf(h2[0], a1), a2);
-            l2[1] = fminf(fminf(l2[1], b1), b2);
-            h2[1] = fmaxf(fmaxf(h2[1], b1), b2);
+            if (POS) {
+                const float m0 = fminf(a1, a2), M0 = fmaxf(a1, a2), m1 = fminf(b1, b2), M1 = fmaxf(b1, b2);
+                const bool w0 = m0 < l2[0], w1 = m1 < l2[1], w2 = M0 > h2[0], w3 = M1 > h2[1];
+                l2[0] = w0 ? m0 : l2[0]; l2[1] = w1 ? m1 : l2[1];
+                h2[0] = w2 ? M0 : h2[0]; h2[1] = w3 ? M1 : h2[1];
+                c4 = w0 ? ((c4 & 0xffffff00u) | (kl4 & 0x000000ffu)) : c4;
+                c4 = w1 ? ((c4 & 0xffff00ffu) | (kl4 & 0x0000ff00u)) : c4;
+                c4 = w2 ? ((c4 & 0xff00ffffu) | (kl4 & 0x00ff0000u)) : c4;
+                c4 = w3 ? ((c4 & 0x00ffffffu) | (kl4 & 0xff000000u)) : c4;
+            } else {
+                l2[0] = fminf(fminf(l2[0], a1), a2);
+                h2[0] = fmaxf(fmaxf(h2[0], a1), a2);
+                l2[1] = fminf(fminf(l2[1], b1), b2);
+                h2[1] = fmaxf(fmaxf(h2[1], b1), b2);
+            }
         };
         // a weight row's marks of the stage, in order; the operands of the next mark are on their way while the
         // current one is used
-        auto compute = [&](int buf, const float (&wv)[TW], const uint32_t (&wa)[TW], const uint32_t (&wb2)[TW])
+        auto compute = [&](int buf, int st, const float (&wv)[TW], const uint32_t (&wa)[TW], const uint32_t (&wb2)[TW])
                            __attribute__((always_inline)) {
             const float* X = smem + buf * kStageFloats + 4 * lane;
+            const uint32_t k0 = (uint32_t)(2 * (st - st_lo));
+            auto kl4 = [&](int n) __attribute__((always_inline)) { return (k0 + (uint32_t)(n >> 5)) * 0x01010101u; };
             #pragma unroll
             for (int r = 0; r < TW; r++) {
                 unsigned long long bm = ((unsigned long long)wb2[r] << 32) | (unsigned long long)wa[r];
@@ -392,19 +416,22 @@ __device__ __forceinline__ void bound_cols_body(const float* __restrict__ xT, co
                     bm &= bm - 1;
                     float4 xa = *reinterpret_cast<const float4*>(X + n * 256), xb;
                     float va = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv[r]), n)), vb;
+                    uint32_t ka = kl4(n), kb;
                     while (true) {
-                        if (!bm) { term(lo[r], hi[r], xa, va); break; }
+                        if (!bm) { term(lo[r], hi[r], cw[r], xa, va, ka); break; }
                         n = __builtin_ctzll(bm);
                         bm &= bm - 1;
                         xb = *reinterpret_cast<const float4*>(X + n * 256);
                         vb = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv[r]), n));
-                        term(lo[r], hi[r], xa, va);
-                        if (!bm) { term(lo[r], hi[r], xb, vb); break; }
+                        kb = kl4(n);
+                        term(lo[r], hi[r], cw[r], xa, va, ka);
+                        if (!bm) { term(lo[r], hi[r], cw[r], xb, vb, kb); break; }
                         n = __builtin_ctzll(bm);
                         bm &= bm - 1;
                         xa = *reinterpret_cast<const float4*>(X + n * 256);
                         va = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv[r]), n));
-                        term(lo[r], hi[r], xb, vb);
+                        ka = kl4(n);
+                        term(lo[r], hi[r], cw[r], xb, vb, kb);
                     }
                 }
             }
@@ -420,7 +447,7 @@ __device__ __forceinline__ void bound_cols_body(const float* __restrict__ xT, co
             const int buf = (st - st_lo) & 1;
             const int nx = st + 1 < st_hi ? st + 1 : st;   // the last stage is fetched once more rather than behind a test
             load_x(nx, xs); load_w(nx, wn); load_words(nx, n0, n1);
-            compute(buf, wc, a0, a1);
+            compute(buf, st, wc, a0, a1);
             store_x(buf ^ 1, xs);
             #pragma unroll
             for (int r = 0; r < TW; r++) { wc[r] = wn[r]; a0[r] = n0[r]; a1[r] = n1[r]; }
@@ -428,6 +455,37 @@ __device__ __forceinline__ void bound_cols_body(const float* __restrict__ xT, co
         }
     }
 
+    if (POS) {
+        // (value, chunk) pairs: [batch row][weight row] through LDS, lower then upper, values and chunk numbers side by side
+        float* tv = smem;
+        uint32_t* tc = reinterpret_cast<uint32_t*>(smem) + kTileB * (kTileW + 1);
+        const uint32_t c_first = (uint32_t)(2 * st_lo);
+        #pragma unroll
+        for (int which = 0; which < 2; which++) {
+            __syncthreads();
+            #pragma unroll
+            for (int r = 0; r < TW; r++) {
+                #pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    tv[(lane + 64 * j) * (kTileW + 1) + row[r]] = which == 0 ? -lo[r][j] : hi[r][j];
+                    tc[(lane + 64 * j) * (kTileW + 1) + row[r]] = (cw[r] >> (16 * which + 8 * j)) & 0xffu;
+                }
+            }
+            __syncthreads();
+            unsigned long long* y = which == 0 ? packedL : packedU;
+            for (int e = tid; e < kTileB * kTileW; e += 1024) {
+                const int bl = e >> 7, ml = e & (kTileW - 1);
+                const uint32_t kl = tc[bl * (kTileW + 1) + ml];
+                if (b0 + bl < B && m0 + ml < M && kl != 0xffu) {
+                    const unsigned long long key =
+                        ((unsigned long long)__float_as_uint(tv[bl * (kTileW + 1) + ml]) << 32) |
+                        (unsigned long long)(0xffffffffu - (c_first + kl));
+                    atomicMax(y + (size_t)(b0 + bl) * M + m0 + ml, key);
+                }
+            }
+        }
+        return;
+    }
     // results: [batch row][weight row] through LDS, lower then upper
     float* tr = smem;
     #pragma unroll
@@ -754,15 +812,18 @@ __device__ __forceinline__ void bound_rows_body(const float* __restrict__ xl, co
 }
 
 // One launch for both orientations (same grid, same LDS): whichever table is below its limit is used
+template <bool POS>
 __global__ void __launch_bounds__(1024, 1)
 bound_table_kernel(const float* __restrict__ xl, const float* __restrict__ xu, const float* __restrict__ w,
                    const float* __restrict__ xT, const uint32_t* __restrict__ bits, const uint32_t* __restrict__ order,
                    const unsigned long long* __restrict__ count, unsigned long long limit_col,
                    unsigned long long limit_row, int B, int Bp, int M, int Mp, int N, int nsplit,
-                   float* __restrict__ yL, float* __restrict__ yU) {
+                   float* __restrict__ yL, float* __restrict__ yU, unsigned long long* __restrict__ packedL,
+                   unsigned long long* __restrict__ packedU) {
     __shared__ __attribute__((aligned(16))) float lds[kLdsWords];
-    if (count[0] <= limit_col) bound_cols_body(xT, w, bits, order, B, M, Mp, N, nsplit, yL, yU, lds);
-    else if (count[1] <= limit_row)
+    if (count[0] <= limit_col)
+        bound_cols_body<POS>(xT, w, bits, order, B, M, Mp, N, nsplit, yL, yU, packedL, packedU, lds);
+    else if (!POS && count[1] <= limit_row)   // positions are only tracked with the tables per weight row
         bound_rows_body(xl, xu, w, bits, B, Bp, M, N, nsplit, yL, yU, lds,
                         reinterpret_cast<uint32_t*>(lds + 2 * kMainTileFloats));
 }
@@ -775,8 +836,11 @@ size_t bound_cols_workspace(int B, int CO, int CI) {
 }
 
 int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float* outL,
-                       float* outU, void* ws, float density, float density_rows, const unsigned long long** gate,
-                       unsigned long long* gate_limit, hipStream_t st) {
+                       float* outU, unsigned long long* packedL, unsigned long long* packedU, void* ws, float density,
+                       float density_rows, const unsigned long long** gate, unsigned long long* gate_limit,
+                       hipStream_t st) {
+    const bool with_pos = packedL != nullptr;
+    if (with_pos) density_rows = 0.f;   // the kernel of the tables per batch row tracks no positions
     if (CI % kChunk != 0 || B < 1 || CO < 1) { set_error("bound_cols_forward: shape not supported"); return SD_ERR_ARG; }
     const Carve c = carve(ws, B, CO, CI);
     const int S = tiles_b(B), Mp = mpad_of(CO), Bp = bpad_of(B), T = Mp / kTileW, NCH = CI / kChunk;
@@ -820,8 +884,16 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
         const double cost = (double)((wgs * n + cus - 1) / cus) / n * (1.0 + 0.04 * n);
         if (n == 1 || cost < best) { best = cost; nsplit = n; }
     }
-    hipLaunchKernelGGL(bound_table_kernel, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.xt, c.bits,
-                       c.order, c.count, limit_col, limit_row, B, Bp, CO, Mp, CI, nsplit, outL, outU);
+    if (with_pos) {
+        // chunk numbers within a slice take 8 bits (255 = none)
+        while ((((NCH + 1) / 2 + nsplit - 1) / nsplit) * 2 > 254) nsplit++;
+        hipLaunchKernelGGL(bound_table_kernel<true>, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.xt,
+                           c.bits, c.order, c.count, limit_col, limit_row, B, Bp, CO, Mp, CI, nsplit, outL, outU, packedL,
+                           packedU);
+        return check_launch("bound_table_kernel");
+    }
+    hipLaunchKernelGGL(bound_table_kernel<false>, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.xt, c.bits,
+                       c.order, c.count, limit_col, limit_row, B, Bp, CO, Mp, CI, nsplit, outL, outU, nullptr, nullptr);
     return check_launch("bound_table_kernel");
 }
 

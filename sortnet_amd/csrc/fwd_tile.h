@@ -769,6 +769,7 @@ struct BoundNogradGated : BoundNograd {
 // -min(t1,t2) (a positive number once it passes 1e-10), the upper side the largest max(t1,t2);
 // resolve_bound_kernel recovers the exact positions and branch bits
 struct BoundChunk : PolicyBase {
+    static constexpr bool GATED = true;   // one of two queued for a result when FwdArgs::gate is set
     static constexpr int NX = 2;
     static constexpr int PIPE_WAVES = 2;
     static constexpr int MIN_WAVES = 2;
@@ -1263,68 +1264,89 @@ __global__ void __launch_bounds__(256) resolve_pos_kernel(FwdArgs a) {
 // Position resolve of the interval kernel: rescans the winning chunk of the lower and of the upper
 // bound for the first input attaining the bound and rebuilds pos = n | (t1 <= t2 ? 0 : 1 << 31);
 // a lower bound that never left its -1e-10 start keeps the 0xffffffff "no gradient" position.
+// As resolve_pos_kernel: a wavefront owns 64 consecutive outputs, posts what the rescan needs in LDS and walks its
+// outputs two at a time, 32 lanes per output and one input of the winning chunk per lane (coalesced 128-byte pieces
+// of l, u and the weight row, for the lower and then for the upper bound); a ballot finds the first input whose term
+// equals the bound bit for bit, a second one says which of its two terms it was.
+struct ResolveBoundSlot { int cl, cu; float vl, vu; unsigned long long xoff, woff; };
+
 template <bool PACKED>
 __global__ void __launch_bounds__(256) resolve_bound_kernel(FwdArgs a) {
-    long long total = (long long)a.R * a.G * a.COg;
-    long long o = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (o >= total) return;
-    int hw = (int)(o % a.HW);
-    long long t = o / a.HW;
-    int c = (int)(t % (a.G * a.COg));
-    int b = (int)(t / (a.G * a.COg));
-    int g = c / a.COg;
-    float vl, vu; int cl, cu;
-    if (PACKED) {
-        unsigned long long pl = a.packed0[o], pu = a.packed1[o];
-        uint32_t ll = (uint32_t)pl, lu = (uint32_t)pu;
-        vl = ll ? __uint_as_float((uint32_t)(pl >> 32)) : kEps; cl = ll ? (int)(0xffffffffu - ll) : -1;
-        vu = lu ? __uint_as_float((uint32_t)(pu >> 32)) : kEps; cu = lu ? (int)(0xffffffffu - lu) : -1;
-    } else { vl = a.y0[o]; cl = a.p0[o]; vu = a.y1[o]; cu = a.p1[o]; }
-    const float* wr = a.w + (size_t)c * a.CIg;
-    const size_t xb = ((size_t)(b * a.G + g) * a.CIg) * a.HW + hw;
+    __shared__ __attribute__((aligned(16))) ResolveBoundSlot slots[4][64];
+    const long long total = (long long)a.R * a.G * a.COg;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long long o_base = ((long long)blockIdx.x * 4 + wave) * 64;
+    if (o_base >= total) return;                       // whole wavefront; no workgroup barrier below
+    const long long o = o_base + lane;
+    const bool mine = o < total;
+    ResolveBoundSlot me;
+    me.cl = me.cu = -1; me.vl = me.vu = kEps; me.xoff = me.woff = 0ull;
+    if (mine) {
+        const int hw = (int)(o % a.HW);
+        const long long t = o / a.HW;
+        const int c = (int)(t % (a.G * a.COg));
+        const int b = (int)(t / (a.G * a.COg));
+        const int g = c / a.COg;
+        if (PACKED) {
+            const unsigned long long pl = a.packed0[o], pu = a.packed1[o];
+            const uint32_t ll = (uint32_t)pl, lu = (uint32_t)pu;
+            me.vl = ll ? __uint_as_float((uint32_t)(pl >> 32)) : kEps; me.cl = ll ? (int)(0xffffffffu - ll) : -1;
+            me.vu = lu ? __uint_as_float((uint32_t)(pu >> 32)) : kEps; me.cu = lu ? (int)(0xffffffffu - lu) : -1;
+        } else { me.vl = a.y0[o]; me.cl = a.p0[o]; me.vu = a.y1[o]; me.cu = a.p1[o]; }
+        me.woff = (unsigned long long)c * a.CIg;
+        me.xoff = ((unsigned long long)(b * a.G + g) * a.CIg) * a.HW + hw;
+    }
+    slots[wave][lane] = me;
+    __builtin_amdgcn_wave_barrier();                   // LDS operations of one wavefront complete in order
+
+    const int half = lane >> 5, l = lane & 31;
     uint32_t posl = kNanId, posu = 0u;
-    #pragma unroll
-    for (int side = 0; side < 2; side++) {
-        const int cid = side ? cu : cl;
-        if (cid < 0) continue;
-        const int n0 = cid * KT, n1 = n0 + KT < a.CIg ? n0 + KT : a.CIg;
-        const float target = side ? vu : vl;
-        uint32_t found = side ? 0u : kNanId;
-        auto probe = [&](float l, float u, float w, int n) {
-            if (l > u) l = u = (l + u) * 0.5f;
-            float t1 = w - l, t2 = u - w;
-            float v = side ? fmaxf(t1, t2) : -fminf(t1, t2);
-            if (v == target) found = (uint32_t)n | (t1 <= t2 ? 0u : kSign);
-        };
-        if (a.fast_x && a.fast_w) {
-            // descending scan over 128-bit loads: the lowest matching input is the one that remains
-            float4 lv[KT / 4], uv[KT / 4], wv[KT / 4];
+    constexpr int U = 4;
+    for (int it0 = 0; it0 < 32; it0 += U) {
+        float t1[U][2], t2[U][2], target[U][2];
+        bool cand[U][2];
+        int nn[U][2];
+        #pragma unroll
+        for (int u = 0; u < U; u++) {
+            const ResolveBoundSlot q = slots[wave][2 * (it0 + u) + half];
             #pragma unroll
-            for (int q4 = 0; q4 < KT / 4; q4++) {
-                int n = n0 + 4 * q4;
-                if (n > a.CIg - 4) n = a.CIg - 4;
-                lv[q4] = *reinterpret_cast<const float4*>(a.x0 + xb + n);
-                uv[q4] = *reinterpret_cast<const float4*>(a.x1 + xb + n);
-                wv[q4] = *reinterpret_cast<const float4*>(wr + n);
+            for (int side = 0; side < 2; side++) {
+                const int cid = side ? q.cu : q.cl;
+                int n = (cid < 0 ? 0 : cid) * KT + l;
+                cand[u][side] = cid >= 0 && n < a.CIg;
+                if (n >= a.CIg) n = 0;
+                float lv = a.x0[q.xoff + (size_t)n * a.HW], uv = a.x1[q.xoff + (size_t)n * a.HW];
+                const float wv = a.w[q.woff + n];
+                if (lv > uv) lv = uv = (lv + uv) * 0.5f;
+                t1[u][side] = wv - lv; t2[u][side] = uv - wv;
+                target[u][side] = side ? q.vu : q.vl;
+                nn[u][side] = n;
             }
+        }
+        #pragma unroll
+        for (int u = 0; u < U; u++) {
             #pragma unroll
-            for (int q4 = KT / 4 - 1; q4 >= 0; q4--) {
-                const int n = n0 + 4 * q4;
-                if (n < a.CIg) {
-                    probe(lv[q4].w, uv[q4].w, wv[q4].w, n + 3);
-                    probe(lv[q4].z, uv[q4].z, wv[q4].z, n + 2);
-                    probe(lv[q4].y, uv[q4].y, wv[q4].y, n + 1);
-                    probe(lv[q4].x, uv[q4].x, wv[q4].x, n);
+            for (int side = 0; side < 2; side++) {
+                const float v = side ? fmaxf(t1[u][side], t2[u][side]) : -fminf(t1[u][side], t2[u][side]);
+                const unsigned long long hit = __ballot(cand[u][side] && v == target[u][side]);
+                const unsigned long long second = __ballot(!(t1[u][side] <= t2[u][side]));
+                if ((lane >> 1) == it0 + u) {          // the two owner lanes of this step
+                    const uint32_t h32 = (lane & 1) ? (uint32_t)(hit >> 32) : (uint32_t)hit;
+                    const uint32_t s32 = (lane & 1) ? (uint32_t)(second >> 32) : (uint32_t)second;
+                    if (h32) {
+                        const int first = __ffs((int)h32) - 1;
+                        const int cid = side ? me.cu : me.cl;
+                        const uint32_t found = (uint32_t)(cid * KT + first) | (((s32 >> first) & 1u) ? kSign : 0u);
+                        if (side) posu = found; else posl = found;
+                    }
                 }
             }
-        } else {
-            for (int n = n1 - 1; n >= n0; n--)
-                probe(a.x0[xb + (size_t)n * a.HW], a.x1[xb + (size_t)n * a.HW], wr[n], n);
         }
-        if (side) posu = found; else posl = found;
     }
-    a.y0[o] = vl; a.y1[o] = vu;
-    a.p0[o] = (int)posl; a.p1[o] = (int)posu;
+    if (mine) {
+        a.y0[o] = me.vl; a.y1[o] = me.vu;
+        a.p0[o] = (int)posl; a.p1[o] = (int)posu;
+    }
 }
 
 inline int launch_resolve_bound(const FwdArgs& a, hipStream_t stream) {

@@ -20,7 +20,11 @@ constexpr float kBoundColsCap = 0.30f, kBoundRowsCap = 0.26f;
 // kernel takes about 0.19 ms, which is what the every-term kernel needs for 2.4 G terms (512 x 10 x 5120: 0.06 ms
 // for every term against 0.10 ms from tables).
 constexpr long long kBoundColsMinTerms = 1ll << 31;
-constexpr int kHintSiteBound = 1, kHintSiteBoundSparse = 8;
+// The forward that also returns positions: its table kernel spends about twice as long per mark (a compare and two
+// selects per output instead of a three-operand minimum or maximum) and the every-term kernel 1.5 times as long per
+// term, so the limit is lower.
+constexpr float kBoundPosColsCap = 0.15f;
+constexpr int kHintSiteBound = 1, kHintSiteBoundSparse = 8, kHintSiteBoundPos = 9;
 constexpr float kBoundSparseCap = 0.03f;   // marked share up to which the kernel without LDS staging runs
 static int g_bound_form = 0;              // 0: chosen per layer, 1: staged tiles, 2: transposed-row walk
 
@@ -340,7 +344,7 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
     if (cols) {
         void* ws = workspace(bound_cols_workspace(B, CO, CI), st);
         if (!ws) return SD_ERR_HIP;
-        if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, outputL, outputU, ws, cap,
+        if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, outputL, outputU, nullptr, nullptr, ws, cap,
                                      g_bound_density >= 0.f ? g_bound_density : kBoundRowsCap, &a.gate, &a.gate_limit, st)))
             return rc;
         a.gate_above = 1;
@@ -381,14 +385,31 @@ extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* input
     static const int kTb42[] = {4, 2};
     const int TB = pick_tb(a, kTb42, 2, 64);
     a.nsplit = pick_nsplit(a, 16 * TB, 64);
+    // dense single-group layers: the table kernel per weight row, tracking the chunk of every result, is queued in front
+    // of the every-term kernel as for the forward without positions; both leave (value, chunk) pairs for the resolve
+    const float cap = g_bound_density >= 0.f ? g_bound_density : kBoundPosColsCap;
+    bool cols = cap > 0.f && G == 1 && HW == 1 && CI % kColsChunk == 0 && a.fast_x && a.fast_w &&
+                (g_bound_density >= 0.f || (long long)B * CO * CI >= kBoundColsMinTerms);
+    const bool hinted = cols && g_bound_density < 0.f;
+    if (hinted && !hint_build_tables(kHintSiteBoundPos, weight, B, CO, CI, st)) cols = false;
+    if (cols && a.nsplit < 2) a.nsplit = 2;   // both kernels merge into the packed pairs
     if (a.nsplit > 1) {
         size_t n = (size_t)a.R * a.G * a.COg;
-        a.packed0 = static_cast<unsigned long long*>(workspace(n * 16, st));
-        if (!a.packed0) return SD_ERR_HIP;
+        const size_t pairs = (n * 16 + 255) / 256 * 256;
+        char* ws = static_cast<char*>(workspace(pairs + (cols ? bound_cols_workspace(B, CO, CI) : 0), st));   // the only request
+        if (!ws) return SD_ERR_HIP;
+        a.packed0 = reinterpret_cast<unsigned long long*>(ws);
         a.packed1 = a.packed0 + n;
         if ((rc = fill_zero(a.packed0, n * 4, st))) return rc;
+        if (cols) {
+            if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, nullptr, nullptr, a.packed0, a.packed1,
+                                         ws + pairs, cap, 0.f, &a.gate, &a.gate_limit, st)))
+                return rc;
+            a.gate_above = 1;
+        }
     }
     rc = TB == 2 ? launch_fwd<BoundChunk, 2, 4>(a, st) : launch_fwd<BoundChunk, 4, 4>(a, st);
     if (rc) return rc;
+    if (hinted && cols) hint_record(kHintSiteBoundPos, weight, B, CO, CI, a.gate, st);   // the gate is 1 when every term ran
     return launch_resolve_bound(a, st);
 }

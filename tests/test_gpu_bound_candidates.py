@@ -71,6 +71,61 @@ def test_bound_candidate_kernel_matches_oracle(oracle, density, dens, form, B, C
             assert np.array_equal(yu.cpu().numpy(), ru), tag
 
 
+@pytest.mark.parametrize("dens", [1.0, 0.0, -1.0])
+@pytest.mark.parametrize("B,CI,CO", [(70, 96, 64), (33, 2048, 300), (130, 1024, 513), (1, 32, 1), (257, 320, 129),
+                                     (512, 512, 640), (700, 160, 72)])
+def test_bound_candidate_kernel_with_positions_matches_oracle(oracle, density, dens, B, CI, CO):
+    """The forward that also returns positions: values, positions and the "no gradient" position of a lower bound that
+    stayed at its floor are the oracle's bits whether the table kernel (with its chunk tracking) or the every-term
+    kernel leaves the (value, chunk) pairs; ties between inputs included (columns duplicated)."""
+    from sortnet_amd import ext
+    dev = _dev()
+    density(dens)
+    for kind in ("rows_alike", "random", "inverted", "images"):
+        for wscale in (0.02, 1.0):
+            xl, xu = _intervals(B, CI, kind, B + CI + 1)
+            g = torch.Generator().manual_seed(3)
+            w = (torch.randn(CO, CI, generator=g) * wscale).contiguous()
+            if CI >= 64:   # equal terms at different inputs, in one chunk and in different chunks: the lowest input wins
+                for src, dst in ((3, 17), (5, CI - 2)):
+                    xl[:, dst], xu[:, dst], w[:, dst] = xl[:, src], xu[:, src], w[:, src]
+            rl, ru, rpl, rpu = oracle.bound_inf_dist_forward(xl.numpy(), xu.numpy(), w.numpy(), 1, need_pos=True)
+            yl = torch.full((B, CO, 1), float("nan"), device=dev)
+            yu = torch.full((B, CO, 1), float("nan"), device=dev)
+            pl = torch.full((B, CO, 1), -7, device=dev, dtype=torch.int32)
+            pu = torch.full((B, CO, 1), -7, device=dev, dtype=torch.int32)
+            ext.bound_inf_dist_forward(xl.to(dev), xu.to(dev), w.to(dev), yl, yu, pl, pu, 1)
+            tag = "dens=%g %s wscale=%g" % (dens, kind, wscale)
+            assert np.array_equal(yl.cpu().numpy(), rl), tag
+            assert np.array_equal(yu.cpu().numpy(), ru), tag
+            assert np.array_equal(pl.cpu().numpy(), rpl), tag
+            assert np.array_equal(pu.cpu().numpy(), rpu), tag
+
+
+def test_bound_candidate_kernel_with_positions_at_layer_size(density):
+    """B = 512, N = M = 5120 with rows that are nearly alike: table kernel, every-term kernel and the built-in choice
+    give the same values and positions."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, N, M = 512, 5120, 5120
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(1, N, 1, generator=g) * 0.02 + torch.randn(B, N, 1, generator=g) * 0.004
+    r = 0.02 + torch.rand(B, N, 1, generator=g) * 0.002
+    xl, xu = (x - r).contiguous().to(dev), (x + r).contiguous().to(dev)
+    w = (torch.randn(M, N, generator=g) * N ** -0.5).contiguous().to(dev)
+    out = {}
+    for dens in (0.0, 1.0, -1.0):
+        density(dens)
+        yl, yu = torch.empty(B, M, 1, device=dev), torch.empty(B, M, 1, device=dev)
+        pl = torch.empty(B, M, 1, device=dev, dtype=torch.int32)
+        pu = torch.empty(B, M, 1, device=dev, dtype=torch.int32)
+        ext.bound_inf_dist_forward(xl, xu, w, yl, yu, pl, pu, 1)
+        out[dens] = (yl, yu, pl, pu)
+    for dens in (1.0, -1.0):
+        for a, b in zip(out[dens], out[0.0]):
+            assert torch.equal(a, b), dens
+
+
 @pytest.mark.parametrize("dens,form", [(1.0, 1), (1.0, 2), (0.0, 0)])
 @pytest.mark.parametrize("kind", ["rows_alike", "images"])
 def test_bound_candidate_kernel_undefined_and_infinite_entries(oracle, density, dens, form, kind):
