@@ -13,6 +13,14 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _built_in_limits_afterwards():
+    """A test that sets a candidate-table limit by hand leaves the built-in ones behind, pass or fail."""
+    yield
+    from sortnet_amd import _lib
+    _lib.set_bound_candidate_density(-1.0)
+
+
 def _dev():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
@@ -188,21 +196,27 @@ def test_graph_replays_of_the_candidate_table_kernels(oracle):
     candidate-table kernel and an every-term kernel for the same result and a count taken on the device picks one, so ONE captured graph serves both kinds of data: replays on weights far
     smaller than the inputs (the table kernel runs) and on weights as large as the inputs (the every-term kernels
     run) must both reproduce eager calls, and the oracle."""
-    from sortnet_amd import ext
+    from sortnet_amd import ext, _lib
     dev = _dev()
     B, CI, CO, p = 160, 1024, 300, 64.0
     g = torch.Generator().manual_seed(25)
+    # the interval forward's built-in limits leave layers of this size to the every-term kernel: a limit set by hand
+    # applies at any size, and the count on the device still decides between the two kernels
+    _lib.set_bound_candidate_density(0.25)
     x = torch.empty(B, CI, 1, device=dev); w = torch.empty(CO, CI, device=dev); gy = torch.empty(B, CO, 1, device=dev)
 
     def outputs():
         return dict(y=torch.empty(B, CO, 1, device=dev), gx=torch.empty_like(x), gw=torch.empty_like(w),
                     gx2=torch.empty_like(x), yl=torch.empty(B, CO, 1, device=dev), yu=torch.empty(B, CO, 1, device=dev),
                     ys=torch.empty(B, CO, 1, device=dev), ysl=torch.empty(B, CO, 1, device=dev),
-                    ysu=torch.empty(B, CO, 1, device=dev))
+                    ysu=torch.empty(B, CO, 1, device=dev), zl=torch.empty(B, CO, 1, device=dev),
+                    zu=torch.empty(B, CO, 1, device=dev), pl=torch.empty(B, CO, 1, device=dev, dtype=torch.int32),
+                    pu=torch.empty(B, CO, 1, device=dev, dtype=torch.int32))
 
     def run(o):
         # the interval forward makes the same kind of choice (rows of the batch alike or not)
         ext.bound_inf_dist_forward_nograd(x - 0.03, x + 0.03, w, o["yl"], o["yu"], 1)
+        ext.bound_inf_dist_forward(x - 0.03, x + 0.03, w, o["zl"], o["zu"], o["pl"], o["pu"], 1)
         # so do the sort neuron and its interval bounds
         ext.sort_neuron_forward_nograd(x, w, o["ys"], 1, 0.5, 6)
         ext.bound_sort_neuron_forward(x - 0.03, x + 0.03, w, o["ysl"], o["ysu"], 1, 0.5, 6)
@@ -235,13 +249,16 @@ def test_graph_replays_of_the_candidate_table_kernels(oracle):
         graph.replay()
         torch.cuda.synchronize()
         for name in eager:
-            if name in ("yl", "yu", "ys", "ysl", "ysu"):
+            if name in ("yl", "yu", "ys", "ysl", "ysu", "zl", "zu", "pl", "pu"):
                 assert torch.equal(captured[name], eager[name]), "%s, replay %d" % (name, replay)
                 continue
             a, b = captured[name].cpu().numpy(), eager[name].cpu().numpy()
             np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-4 * float(np.abs(b).max()), err_msg="%s, replay %d" % (name, replay))
         rl, ru = oracle.bound_inf_dist_forward((x - 0.03).cpu().numpy(), (x + 0.03).cpu().numpy(), w.cpu().numpy(), 1, need_pos=False)
         assert np.array_equal(captured["yl"].cpu().numpy(), rl) and np.array_equal(captured["yu"].cpu().numpy(), ru), replay
+        _, _, rpl, rpu = oracle.bound_inf_dist_forward((x - 0.03).cpu().numpy(), (x + 0.03).cpu().numpy(), w.cpu().numpy(), 1, need_pos=True)
+        assert np.array_equal(captured["zl"].cpu().numpy(), rl) and np.array_equal(captured["zu"].cpu().numpy(), ru), replay
+        assert np.array_equal(captured["pl"].cpu().numpy(), rpl) and np.array_equal(captured["pu"].cpu().numpy(), rpu), replay
         rs = oracle.sort_neuron_forward(x.cpu().numpy(), w.cpu().numpy(), 0.5, 6, need_pos=False)
         np.testing.assert_allclose(captured["ys"].cpu().numpy(), rs, rtol=1e-5, err_msg="replay %d" % replay)
         rsl, rsu = oracle.bound_sort_neuron_forward((x - 0.03).cpu().numpy(), (x + 0.03).cpu().numpy(), w.cpu().numpy(), 0.5, 6)
