@@ -366,6 +366,42 @@ def run_lp_layer(args, p, steps, warmup):
                         "x~N(0,1), w~N(0,1/N)" % (B, N, N, p)}
 
 
+def run_interval_layer(args, steps, warmup):
+    """One interval layer of the headline width as certified training differentiates it: forward with positions and
+    backward (both input gradients and grad_weight), on bounds that are alike from sample to sample (those of a hidden
+    layer) and weights ~ N(0, 1/N)."""
+    import torch
+    from sortnet_amd import ext
+    dev = torch.device("cuda:0")
+    B, N = args.batch, args.width
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(1, N, 1, generator=g) * 0.02 + torch.randn(B, N, 1, generator=g) * 0.004
+    r = 0.02 + torch.rand(B, N, 1, generator=g) * 0.002
+    xl, xu = (x - r).contiguous().to(dev), (x + r).contiguous().to(dev)
+    w = (torch.randn(N, N, generator=g) * N ** -0.5).to(dev)
+    gl, gu = torch.randn(B, N, 1, generator=g).to(dev), torch.randn(B, N, 1, generator=g).to(dev)
+    yl, yu = torch.empty(B, N, 1, device=dev), torch.empty(B, N, 1, device=dev)
+    pl = torch.empty(B, N, 1, device=dev, dtype=torch.int32)
+    pu = torch.empty_like(pl)
+    gxl, gxu, gw = torch.empty_like(xl), torch.empty_like(xu), torch.empty_like(w)
+
+    def step():
+        ext.bound_inf_dist_forward(xl, xu, w, yl, yu, pl, pu, 1)
+        ext.bound_inf_dist_backward_input_weight(gl, gu, pl, pu, gxl, gxu, gw, 1)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {"ms_per_step": ms, "samples_per_s": B / (ms * 1e-3), "steps": steps,
+            "workload": "one interval layer %dx%dx%d with positions: forward + backward (both inputs and weight), "
+                        "bounds alike from sample to sample, w~N(0,1/N)" % (B, N, N)}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -481,6 +517,7 @@ def main():
         sec["index_lists_q0.75_p8"] = {k: r[k] for k in ("ms_per_step", "samples_per_s", "steps", "workload")}
         for pp in (8.0, 64.0):
             sec["lp_layer_p%g" % pp] = run_lp_layer(args, pp, short, warm)
+        sec["interval_layer_with_pos"] = run_interval_layer(args, short, warm)
         if (args.batch, args.width, args.in_features, args.classes) == (512, 5120, 3072, 10):
             r = run_masked(args, args.mask, args.q, short, warm, batch=256, in_features=12288, width=10240, classes=200,
                            eps=1.0 / 255)
