@@ -77,8 +77,8 @@ int sd_set_lp_candidate_density(float density);
  * from a table of the inputs that can hold the maximum of a weight row over a tile of 128 batch rows, and the kernel
  * that evaluates every term; both give the same bits.  Built-in limits: 0.30 (0.26 where the table is built per batch
  * row and tile of 128 weight rows instead, which the call decides from its operands), layers of at least 2^31 terms;
- * a `density` of 0 or more applies at any size.  The form with positions uses the table per weight row only, with a
- * built-in limit of 0.15; values and positions are the every-term kernel's.  No reference counterpart
+ * a `density` of 0 or more applies at any size.  The form with positions has a built-in limit of 0.15; values and
+ * positions are the every-term kernel's.  No reference counterpart
  * (core/cuda/bound_inf_dist_cuda.cu evaluates every term). */
 int sd_set_bound_candidate_density(float density);
 /* Which table kernel serves sd_bound_inf_dist_forward_nograd: 1 = the one that stages tiles of inputs and weights

@@ -26,8 +26,7 @@ size_t bound_cols_workspace(int B, int CO, int CI);
 // per weight row are so few (below a sixteenth of the limit) that a kernel without LDS staging would serve better.
 // With packedL / packedU (B x CO words each, zero-filled) instead of outL / outU the table kernel leaves (value bits
 // << 32 | ~chunk of 32 inputs) per output, merged by atomic maximum, as the every-term kernel with chunk tracking does
-// (fwd_tile.h: store_chunk_winner), for resolve_bound_kernel to take values and positions from; only the tables per
-// weight row serve this form.
+// (fwd_tile.h: store_chunk_winner), for resolve_bound_kernel to take values and positions from.
 int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float* outL,
                        float* outU, unsigned long long* packedL, unsigned long long* packedU, void* ws, float density,
                        float density_rows, const unsigned long long** gate, unsigned long long* gate_limit,

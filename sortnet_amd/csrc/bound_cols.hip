@@ -694,10 +694,13 @@ __global__ void __launch_bounds__(1024) sum_tables_kernel(const uint32_t* __rest
 // of 64 chunks at a time are copied to LDS ahead of the loop over them; a chunk nobody marks is not staged.  One
 // loop per batch row over that row's own marks (find-first-set, clear, branch); the results are written along the
 // weight rows as they are.
+// POS as in bound_cols_body: a batch row's marks go by in input order as well.
+template <bool POS>
 __device__ __forceinline__ void bound_rows_body(const float* __restrict__ xl, const float* __restrict__ xu,
                                                 const float* __restrict__ w, const uint32_t* __restrict__ bits, int B,
                                                 int Bp, int M, int N, int nsplit, float* __restrict__ yL,
-                                                float* __restrict__ yU, float* smem, uint32_t* wb) {
+                                                float* __restrict__ yU, unsigned long long* __restrict__ packedL,
+                                                unsigned long long* __restrict__ packedU, float* smem, uint32_t* wb) {
     constexpr int TR = 8;
     constexpr int WROW = 2 * 64 + 4;      // floats per input in the weight tile: 64 lanes x (w, w')
     constexpr int XROW = 2 * kTileB + 4;  // floats per input in the l/u tile: 128 batch rows x (l, u)
@@ -714,8 +717,9 @@ __device__ __forceinline__ void bound_rows_body(const float* __restrict__ xl, co
     auto wt = [&](int buf) { return smem + buf * kTileFloats + kChunk * XROW; };
 
     float lo[TR][2], hi[TR][2];
+    uint32_t cw[TR];   // POS: chunk numbers of (lower, lower', upper, upper') of a batch row, one byte each, 255 = none
     #pragma unroll
-    for (int r = 0; r < TR; r++) { lo[r][0] = lo[r][1] = -kEps; hi[r][0] = hi[r][1] = kEps; }
+    for (int r = 0; r < TR; r++) { lo[r][0] = lo[r][1] = -kEps; hi[r][0] = hi[r][1] = kEps; cw[r] = 0xffffffffu; }
 
     // word of (chunk c, batch row b0 + i): bw[c * Bp + i]; rows past the batch, up to the padded count, hold zero
     const uint32_t* __restrict__ bw = bits + (size_t)t * NCH * Bp + b0;
@@ -757,10 +761,24 @@ __device__ __forceinline__ void bound_rows_body(const float* __restrict__ xl, co
                 const float2 ww = *reinterpret_cast<const float2*>(W + n * WROW);        // the lane's two weights
                 const float2 lu = *reinterpret_cast<const float2*>(X + n * XROW + 2 * r);   // l, u of the row
                 const float a1 = ww.x - lu.x, a2 = lu.y - ww.x, b1 = ww.y - lu.x, b2 = lu.y - ww.y;
-                lo[r][0] = fminf(fminf(lo[r][0], a1), a2);
-                hi[r][0] = fmaxf(fmaxf(hi[r][0], a1), a2);
-                lo[r][1] = fminf(fminf(lo[r][1], b1), b2);
-                hi[r][1] = fmaxf(fmaxf(hi[r][1], b1), b2);
+                if (POS) {
+                    const uint32_t kl4 = (uint32_t)(c - c_lo) * 0x01010101u;
+                    const float v0 = fminf(a1, a2), V0 = fmaxf(a1, a2), v1 = fminf(b1, b2), V1 = fmaxf(b1, b2);
+                    const bool w0 = v0 < lo[r][0], w1 = v1 < lo[r][1], w2 = V0 > hi[r][0], w3 = V1 > hi[r][1];
+                    lo[r][0] = w0 ? v0 : lo[r][0]; lo[r][1] = w1 ? v1 : lo[r][1];
+                    hi[r][0] = w2 ? V0 : hi[r][0]; hi[r][1] = w3 ? V1 : hi[r][1];
+                    uint32_t c4 = cw[r];
+                    c4 = w0 ? ((c4 & 0xffffff00u) | (kl4 & 0x000000ffu)) : c4;
+                    c4 = w1 ? ((c4 & 0xffff00ffu) | (kl4 & 0x0000ff00u)) : c4;
+                    c4 = w2 ? ((c4 & 0xff00ffffu) | (kl4 & 0x00ff0000u)) : c4;
+                    c4 = w3 ? ((c4 & 0x00ffffffu) | (kl4 & 0xff000000u)) : c4;
+                    cw[r] = c4;
+                } else {
+                    lo[r][0] = fminf(fminf(lo[r][0], a1), a2);
+                    hi[r][0] = fmaxf(fmaxf(hi[r][0], a1), a2);
+                    lo[r][1] = fminf(fminf(lo[r][1], b1), b2);
+                    hi[r][1] = fmaxf(fmaxf(hi[r][1], b1), b2);
+                }
             }
         }
     };
@@ -801,6 +819,16 @@ __device__ __forceinline__ void bound_rows_body(const float* __restrict__ xl, co
             const int col = m0 + lane + 64 * j;
             if (row < B && col < M) {
                 const size_t o = (size_t)row * M + col;
+                if (POS) {
+                    const uint32_t kL = (cw[r] >> (8 * j)) & 0xffu, kU = (cw[r] >> (16 + 8 * j)) & 0xffu;
+                    if (kL != 0xffu)
+                        atomicMax(packedL + o, ((unsigned long long)__float_as_uint(-lo[r][j]) << 32) |
+                                                   (unsigned long long)(0xffffffffu - (uint32_t)(c_lo + (int)kL)));
+                    if (kU != 0xffu)
+                        atomicMax(packedU + o, ((unsigned long long)__float_as_uint(hi[r][j]) << 32) |
+                                                   (unsigned long long)(0xffffffffu - (uint32_t)(c_lo + (int)kU)));
+                    continue;
+                }
                 // both results are >= 1e-10 > 0, so their bit patterns order like integers
                 if (nsplit > 1) {
                     atomicMax(reinterpret_cast<int*>(yL + o), __float_as_int(-lo[r][j]));
@@ -823,9 +851,9 @@ bound_table_kernel(const float* __restrict__ xl, const float* __restrict__ xu, c
     __shared__ __attribute__((aligned(16))) float lds[kLdsWords];
     if (count[0] <= limit_col)
         bound_cols_body<POS>(xT, w, bits, order, B, M, Mp, N, nsplit, yL, yU, packedL, packedU, lds);
-    else if (!POS && count[1] <= limit_row)   // positions are only tracked with the tables per weight row
-        bound_rows_body(xl, xu, w, bits, B, Bp, M, N, nsplit, yL, yU, lds,
-                        reinterpret_cast<uint32_t*>(lds + 2 * kMainTileFloats));
+    else if (count[1] <= limit_row)
+        bound_rows_body<POS>(xl, xu, w, bits, B, Bp, M, N, nsplit, yL, yU, packedL, packedU, lds,
+                             reinterpret_cast<uint32_t*>(lds + 2 * kMainTileFloats));
 }
 
 }  // namespace
@@ -840,7 +868,6 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
                        float density_rows, const unsigned long long** gate, unsigned long long* gate_limit,
                        hipStream_t st) {
     const bool with_pos = packedL != nullptr;
-    if (with_pos) density_rows = 0.f;   // the kernel of the tables per batch row tracks no positions
     if (CI % kChunk != 0 || B < 1 || CO < 1) { set_error("bound_cols_forward: shape not supported"); return SD_ERR_ARG; }
     const Carve c = carve(ws, B, CO, CI);
     const int S = tiles_b(B), Mp = mpad_of(CO), Bp = bpad_of(B), T = Mp / kTileW, NCH = CI / kChunk;
@@ -885,8 +912,8 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
         if (n == 1 || cost < best) { best = cost; nsplit = n; }
     }
     if (with_pos) {
-        // chunk numbers within a slice take 8 bits (255 = none)
-        while ((((NCH + 1) / 2 + nsplit - 1) / nsplit) * 2 > 254) nsplit++;
+        // chunk numbers within a slice take 8 bits (255 = none), in either orientation
+        while ((((NCH + 1) / 2 + nsplit - 1) / nsplit) * 2 > 254 || (NCH + nsplit - 1) / nsplit > 254) nsplit++;
         hipLaunchKernelGGL(bound_table_kernel<true>, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.xt,
                            c.bits, c.order, c.count, limit_col, limit_row, B, Bp, CO, Mp, CI, nsplit, outL, outU, packedL,
                            packedU);

@@ -385,7 +385,7 @@ extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* input
     static const int kTb42[] = {4, 2};
     const int TB = pick_tb(a, kTb42, 2, 64);
     a.nsplit = pick_nsplit(a, 16 * TB, 64);
-    // dense single-group layers: the table kernel per weight row, tracking the chunk of every result, is queued in front
+    // dense single-group layers: the table kernel, tracking the chunk of every result, is queued in front
     // of the every-term kernel as for the forward without positions; both leave (value, chunk) pairs for the resolve
     const float cap = g_bound_density >= 0.f ? g_bound_density : kBoundPosColsCap;
     bool cols = cap > 0.f && G == 1 && HW == 1 && CI % kColsChunk == 0 && a.fast_x && a.fast_w &&
@@ -403,7 +403,7 @@ extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* input
         if ((rc = fill_zero(a.packed0, n * 4, st))) return rc;
         if (cols) {
             if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, nullptr, nullptr, a.packed0, a.packed1,
-                                         ws + pairs, cap, 0.f, &a.gate, &a.gate_limit, st)))
+                                         ws + pairs, cap, cap, &a.gate, &a.gate_limit, st)))
                 return rc;
             a.gate_above = 1;
         }
