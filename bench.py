@@ -59,6 +59,10 @@ def parse():
                          "the reference initialises with 1.0)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the short runs of the other formulations")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="queue the certification pass behind the optimizer on the one stream instead of on a second "
+                         "stream beside forward and backward (per-kernel durations in a profiler trace are then those "
+                         "of kernels that have the device to themselves)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain device copy of a width x width fp32 matrix after the timed steps "
                          "(a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE counters with)")
@@ -173,12 +177,13 @@ def run_index_lists(args, q, p, steps, warmup, certify_runs=0):
 
 
 def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width=None, classes=None, eps=None,
-               time_ibp=False, calib_copy=False, weight_std=None):
+               time_ibp=False, calib_copy=False, weight_std=None, overlap=None):
     """K timed steps of the fused-mask formulation; returns timings, phase split and the per-launch events of the
     interval-bound forward of the width x width layers."""
     import torch
     from sortnet_amd import ext, _lib
     from sortnet_amd.model import DistanceMLP, margins, hinge_loss
+    overlap = (not args.no_overlap) if overlap is None else overlap
     batch = batch or args.batch
     in_features = in_features or args.in_features
     width = width or args.width
@@ -203,21 +208,17 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     dense_ms = []                # every-term interval kernel, per launch
     fwd_ms, fwd_kernel = [], [None]   # masked l-inf forward tile kernel, per launch
 
-    def step(i, timed, after_layer=None):
-        marks = [ev() for _ in range(5)]
-        marks[0].record()
-        dist = model.forward(x, step_seed=i, after_layer=after_layer)
-        logits, worst = margins(dist, targets, eps)
-        loss = hinge_loss(worst)
-        marks[1].record()
-        opt.zero_grad(set_to_none=True)
-        loss.backward()
-        marks[2].record()
-        opt.step()
-        marks[3].record()
+    # The certification pass needs the weights and nothing of the training step, so it is queued on a second stream
+    # (default priority) beside forward and backward, on the weights the forward uses and a snapshot of the running
+    # means; the optimizer waits for it before it changes the weights.  Its small kernels (tables, fills, shifts) and
+    # the partly filled last rounds of workgroups of either stream then fill each other's gaps.
+    main = torch.cuda.current_stream(dev)
+    side = torch.cuda.Stream(device=dev) if overlap else None
+
+    def certification(timed, means):
         if timed and time_ibp:
-            # same certification pass, spelled out to time every launch of the dominant kernel (the interval-bound
-            # forward of a width x width layer) with events on the stream it is queued on (torch's current stream)
+            # the pass spelled out, to time every call of the interval forward of a width x width layer with events on
+            # the stream it is queued on (torch's current stream)
             lo, up = lower.unsqueeze(-1).contiguous(), upper.unsqueeze(-1).contiguous()
             with torch.no_grad():
                 for li, w in enumerate(model.weights):
@@ -230,13 +231,40 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
                     if w.size(0) == width and w.size(1) == width:
                         ibp_events.append((e0, e1))
                         probe[:] = [lo, up, w]
-                    shift = (model.running_mean[li].view(1, -1, 1) if li < model.num_layers - 1
-                             else -model.bias.view(1, -1, 1))
+                    shift = (means[li].view(1, -1, 1) if li < model.num_layers - 1 else -model.bias.view(1, -1, 1))
                     lo, up = ylo - shift, yup - shift
-                cert = margins(dist.detach(), targets, eps, lo.squeeze(-1), up.squeeze(-1))[1]
-        else:
-            lo, up = model.bounds(lower, upper)
-            cert = margins(dist.detach(), targets, eps, lo, up)[1]
+            return lo.squeeze(-1), up.squeeze(-1)
+        return model.bounds(lower, upper, means=means)
+
+    def step(i, timed, after_layer=None, concurrent=None):
+        concurrent = overlap if concurrent is None else concurrent
+        marks = [ev() for _ in range(7)]
+        marks[0].record()
+        if concurrent:
+            means = [m.clone() for m in model.running_mean]
+            side.wait_stream(main)                       # the previous step's optimizer is done with the weights
+            with torch.cuda.stream(side):
+                marks[5].record()
+                lo, up = certification(timed, means)
+                marks[6].record()
+        dist = model.forward(x, step_seed=i, after_layer=after_layer)
+        logits, worst = margins(dist, targets, eps)
+        loss = hinge_loss(worst)
+        marks[1].record()
+        opt.zero_grad(set_to_none=True)
+        loss.backward()
+        marks[2].record()
+        if concurrent:
+            main.wait_stream(side)                       # the certification pass has read the weights
+            lo.record_stream(main)
+            up.record_stream(main)
+        opt.step()
+        marks[3].record()
+        if not concurrent:
+            marks[5].record()
+            lo, up = certification(timed, model.running_mean)
+            marks[6].record()
+        cert = margins(dist.detach(), targets, eps, lo, up)[1]
         marks[4].record()
         return marks, loss, cert
 
@@ -246,10 +274,30 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     t0 = time.perf_counter()
     all_marks = []
     for i in range(steps):
-        marks, loss, cert = step(warmup + i, True)
+        marks, loss, cert = step(warmup + i, False)
         all_marks.append(marks)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+
+    if time_ibp:
+        # A few more steps on one stream, not part of `value`, for the figures about single kernels and calls: the
+        # interval forward of every width x width layer between two events (roofline's in_step), and - the kernel with
+        # the largest share of the step - the masked l-inf forward with chunk tracking of those layers by the library's
+        # events around the tile kernel's launch, read back after every such layer (which makes the host wait).
+        def read_timer(i, w):
+            if i > 0 and tuple(w.shape) == (width, width):
+                ms = _lib.last_forward_kernel_ms()
+                if ms is not None:
+                    fwd_ms.append(ms)
+                    fwd_kernel[0] = _lib.last_forward_kernel()
+
+        _lib.time_forward_kernels(True)
+        try:
+            for k in range(max(4, steps // 4)):
+                step(warmup + steps + k, True, after_layer=read_timer, concurrent=False)
+        finally:
+            _lib.time_forward_kernels(False)
+        torch.cuda.synchronize()
 
     if time_ibp and probe:
         # The interval forward picks, on the device, between a kernel that evaluates only the inputs a table marks
@@ -274,25 +322,6 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
             _lib.time_forward_kernels(False)
         torch.cuda.synchronize()
 
-    if time_ibp and q < 1.0:
-        # The kernel with the largest share of the step: the masked l-inf forward with chunk tracking of a
-        # width x width layer.  A few more steps, with the library's events around the tile kernel's launch switched
-        # on and read back after every such layer (which makes the host wait: these steps are not part of `value`).
-        def read_timer(i, w):
-            if i > 0 and tuple(w.shape) == (width, width):
-                ms = _lib.last_forward_kernel_ms()
-                if ms is not None:
-                    fwd_ms.append(ms)
-                    fwd_kernel[0] = _lib.last_forward_kernel()
-
-        _lib.time_forward_kernels(True)
-        try:
-            for k in range(max(4, steps // 4)):
-                step(warmup + steps + k, False, after_layer=read_timer)
-        finally:
-            _lib.time_forward_kernels(False)
-        torch.cuda.synchronize()
-
     if calib_copy:
         src = model.weights[1]
         dst = torch.empty_like(src)
@@ -300,8 +329,10 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
         torch.cuda.synchronize()
 
     for marks in all_marks:
-        for k, (a, b) in zip(phase_ms, zip(marks[:-1], marks[1:])):
-            phase_ms[k] += a.elapsed_time(b) / steps
+        phase_ms["forward"] += marks[0].elapsed_time(marks[1]) / steps
+        phase_ms["backward"] += marks[1].elapsed_time(marks[2]) / steps
+        phase_ms["optimizer"] += marks[2].elapsed_time(marks[3]) / steps   # with `overlap`: and the wait for the second stream
+        phase_ms["bounds"] += marks[5].elapsed_time(marks[6]) / steps      # on its own stream with `overlap`
     res = {
         "ms_per_step": elapsed * 1e3 / steps, "samples_per_s": batch / (elapsed / steps), "steps": steps,
         "phase_ms": phase_ms, "terms_per_step": model.terms_per_sample() * batch,
@@ -441,7 +472,8 @@ def main():
         "in_step": {
             "avg_call_ms": step_ms if launches else None, "calls_timed": len(launches),
             "algorithmic_tflops": 6.0 * layer_terms / (step_ms * 1e-3) / 1e12 if launches else None,
-            "note": "the same entry point as the timed steps call it on their width x width layers: a table of the "
+            "note": "the same entry point as the steps call it on their width x width layers (timed in a few further "
+                    "steps that queue everything on one stream): a table of the "
                     "inputs that can hold a maximum (per weight row and tile of 128 batch rows) is built first and a "
                     "count taken on the device picks the table kernel or the every-term kernel; terms that cannot "
                     "hold a maximum are never formed, so this rate is not bounded by the vector peak",
@@ -452,13 +484,15 @@ def main():
                 "(in_step), so these launches are queued after the steps, on the operands of their last width x width "
                 "layer with the table switched off",
     }
-    if fwd:
+    if fwd and args.q < 1.0:
         achieved = 2.0 * layer_terms / (fwd_ms * 1e-3) / 1e12
         roofline = {
             "bound": "valu",
-            "kernel": "sd::%s, policy %s (l-inf forward under the %s mask with the winning chunk tracked for the "
-                      "positions, every term, %dx%dx%d)" % (head["fwd_kernel"], "LinfChunkPacked" if factored else "MaskedTermChunk",
-                                                            args.mask, args.batch, args.width, args.width),
+            "kernel": "sd::%s, policy %s (l-inf forward %s with the winning chunk tracked for the positions, every "
+                      "term, %dx%dx%d)" % (head["fwd_kernel"],
+                                           "LinfChunkPacked" if factored else "MaskedTermChunk",
+                                           "under the %s mask" % args.mask,
+                                           args.batch, args.width, args.width),
             "achieved": achieved, "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": achieved / FP32_VECTOR_PEAK_TFLOPS,
             "traffic": committed_traffic("traffic_bytes_per_launch_masked_forward") if at_size and factored else None,
@@ -472,10 +506,11 @@ def main():
                      "the kernel with the largest share of the step; 2 flops per term, and the keep decision of every "
                      "term comes from a counter hash that costs more than the term; ") +
                     "timed by events around the kernel's own launch (sd_time_forward_kernels) in a few further steps "
-                    "after the timed ones, every width x width layer",
+                    "after the timed ones, every width x width layer; those steps queue everything on one stream, so "
+                    "that the kernel has the device to itself as in a profiler trace of --no-overlap",
             "interval_every_term": interval,
         }
-    else:   # q = 1: no masked layers; the interval kernel is the one to report
+    else:   # q = 1: no masked layers (and most l-inf layers are served from candidate tables); the interval kernel is the one to report
         roofline = dict(interval, bound="valu", peak=FP32_VECTOR_PEAK_TFLOPS)
     out = {
         "metric": "train samples/s (fwd+bwd+IBP) 5x5120 SortNet-MLP, B=512; % FP32 VALU peak",
@@ -483,9 +518,14 @@ def main():
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": workload_text(args, args.mask, args.q),
-                   "batch": args.batch, "width": args.width, "distance_layers": args.depth, "mask": args.mask},
+                   "batch": args.batch, "width": args.width, "distance_layers": args.depth, "mask": args.mask,
+                   "streams": 1 if args.no_overlap else 2},
         "step_fp32_vector_frac": step_flops / step_s / (FP32_VECTOR_PEAK_TFLOPS * 1e12),
         "phase_ms": head["phase_ms"],
+        "phase_note": ("the certification pass (bounds) is queued on a second stream beside forward and backward, on "
+                       "the weights the forward uses, and the optimizer waits for it: the phases overlap and do not add "
+                       "up to ms_per_step; forward and backward are longer than alone because they share the device"
+                       if not args.no_overlap else "one stream: forward, backward, optimizer, certification pass in turn"),
         "roofline": roofline,
         "loss": head["loss"], "certified_frac": head["certified_frac"],
     }

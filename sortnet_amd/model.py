@@ -71,12 +71,14 @@ class DistanceMLP:
         return h.squeeze(-1)
 
     @torch.no_grad()
-    def bounds(self, lower, upper):
-        """Certification pass: interval bounds of the distances for inputs in [lower, upper]."""
+    def bounds(self, lower, upper, means=None):
+        """Certification pass: interval bounds of the distances for inputs in [lower, upper].  `means` replaces the
+        running means (a snapshot, for a caller that runs this pass beside a training forward that updates them)."""
+        means = self.running_mean if means is None else means
         lo, up = lower.unsqueeze(-1).contiguous(), upper.unsqueeze(-1).contiguous()
         for i, w in enumerate(self.weights):
             lo, up = F.bound_inf_dist(lo, up, w)
-            shift = self.running_mean[i].view(1, -1, 1) if i < self.num_layers - 1 else -self.bias.view(1, -1, 1)
+            shift = means[i].view(1, -1, 1) if i < self.num_layers - 1 else -self.bias.view(1, -1, 1)
             lo, up = lo - shift, up - shift
         return lo.squeeze(-1), up.squeeze(-1)
 
