@@ -272,12 +272,16 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
         step(i, False)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    all_marks = []
+    all_marks, trace = [], []
     for i in range(steps):
         marks, loss, cert = step(warmup + i, False)
         all_marks.append(marks)
+        trace.append((loss.detach(), cert))      # read after the timed region
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    loss_trace = [float(l) for l, _ in trace]
+    margin_trace = [float(c.double().sum()) for _, c in trace]
+    del trace
 
     if time_ibp:
         # A few more steps on one stream, not part of `value`, for the figures about single kernels and calls: the
@@ -339,6 +343,8 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
         "ibp_launch_ms": [a.elapsed_time(b) for a, b in ibp_events], "ibp_kernel": ibp_kernel[0],
         "ibp_every_term_ms": dense_ms, "fwd_kernel_ms": fwd_ms, "fwd_kernel": fwd_kernel[0],
         "loss": float(loss.detach()), "certified_frac": float((cert.max(dim=1)[0] < 0).float().mean()),
+        # per timed step: the training loss, and the sum of the certification pass's worst-case margins
+        "loss_trace": loss_trace, "margin_trace": margin_trace,
     }
     del model, opt
     torch.cuda.empty_cache()
