@@ -60,9 +60,10 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the short runs of the other formulations")
     ap.add_argument("--no-overlap", action="store_true",
-                    help="queue the certification pass behind the optimizer on the one stream instead of on a second "
-                         "stream beside forward and backward (per-kernel durations in a profiler trace are then those "
-                         "of kernels that have the device to themselves)")
+                    help="queue forward, backward, optimizer and certification pass in turn on the one stream, instead of "
+                         "the certification pass on a second stream beside forward and backward and the optimizer's "
+                         "steps layer by layer on a third (per-kernel durations in a profiler trace are then those of "
+                         "kernels that have the device to themselves)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain device copy of a width x width fp32 matrix after the timed steps "
                          "(a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE counters with)")
@@ -176,14 +177,28 @@ def run_index_lists(args, q, p, steps, warmup, certify_runs=0):
     return out
 
 
+_EXTRA_STREAMS = {}
+
+
+def extra_streams(dev):
+    """The two streams (default priority) beside torch's current one that the overlapped step uses, made once per
+    process: the runtime deals streams to a few hardware queues in the order they are made, and two streams that
+    share a queue do not overlap, so every run of the step uses the same two."""
+    import torch
+    if dev not in _EXTRA_STREAMS:
+        _EXTRA_STREAMS[dev] = (torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev))
+    return _EXTRA_STREAMS[dev]
+
+
 def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width=None, classes=None, eps=None,
-               time_ibp=False, calib_copy=False, weight_std=None, overlap=None):
+               time_ibp=False, calib_copy=False, weight_std=None, overlap=None, pipeline=None, stages=None):
     """K timed steps of the fused-mask formulation; returns timings, phase split and the per-launch events of the
     interval-bound forward of the width x width layers."""
     import torch
     from sortnet_amd import ext, _lib
     from sortnet_amd.model import DistanceMLP, margins, hinge_loss
     overlap = (not args.no_overlap) if overlap is None else overlap
+    pipeline = overlap if pipeline is None else (pipeline and overlap)
     batch = batch or args.batch
     in_features = in_features or args.in_features
     width = width or args.width
@@ -194,7 +209,16 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     mode = ext.MASK_TERM if mask == "term" else ext.MASK_FACTORED
     model = DistanceMLP(in_features, width, args.depth, classes, q=q, device=dev, seed=0, mask_mode=mode,
                         weight_std=weight_std)
-    opt = torch.optim.AdamW(model.parameters(), lr=1e-4, fused=True)
+    # AdamW couples no two parameters, so one optimizer per layer (the class layer's with the bias) takes the same
+    # steps as one over all of them; with `pipeline` they are queued layer by layer on a stream of their own
+    if pipeline:
+        # three steps: the first layer's, the second layer's, and the rest in one (measured: the next step's first
+        # two layers are enough to hide the rest's update, and fewer optimizer calls cost the host less)
+        stages = stages or [st for st in ([0], [1], list(range(2, model.num_layers))) if st and st[0] < model.num_layers]
+        groups = [[model.weights[i] for i in st] + ([model.bias] if model.num_layers - 1 in st else []) for st in stages]
+    else:
+        groups = [model.parameters()]
+    opts = [torch.optim.AdamW(g, lr=1e-4, fused=True) for g in groups]
     g = torch.Generator().manual_seed(0)
     x = torch.rand(batch, in_features, generator=g).to(dev)
     targets = torch.randint(0, classes, (batch,), generator=g).to(dev)
@@ -212,10 +236,22 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     # (default priority) beside forward and backward, on the weights the forward uses and a snapshot of the running
     # means; the optimizer waits for it before it changes the weights.  Its small kernels (tables, fills, shifts) and
     # the partly filled last rounds of workgroups of either stream then fill each other's gaps.
+    #
+    # With `pipeline` the optimizer's steps, layer by layer on a third stream, wait for the backward and for the
+    # certification pass and each leaves an event; the next step's forward and certification pass wait for layer i's
+    # event right before they read layer i's weights.  The update of the later layers, a stream of reads and writes to HBM,
+    # then runs beside the next step's first layers, which are bound by the vector units.
     main = torch.cuda.current_stream(dev)
-    side = torch.cuda.Stream(device=dev) if overlap else None
+    side, upd_stream = extra_streams(dev) if overlap else (None, None)
+    updated = [None] * model.num_layers          # per layer: the event after its last queued update
 
-    def certification(timed, means):
+    def wait_updated(stream):
+        def hook(i):
+            if updated[i] is not None:
+                stream.wait_event(updated[i])
+        return hook
+
+    def certification(timed, means, before_layer=None):
         if timed and time_ibp:
             # the pass spelled out, to time every call of the interval forward of a width x width layer with events on
             # the stream it is queued on (torch's current stream)
@@ -234,32 +270,53 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
                     shift = (means[li].view(1, -1, 1) if li < model.num_layers - 1 else -model.bias.view(1, -1, 1))
                     lo, up = ylo - shift, yup - shift
             return lo.squeeze(-1), up.squeeze(-1)
-        return model.bounds(lower, upper, means=means)
+        return model.bounds(lower, upper, means=means, before_layer=before_layer)
 
     def step(i, timed, after_layer=None, concurrent=None):
         concurrent = overlap if concurrent is None else concurrent
+        piped = pipeline and concurrent
+        if pipeline and not piped:
+            main.wait_stream(upd_stream)                 # a step on one stream after pipelined ones
+            updated[:] = [None] * len(updated)
         marks = [ev() for _ in range(7)]
         marks[0].record()
         if concurrent:
             means = [m.clone() for m in model.running_mean]
-            side.wait_stream(main)                       # the previous step's optimizer is done with the weights
+            side.wait_stream(main)                       # the snapshot; without `pipeline` also the previous step's optimizer
             with torch.cuda.stream(side):
                 marks[5].record()
-                lo, up = certification(timed, means)
+                lo, up = certification(timed, means, wait_updated(side) if piped else None)
                 marks[6].record()
-        dist = model.forward(x, step_seed=i, after_layer=after_layer)
+        dist = model.forward(x, step_seed=i, after_layer=after_layer,
+                             before_layer=wait_updated(main) if piped else None)
         logits, worst = margins(dist, targets, eps)
         loss = hinge_loss(worst)
         marks[1].record()
-        opt.zero_grad(set_to_none=True)
+        # (with `pipeline` the forward has waited for every layer's update by now, so the optimizer is done with the
+        # gradients that are freed here)
+        for opt in opts:
+            opt.zero_grad(set_to_none=True)
         loss.backward()
         marks[2].record()
+        if piped:
+            upd_stream.wait_stream(main)                 # the gradients
+            upd_stream.wait_stream(side)                 # the certification pass has read the weights
+            with torch.cuda.stream(upd_stream):
+                for st, opt in zip(stages, opts):
+                    opt.step()
+                    e = torch.cuda.Event()
+                    e.record()
+                    for li in st:
+                        updated[li] = e
+                marks[3].record()
         if concurrent:
             main.wait_stream(side)                       # the certification pass has read the weights
             lo.record_stream(main)
             up.record_stream(main)
-        opt.step()
-        marks[3].record()
+        if not piped:
+            for opt in opts:
+                opt.step()
+            marks[3].record()
         if not concurrent:
             marks[5].record()
             lo, up = certification(timed, model.running_mean)
@@ -277,6 +334,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
         marks, loss, cert = step(warmup + i, False)
         all_marks.append(marks)
         trace.append((loss.detach(), cert))      # read after the timed region
+    queued = time.perf_counter() - t0
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     loss_trace = [float(l) for l, _ in trace]
@@ -335,10 +393,11 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     for marks in all_marks:
         phase_ms["forward"] += marks[0].elapsed_time(marks[1]) / steps
         phase_ms["backward"] += marks[1].elapsed_time(marks[2]) / steps
-        phase_ms["optimizer"] += marks[2].elapsed_time(marks[3]) / steps   # with `overlap`: and the wait for the second stream
+        phase_ms["optimizer"] += marks[2].elapsed_time(marks[3]) / steps   # with `pipeline`: on its own stream, beside the next step
         phase_ms["bounds"] += marks[5].elapsed_time(marks[6]) / steps      # on its own stream with `overlap`
     res = {
         "ms_per_step": elapsed * 1e3 / steps, "samples_per_s": batch / (elapsed / steps), "steps": steps,
+        "host_ms_per_step": queued * 1e3 / steps,      # the host's time to queue a step
         "phase_ms": phase_ms, "terms_per_step": model.terms_per_sample() * batch,
         "ibp_launch_ms": [a.elapsed_time(b) for a, b in ibp_events], "ibp_kernel": ibp_kernel[0],
         "ibp_every_term_ms": dense_ms, "fwd_kernel_ms": fwd_ms, "fwd_kernel": fwd_kernel[0],
@@ -346,7 +405,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
         # per timed step: the training loss, and the sum of the certification pass's worst-case margins
         "loss_trace": loss_trace, "margin_trace": margin_trace,
     }
-    del model, opt
+    del model, opts
     torch.cuda.empty_cache()
     return res
 
@@ -525,12 +584,14 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": workload_text(args, args.mask, args.q),
                    "batch": args.batch, "width": args.width, "distance_layers": args.depth, "mask": args.mask,
-                   "streams": 1 if args.no_overlap else 2},
+                   "streams": 1 if args.no_overlap else 3},
         "step_fp32_vector_frac": step_flops / step_s / (FP32_VECTOR_PEAK_TFLOPS * 1e12),
         "phase_ms": head["phase_ms"],
         "phase_note": ("the certification pass (bounds) is queued on a second stream beside forward and backward, on "
-                       "the weights the forward uses, and the optimizer waits for it: the phases overlap and do not add "
-                       "up to ms_per_step; forward and backward are longer than alone because they share the device"
+                       "the weights the forward uses; the optimizer, layer by layer on a third stream, waits for both, "
+                       "and the next step's forward and certification pass wait for a layer's update right before they "
+                       "read that layer's weights: the phases overlap and do not add up to ms_per_step, and each is "
+                       "longer than alone because they share the device"
                        if not args.no_overlap else "one stream: forward, backward, optimizer, certification pass in turn"),
         "roofline": roofline,
         "loss": head["loss"], "certified_frac": head["certified_frac"],

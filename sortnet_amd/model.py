@@ -37,12 +37,15 @@ class DistanceMLP:
     def terms_per_sample(self):
         return sum(w.numel() for w in self.weights)
 
-    def forward(self, x, step_seed, trace=None, after_layer=None):
+    def forward(self, x, step_seed, trace=None, after_layer=None, before_layer=None):
         """Training forward: x (B, in_features) -> distances to the class prototypes (B, classes).
         `trace`, a list, receives per layer (input, raw distances, batch mean or None) for inspection;
-        `after_layer(i, weight)` is called right after layer i's distance op has been queued."""
+        `before_layer(i)` is called before anything that reads layer i's weight (or, on the last layer, the bias) is
+        queued, `after_layer(i, weight)` right after layer i's distance op has been queued."""
         h = x.unsqueeze(-1)
         for i, w in enumerate(self.weights):
+            if before_layer is not None:
+                before_layer(i)
             h_in = h
             if i == 0 or self.q is None or self.q == 1.0:
                 h = F.norm_dist(h, w, float("inf"))
@@ -71,12 +74,15 @@ class DistanceMLP:
         return h.squeeze(-1)
 
     @torch.no_grad()
-    def bounds(self, lower, upper, means=None):
+    def bounds(self, lower, upper, means=None, before_layer=None):
         """Certification pass: interval bounds of the distances for inputs in [lower, upper].  `means` replaces the
-        running means (a snapshot, for a caller that runs this pass beside a training forward that updates them)."""
+        running means (a snapshot, for a caller that runs this pass beside a training forward that updates them);
+        `before_layer(i)` as in `forward`."""
         means = self.running_mean if means is None else means
         lo, up = lower.unsqueeze(-1).contiguous(), upper.unsqueeze(-1).contiguous()
         for i, w in enumerate(self.weights):
+            if before_layer is not None:
+                before_layer(i)
             lo, up = F.bound_inf_dist(lo, up, w)
             shift = means[i].view(1, -1, 1) if i < self.num_layers - 1 else -self.bias.view(1, -1, 1)
             lo, up = lo - shift, up - shift

@@ -195,11 +195,12 @@ def test_benchmark_size_stack(oracle):
     assert np.array_equal(y_lo[:rows].cpu().numpy(), rl) and np.array_equal(y_up[:rows].cpu().numpy(), ru)
 
 
-def test_two_stream_step_matches_one_stream_step(monkeypatch):
-    """bench.py's default step queues the certification pass on a second stream beside forward and backward; with
-    --no-overlap it follows the optimizer on the one stream.  Both train the same weights: the loss of every step
-    agrees.  The two-stream pass of step i + 1 reads the weights and running means that the one-stream pass of step i
-    reads (those left by step i's optimizer and forward), so its margins agree with that pass's."""
+def test_overlapped_steps_match_one_stream_step(monkeypatch):
+    """bench.py's default step queues the certification pass on a second stream beside forward and backward and the
+    optimizer layer by layer on a third, each reader of a layer's weights waiting for that layer's update; with
+    --no-overlap everything follows in turn on one stream.  All train the same weights: the loss of every step agrees.
+    An overlapped certification pass of step i + 1 reads the weights and running means that the one-stream pass of
+    step i reads (those left by step i's optimizer and forward), so its margins agree with that pass's."""
     import os
     import sys
     _dev()
@@ -209,10 +210,11 @@ def test_two_stream_step_matches_one_stream_step(monkeypatch):
     args = bench.parse()
     args.batch, args.in_features, args.width, args.depth, args.classes = 256, 784, 1024, 4, 10
     steps, warmup = 6, 2
-    two = bench.run_masked(args, "factored", 0.3, steps, warmup, overlap=True)
     one = bench.run_masked(args, "factored", 0.3, steps, warmup, overlap=False)
-    np.testing.assert_allclose(two["loss_trace"], one["loss_trace"], rtol=1e-4)
-    np.testing.assert_allclose(two["margin_trace"][1:], one["margin_trace"][:-1], rtol=1e-4)
-    # a step moves the margins by well more than the tolerance: the comparison above tells neighbouring steps apart
+    # a step moves the margins by well more than the tolerance: the comparison below tells neighbouring steps apart
     m = np.asarray(one["margin_trace"])
     assert np.abs(np.diff(m)).min() > 5e-4 * np.abs(m).max()
+    for pipeline in (True, False):
+        two = bench.run_masked(args, "factored", 0.3, steps, warmup, overlap=True, pipeline=pipeline)
+        np.testing.assert_allclose(two["loss_trace"], one["loss_trace"], rtol=1e-4, err_msg=str(pipeline))
+        np.testing.assert_allclose(two["margin_trace"][1:], one["margin_trace"][:-1], rtol=1e-4, err_msg=str(pipeline))
