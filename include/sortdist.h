@@ -30,7 +30,12 @@
  * (split reductions, mask bits, candidate lists, per-slice sums) and grows it on demand with
  * hipMalloc; growing waits for that stream first.  Calls are asynchronous on `stream`; calls
  * on different streams never share a buffer and may overlap, calls on one stream use it in
- * queue order.  A call that would have to grow the buffer while its stream is being captured
+ * queue order.  Host threads: every entry point may be called from any thread at any time; while
+ * a call queues its kernels it holds a library-wide lock, so the calls of several threads reach
+ * a shared stream whole, one after the other, and each gets the results it would get alone.
+ * The sd_set_* limits are process-wide atomics that a call reads once when it starts; per-layer
+ * table hints (which of two queued kernels has been running lately) are kept for the 256 most
+ * recently used (entry point, weight pointer, shape) triples and never change a result.  A call that would have to grow the buffer while its stream is being captured
  * into a graph fails with SD_ERR_HIP: run it once on that stream before the capture.
  * Outputs that are zero-filled or merged with 128-bit stores must be 16-byte aligned.
  */
@@ -162,7 +167,13 @@ int sd_bound_inf_dist_backward_input_weight(const float* grad_outputL, const flo
                                             float* grad_inputL, float* grad_inputU, float* grad_weight,
                                             sd_stream_t stream);
 
-/* ---- sort neuron: struct sort_neuron, norm_dist.h:47-57; K in 2..25 ---- */
+/* ---- sort neuron: struct sort_neuron, norm_dist.h:47-57; K in 2..25 ----
+ * Undefined (NaN) terms: a term |input - weight| that is NaN is LEFT OUT of the K largest here (values, positions and
+ * interval form alike), whichever kernel serves the call.  The reference's insertion max(res[k], min(res[k+1], v))
+ * (core/cuda/sort_neuron.cu:73-77, 283-287) instead shifts its list down by one on such a term, i.e. counts the
+ * largest entry so far twice; that behaviour depends on the order in which the inputs are scanned and is not
+ * reproduced.  Finite inputs, +-inf included, give the reference's results.  (The l-inf and interval-bound entry points
+ * drop NaN terms exactly as the reference's strict comparisons and fminf / fmaxf do.) */
 
 /* sort_neuron::forward_nograd (norm_dist.h:48-49; core/cuda/sort_neuron.cu:387-434). */
 int sd_sort_neuron_forward_nograd(const float* input, const float* weight,

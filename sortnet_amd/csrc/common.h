@@ -90,6 +90,17 @@ int num_cus();
 // Growing waits for that stream and re-allocates (bytes == 0 returns the current buffer).
 void* workspace(size_t bytes, hipStream_t stream);
 
+// Held by an entry point while it queues its kernels.  The calls of several host threads then reach their streams
+// one after the other, whole, so that a stream's workspace is used in call order even when threads share the stream
+// (as they do by default); only the queueing is serialised, the work of different streams still overlaps.
+class CallGuard {
+public:
+    CallGuard();
+    ~CallGuard();
+    CallGuard(const CallGuard&) = delete;
+    CallGuard& operator=(const CallGuard&) = delete;
+};
+
 // Whether a call site's candidate tables have paid lately.  Calls that queue a table kernel and an every-term kernel
 // for one result let the device choose, and report afterwards which ran (hint_record: an 8-byte copy of the device's
 // flag into pinned host memory, read by a later call once its event has completed; nothing waits).  When the every-term

@@ -36,7 +36,7 @@ __device__ __forceinline__ void load_group_to_lds(const float* base, uint32_t vo
                         (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
     base = reinterpret_cast<const float*>(sb);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(lds), "v"(voff), "s"(base) : "memory");
+                 :: "s"(lds), "v"(voff), "s"(base) : "memory", "m0");
 }
 
 __device__ __forceinline__ uint32_t lds_address(const void* p) {

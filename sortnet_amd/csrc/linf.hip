@@ -3,6 +3,7 @@
 #include "fwd_args.h"
 #include "bound_cols.h"
 #include "sort_cols.h"
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 
@@ -10,7 +11,7 @@ using namespace sd;
 
 // largest share of marked (tile, weight row, input) triples at which the candidate-table kernel of the interval
 // forward runs instead of the kernel that evaluates every term (sd_set_bound_candidate_density); negative: built-in
-static float g_bound_density = -1.f;
+static std::atomic<float> g_bound_density{-1.f};
 // measured at B = 512, M = N = 5120: the table kernel takes 0.09 + 2.6 x share ms (about 60 SIMD cycles per marked
 // (tile, weight row, input)) after 0.10 ms for the tables, against 1.03-1.09 ms for every term; the kernel of the
 // tables per batch row 0.14 + 3.3 x share ms.  The tables are paid for by the time the choice is made, so the limits
@@ -26,30 +27,40 @@ constexpr long long kBoundColsMinTerms = 1ll << 31;
 constexpr float kBoundPosColsCap = 0.15f;
 constexpr int kHintSiteBound = 1, kHintSiteBoundSparse = 8, kHintSiteBoundPos = 9;
 constexpr float kBoundSparseCap = 0.03f;   // marked share up to which the kernel without LDS staging runs
-static int g_bound_form = 0;              // 0: chosen per layer, 1: staged tiles, 2: transposed-row walk
+static std::atomic<int> g_bound_form{0};            // 0: chosen per layer, 1: staged tiles, 2: transposed-row walk
 
 // The l-inf forward (plain, and under the factored mask) on dense single-group layers queues a kernel that works from
 // per-weight-row candidate tables in front of the kernels that evaluate every term; a count taken on the device
 // decides which runs.  Negative g_linf_density: built-in limit, layers of at least kMaxColsMinTerms terms, and not
 // where the tables have not paid lately (hint_build_tables); 0 never; up to 1: that share, at any size.
-static float g_linf_density = -1.f;
-static int g_linf_depth = 0;   // under the mask: inputs the bound of a weight row rests on (0 = from the keep probability)
+static std::atomic<float> g_linf_density{-1.f};
+static std::atomic<int> g_linf_depth{0};   // under the mask: inputs the bound of a weight row rests on (0 = from the keep probability)
 constexpr float kMaxColsCap = 0.10f;
 constexpr long long kMaxColsMinTerms = 1ll << 31;   // below, the tables cost more than evaluating every term
 constexpr int kHintSiteLinf = 4, kHintSiteMasked = 5;
 
-// depth of the tables' bound (0 = no tables for this call)
-static int max_cols_wanted(const FwdArgs& a, int site, float keep_x, int B, int CO, int CI, int G, int HW, hipStream_t st) {
-    if (g_linf_density == 0.f || G != 1 || HW != 1 || CI % kSortColsChunk != 0 || CI > 65536 || !a.fast_x || !a.fast_w ||
+// Depth of the tables' bound for this shape and mask (0 = the call is not served from tables), by shape and size
+// alone: the workspace is sized by this, so that a call under graph capture (which always builds tables) never needs
+// more than the eager call before it did.
+static int max_cols_eligible(const FwdArgs& a, float keep_x, int B, int CO, int CI, int G, int HW) {
+    const float density = g_linf_density.load(std::memory_order_relaxed);
+    const int depth = g_linf_depth.load(std::memory_order_relaxed);
+    if (density == 0.f || G != 1 || HW != 1 || CI % kSortColsChunk != 0 || CI > 65536 || !a.fast_x || !a.fast_w ||
         a.ci_idx || a.co_idx) return 0;
     int K = max_cols_depth(keep_x);
-    if (g_linf_depth > 0 && keep_x < 1.f) K = g_linf_depth;
-    if (K == 0 || g_linf_density > 0.f) return K;
-    return ((long long)B * CO * CI >= kMaxColsMinTerms && hint_build_tables(site, a.w, B, CO, CI, st)) ? K : 0;
+    if (depth > 0 && keep_x < 1.f) K = depth;
+    if (K == 0 || density > 0.f) return K;
+    return (long long)B * CO * CI >= kMaxColsMinTerms ? K : 0;
+}
+// eligible depth `K`, or 0 when (with the built-in limit) the layer's tables have not paid lately
+static int max_cols_wanted(const FwdArgs& a, int K, int site, int B, int CO, int CI, hipStream_t st) {
+    if (K == 0 || g_linf_density.load(std::memory_order_relaxed) > 0.f) return K;
+    return hint_build_tables(site, a.w, B, CO, CI, st) ? K : 0;
 }
 
 static int queue_max_cols(FwdArgs& a, int K, int B, int CO, int CI, void* ws, hipStream_t st) {
-    const float cap = g_linf_density > 0.f ? g_linf_density : kMaxColsCap;
+    const float density = g_linf_density.load(std::memory_order_relaxed);
+    const float cap = density > 0.f ? density : kMaxColsCap;
     // depth 1: the mask keeps everything
     int rc = max_cols_forward(a.x0, a.w, K == 1 ? nullptr : a.xmask, K == 1 ? nullptr : a.wmask, B, CO, CI, K, a.y0, a.p0,
                               ws, cap, &a.gate, &a.gate_limit, st);
@@ -58,7 +69,7 @@ static int queue_max_cols(FwdArgs& a, int K, int B, int CO, int CI, void* ws, hi
 }
 
 static void max_cols_report(const FwdArgs& a, int site, int B, int CO, int CI, hipStream_t st) {
-    if (g_linf_density < 0.f && a.gate) hint_record(site, a.w, B, CO, CI, a.gate + 1, st);
+    if (g_linf_density.load(std::memory_order_relaxed) < 0.f && a.gate) hint_record(site, a.w, B, CO, CI, a.gate + 1, st);
 }
 
 extern "C" int sd_set_linf_candidate_density(float density) {
@@ -138,6 +149,7 @@ static int run_chunk_pos(FwdArgs& a, bool index_lists, hipStream_t st, void* mer
 
 extern "C" int sd_inf_dist_forward_nograd(const float* input, const float* weight,
                                           int B, int CO, int CI, int G, int HW, float* output, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     FwdArgs a;
     int rc = make_fwd_args(a, "inf_dist_forward_nograd", input, nullptr, weight, B, CO, CI, G, HW, nullptr, nullptr, 0, 0);
     if (rc) return rc;
@@ -148,11 +160,12 @@ extern "C" int sd_inf_dist_forward_nograd(const float* input, const float* weigh
     const int TB = pick_tb(a, kTb42, 2, 128);
     a.nsplit = pick_nsplit(a, 16 * TB, 128);
     if (a.nsplit > 1 && (rc = fill_zero(output, (size_t)B * CO * HW, st))) return rc;
-    const int K = max_cols_wanted(a, kHintSiteLinf, 1.f, B, CO, CI, G, HW, st);
-    if (K) {
-        void* ws = workspace(max_cols_workspace(B, CO, CI, K), st);   // the only request of this call
+    const int KE = max_cols_eligible(a, 1.f, B, CO, CI, G, HW);
+    const int K = max_cols_wanted(a, KE, kHintSiteLinf, B, CO, CI, st);
+    if (KE) {
+        void* ws = workspace(max_cols_workspace(B, CO, CI, KE), st);   // the only request of this call
         if (!ws) return SD_ERR_HIP;
-        if ((rc = queue_max_cols(a, K, B, CO, CI, ws, st))) return rc;
+        if (K && (rc = queue_max_cols(a, K, B, CO, CI, ws, st))) return rc;
     }
     rc = TB == 2 ? launch_fwd<LinfNograd, 2, 8>(a, st) : launch_fwd<LinfNograd, 4, 8>(a, st);
     if (K && rc == SD_OK) max_cols_report(a, kHintSiteLinf, B, CO, CI, st);
@@ -163,6 +176,7 @@ extern "C" int sd_inf_dist_forward(const float* input, const float* weight,
                                    int B, int CO, int CI, int G, int HW, float* output, int* pos,
                                    const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
                                    sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     FwdArgs a;
     int rc = make_fwd_args(a, "inf_dist_forward", input, nullptr, weight, B, CO, CI, G, HW,
                            w_index_ci, w_index_co, W_CO, W_CI);
@@ -170,16 +184,17 @@ extern "C" int sd_inf_dist_forward(const float* input, const float* weight,
     SD_REQUIRE(output && pos, "inf_dist_forward: null output or pos");
     a.y0 = output; a.p0 = pos;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int K = max_cols_wanted(a, kHintSiteLinf, 1.f, B, CO, CI, G, HW, st);
-    if (!K) return run_chunk_pos<LinfChunk>(a, w_index_ci || w_index_co, st);
+    const int KE = max_cols_eligible(a, 1.f, B, CO, CI, G, HW);
+    if (!KE) return run_chunk_pos<LinfChunk>(a, w_index_ci || w_index_co, st);
+    const int K = max_cols_wanted(a, KE, kHintSiteLinf, B, CO, CI, st);
     // one workspace request for both users: the split-N merge buffer first, the tables (with the counter the gates
     // read) behind it
     const size_t merge = (((size_t)B * CO * 8) + 255) / 256 * 256;
-    char* base = static_cast<char*>(workspace(merge + max_cols_workspace(B, CO, CI, K), st));
+    char* base = static_cast<char*>(workspace(merge + max_cols_workspace(B, CO, CI, KE), st));
     if (!base) return SD_ERR_HIP;
-    if ((rc = queue_max_cols(a, K, B, CO, CI, base + merge, st))) return rc;
+    if (K && (rc = queue_max_cols(a, K, B, CO, CI, base + merge, st))) return rc;
     rc = run_chunk_pos<LinfChunk>(a, false, st, base, merge);
-    if (rc == SD_OK) max_cols_report(a, kHintSiteLinf, B, CO, CI, st);
+    if (K && rc == SD_OK) max_cols_report(a, kHintSiteLinf, B, CO, CI, st);
     return rc;
 }
 
@@ -221,6 +236,7 @@ extern "C" int sd_inf_dist_forward_noalloc(const float* input, const float* weig
                                            int B, int CO, int CI, int G, int HW, float* output, int* pos,
                                            const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
                                            sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     FwdArgs a;
     int rc = make_fwd_args(a, "inf_dist_forward_noalloc", input, nullptr, weight, B, CO, CI, G, HW,
                            w_index_ci, w_index_co, W_CO, W_CI);
@@ -239,6 +255,7 @@ extern "C" int sd_inf_dist_forward_noalloc(const float* input, const float* weig
 extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weight,
                                           int B, int CO, int CI, int G, int HW, float* output, int* pos,
                                           float q, uint32_t seed, int mode, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     FwdArgs a;
     int rc = make_fwd_args(a, "masked_inf_dist_forward", input, nullptr, weight, B, CO, CI, G, HW, nullptr, nullptr, 0, 0);
     if (rc) return rc;
@@ -268,8 +285,9 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
         packed_bytes = pos ? (((size_t)a.R * CO * 8 + 255) / 256) * 256 : 0;
         // one request for every user of the workspace: merge buffer, keep bits, candidate tables
         const size_t mask_bytes = ((size_t)(xrows + wrows) * nchunks * 4 + 255) / 256 * 256;
-        K = max_cols_wanted(a, kHintSiteMasked, (float)a.t16 / 65536.f, B, CO, CI, G, HW, st);
-        char* base = static_cast<char*>(workspace(packed_bytes + mask_bytes + (K ? max_cols_workspace(B, CO, CI, K) : 0), st));
+        const int KE = max_cols_eligible(a, (float)a.t16 / 65536.f, B, CO, CI, G, HW);
+        K = max_cols_wanted(a, KE, kHintSiteMasked, B, CO, CI, st);
+        char* base = static_cast<char*>(workspace(packed_bytes + mask_bytes + (KE ? max_cols_workspace(B, CO, CI, KE) : 0), st));
         if (!base) return SD_ERR_HIP;
         tables = base + packed_bytes + mask_bytes;
         uint32_t* xm = reinterpret_cast<uint32_t*>(base + packed_bytes);
@@ -300,6 +318,7 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
 extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float* inputU, const float* weight,
                                                 int B, int CO, int CI, int G, int HW, float* outputL, float* outputU,
                                                 sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     FwdArgs a;
     SD_REQUIRE(inputU, "bound_inf_dist_forward_nograd: null upper input");
     int rc = make_fwd_args(a, "bound_inf_dist_forward_nograd", inputL, inputU, weight, B, CO, CI, G, HW,
@@ -313,27 +332,36 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
     a.nsplit = pick_nsplit(a, 16 * TB, 16 * 8);
     // dense single-group layers: a kernel that works from per-weight-row candidate tables is queued in front of the
     // one that evaluates every term, and a count taken on the device decides which of the two runs
-    const float cap = g_bound_density >= 0.f ? g_bound_density : kBoundColsCap;
+    const float bound_density = g_bound_density.load(std::memory_order_relaxed);
+    const int bound_form = g_bound_form.load(std::memory_order_relaxed);
+    const float cap = bound_density >= 0.f ? bound_density : kBoundColsCap;
     bool cols = cap > 0.f && G == 1 && HW == 1 && CI % kColsChunk == 0 && a.fast_x && a.fast_w &&
-                (g_bound_density >= 0.f || (long long)B * CO * CI >= kBoundColsMinTerms);
+                (bound_density >= 0.f || (long long)B * CO * CI >= kBoundColsMinTerms);
+    // The workspace is sized by shape alone (whatever the hints below decide), so that a call under graph capture,
+    // which always builds the staged tables, never needs more than the eager call before it did.
+    char* wsbase = nullptr;
+    if (cols) {
+        const size_t staged = bound_cols_workspace(B, CO, CI), walk = CI <= 65536 ? sort_cols_workspace(B, CO, CI, 1) : 0;
+        wsbase = static_cast<char*>(workspace(staged > walk ? staged : walk, st));   // the only request of this call
+        if (!wsbase) return SD_ERR_HIP;
+    }
     // with the built-in limit, a layer whose tables have not paid lately is not given any for a while
-    const bool hinted = cols && g_bound_density < 0.f;
+    const bool hinted = cols && bound_density < 0.f;
     if (hinted && !hint_build_tables(kHintSiteBound, weight, B, CO, CI, st)) cols = false;
     // Very few marks (weights of unit scale against rows that are alike: below 1 %): the staged kernel would spend its
     // time moving tiles through LDS, and the kernel that walks a weight row's marks over a transposed copy of the
     // inputs serves better.  Chosen by hand (sd_set_bound_candidate_form) or, with the built-in limit, for a layer
     // whose last three staged calls reported that few marks ("not building" the staged tables, in the hint's terms).
-    bool sparse = cols && g_bound_form == 2 && CI <= 65536;
-    if (cols && g_bound_form == 0 && hinted && CI <= 65536)
+    bool sparse = cols && bound_form == 2 && CI <= 65536;
+    if (cols && bound_form == 0 && hinted && CI <= 65536)
         sparse = !hint_build_tables(kHintSiteBoundSparse, weight, B, CO, CI, st);
     if (sparse) {
-        void* ws = workspace(sort_cols_workspace(B, CO, CI, 1), st);   // the only request of this call
-        if (!ws) return SD_ERR_HIP;
+        void* ws = wsbase;
         if (a.nsplit > 1) {   // the every-term kernel, should it run, merges its slices into zeros
             if ((rc = fill_zero2(outputL, (size_t)B * CO * HW, outputU, (size_t)B * CO * HW, st))) return rc;
         }
         if ((rc = sort_cols_forward(inputL, inputU, weight, B, CO, CI, 0.f, 1, outputL, outputU, nullptr, ws,
-                                    g_bound_density > 0.f ? g_bound_density : kBoundSparseCap, &a.gate, &a.gate_limit, st)))
+                                    bound_density > 0.f ? bound_density : kBoundSparseCap, &a.gate, &a.gate_limit, st)))
             return rc;
         a.gate_above = 1;
         return TB == 2 ? launch_fwd<BoundNogradGated, 2, 8>(a, st) : launch_fwd<BoundNogradGated, 4, 8>(a, st);
@@ -342,16 +370,15 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
         if ((rc = fill_zero2(outputL, (size_t)B * CO * HW, outputU, (size_t)B * CO * HW, st))) return rc;
     }
     if (cols) {
-        void* ws = workspace(bound_cols_workspace(B, CO, CI), st);
-        if (!ws) return SD_ERR_HIP;
+        void* ws = wsbase;
         if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, outputL, outputU, nullptr, nullptr, ws, cap,
-                                     g_bound_density >= 0.f ? g_bound_density : kBoundRowsCap, &a.gate, &a.gate_limit, st)))
+                                     bound_density >= 0.f ? bound_density : kBoundRowsCap, &a.gate, &a.gate_limit, st)))
             return rc;
         a.gate_above = 1;
         rc = TB == 2 ? launch_fwd<BoundNogradGated, 2, 8>(a, st) : launch_fwd<BoundNogradGated, 4, 8>(a, st);
         if (hinted && rc == SD_OK) {
             hint_record(kHintSiteBound, weight, B, CO, CI, a.gate, st);   // the gate is 1 when every term ran
-            if (g_bound_form == 0) hint_record(kHintSiteBoundSparse, weight, B, CO, CI, a.gate + 1, st);   // 1: very few marks
+            if (bound_form == 0) hint_record(kHintSiteBoundSparse, weight, B, CO, CI, a.gate + 1, st);   // 1: very few marks
         }
         return rc;
     }
@@ -374,6 +401,7 @@ extern "C" int sd_set_bound_candidate_form(int form) {
 extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* inputU, const float* weight,
                                          int B, int CO, int CI, int G, int HW, float* outputL, float* outputU,
                                          int* posL, int* posU, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     FwdArgs a;
     SD_REQUIRE(inputU, "bound_inf_dist_forward: null upper input");
     int rc = make_fwd_args(a, "bound_inf_dist_forward", inputL, inputU, weight, B, CO, CI, G, HW,
@@ -387,20 +415,22 @@ extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* input
     a.nsplit = pick_nsplit(a, 16 * TB, 64);
     // dense single-group layers: the table kernel, tracking the chunk of every result, is queued in front
     // of the every-term kernel as for the forward without positions; both leave (value, chunk) pairs for the resolve
-    const float cap = g_bound_density >= 0.f ? g_bound_density : kBoundPosColsCap;
+    const float bound_density = g_bound_density.load(std::memory_order_relaxed);
+    const float cap = bound_density >= 0.f ? bound_density : kBoundPosColsCap;
     bool cols = cap > 0.f && G == 1 && HW == 1 && CI % kColsChunk == 0 && a.fast_x && a.fast_w &&
-                (g_bound_density >= 0.f || (long long)B * CO * CI >= kBoundColsMinTerms);
-    const bool hinted = cols && g_bound_density < 0.f;
+                (bound_density >= 0.f || (long long)B * CO * CI >= kBoundColsMinTerms);
+    const bool elig = cols;   // by shape alone: what the workspace is sized by (a captured call always builds tables)
+    const bool hinted = cols && bound_density < 0.f;
     if (hinted && !hint_build_tables(kHintSiteBoundPos, weight, B, CO, CI, st)) cols = false;
     if (cols && a.nsplit < 2) a.nsplit = 2;   // both kernels merge into the packed pairs
-    if (a.nsplit > 1) {
+    if (a.nsplit > 1 || elig) {
         size_t n = (size_t)a.R * a.G * a.COg;
         const size_t pairs = (n * 16 + 255) / 256 * 256;
-        char* ws = static_cast<char*>(workspace(pairs + (cols ? bound_cols_workspace(B, CO, CI) : 0), st));   // the only request
+        char* ws = static_cast<char*>(workspace(pairs + (elig ? bound_cols_workspace(B, CO, CI) : 0), st));   // the only request
         if (!ws) return SD_ERR_HIP;
         a.packed0 = reinterpret_cast<unsigned long long*>(ws);
         a.packed1 = a.packed0 + n;
-        if ((rc = fill_zero(a.packed0, n * 4, st))) return rc;
+        if (a.nsplit > 1 && (rc = fill_zero(a.packed0, n * 4, st))) return rc;
         if (cols) {
             if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, nullptr, nullptr, a.packed0, a.packed1,
                                          ws + pairs, cap, cap, &a.gate, &a.gate_limit, st)))

@@ -1,4 +1,5 @@
 // l-p norm distance: forward entry points and the fused backward kernel.
+#include <atomic>
 #include <cstdlib>
 #include "fwd_tile.h"
 #include "fwd_args.h"
@@ -16,7 +17,7 @@ constexpr float kLpSkipFromFused = 0.68f, kLpSkipFromGeneral = 0.73f;
 
 // largest share of marked (tile, row, input) triples at which the candidate-table kernels run instead of the
 // kernels that evaluate every term (sd_set_lp_candidate_density); negative: the built-in limits below
-static float g_rows_density = -1.f;
+static std::atomic<float> g_rows_density{-1.f};
 // Measured at B = 512, M = N = 5120 on three kinds of data (normal or uniform inputs against small weights,
 // normal inputs against weights of the same size), in ms against the marked share d:
 //   forward   table kernel 0.2 + 3.6 d    every term 2.8, with wave-level significance tests 1.3 .. 3.6
@@ -30,7 +31,8 @@ constexpr float kRowsCapBackwardInput = 0.55f, kRowsCapBackwardInputSkip = 0.3f;
 // below this threshold (p of about 12 forward, 20 backward) most inputs are marked on all three
 constexpr float kRowsFromThr = 0.15f;
 static inline float rows_cap(float builtin, float thr) {
-    if (g_rows_density >= 0.f) return g_rows_density;
+    const float density = g_rows_density.load(std::memory_order_relaxed);
+    if (density >= 0.f) return density;
     return thr >= kRowsFromThr ? builtin : 0.f;
 }
 
@@ -662,6 +664,7 @@ extern "C" int sd_norm_dist_forward(const float* input, const float* weight,
                                     int B, int CO, int CI, int G, int HW, float* output, float p,
                                     const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
                                     sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     FwdArgs a;
     int rc = make_fwd_args(a, "norm_dist_forward", input, nullptr, weight, B, CO, CI, G, HW,
                            w_index_ci, w_index_co, W_CO, W_CI);
@@ -691,6 +694,7 @@ extern "C" int sd_norm_dist_forward_with_max(const float* input, const float* we
                                              int B, int CO, int CI, int G, int HW, float* output, float p,
                                              const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
                                              sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     FwdArgs a;
     int rc = make_fwd_args(a, "norm_dist_forward_with_max", input, nullptr, weight, B, CO, CI, G, HW,
                            w_index_ci, w_index_co, W_CO, W_CI);
@@ -706,6 +710,7 @@ extern "C" int sd_norm_dist_backward_input(const float* grad_output, const float
                                            float* grad_input, float p,
                                            const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
                                            sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     return lp_backward("norm_dist_backward_input", grad_output, input, weight, output, B, CO, CI, G, HW,
                        grad_input, nullptr, p, w_index_ci, w_index_co, W_CO, W_CI, stream);
 }
@@ -715,6 +720,7 @@ extern "C" int sd_norm_dist_backward_input_weight(const float* grad_output, cons
                                                   float* grad_input, float* grad_weight, float p,
                                                   const int* w_index_ci, const int* w_index_co, int W_CO, int W_CI,
                                                   sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     SD_REQUIRE(grad_weight, "norm_dist_backward_input_weight: null grad_weight");
     return lp_backward("norm_dist_backward_input_weight", grad_output, input, weight, output, B, CO, CI, G, HW,
                        grad_input, grad_weight, p, w_index_ci, w_index_co, W_CO, W_CI, stream);

@@ -134,6 +134,7 @@ using namespace sd;
 
 extern "C" int sd_mean_shift_forward(const float* input, int B, int C, int HW, float* mean, float* running_mean,
                                      float momentum, float* output, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     int rc = check_dims("mean_shift_forward", B, C, HW);
     if (rc) return rc;
     SD_REQUIRE(input && mean && output, "mean_shift_forward: null pointer");
@@ -151,6 +152,7 @@ extern "C" int sd_mean_shift_forward(const float* input, int B, int C, int HW, f
 
 extern "C" int sd_channel_shift(const float* input, const float* shift, int B, int C, int HW, float sign,
                                 float* output, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     int rc = check_dims("channel_shift", B, C, HW);
     if (rc) return rc;
     SD_REQUIRE(input && shift && output, "channel_shift: null pointer");
@@ -165,6 +167,7 @@ extern "C" int sd_channel_shift(const float* input, const float* shift, int B, i
 extern "C" int sd_mean_shift_index_forward(const float* input, const int* index, int B, int G, int cnt, int Cg, int HW,
                                            float* mean, float* running_mean, float momentum, float* output,
                                            sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     SD_REQUIRE(G > 0 && cnt > 0 && Cg >= cnt, "mean_shift_index_forward: need G > 0 and 0 < cnt <= Cg (cnt=%d Cg=%d)", cnt, Cg);
     SD_REQUIRE((long long)G * cnt < (1ll << 31) && (long long)G * Cg < (1ll << 31), "mean_shift_index_forward: too many channels");
     int rc = check_dims("mean_shift_index_forward", B, G * cnt, HW);

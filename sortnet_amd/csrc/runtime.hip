@@ -1,4 +1,5 @@
 // Library runtime: error reporting, device queries, fill kernel and the verification exports.
+#include <atomic>
 #include <cmath>
 #include <mutex>
 #include <vector>
@@ -50,16 +51,20 @@ void forward_kernel_timer(hipStream_t stream, bool after) {
     g_timed = after;
 }
 
+static std::recursive_mutex g_call_mu;
+CallGuard::CallGuard() { g_call_mu.lock(); }
+CallGuard::~CallGuard() { g_call_mu.unlock(); }
+
 int num_cus() {
-    static int cached[64] = {0};
+    static std::atomic<int> cached[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int n = 0;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev] = n;
+        cached[dev].store(n, std::memory_order_relaxed);
     }
-    return cached[dev];
+    return n;
 }
 
 void* workspace(size_t bytes, hipStream_t stream) {
@@ -93,16 +98,20 @@ void* workspace(size_t bytes, hipStream_t stream) {
 
 namespace {
 constexpr int kHintRing = 4;   // outcomes of a layer that may be on their way to the host at once
+constexpr size_t kHintSlots = 256;   // layers (site, weight matrix) the hints remember at a time
 struct HintSlot {
     int dev, site, B, CO, CI;
     const void* weight;         // the layer: same shapes with other weights are other layers
     unsigned long long* host;   // pinned: kHintRing flags
     hipEvent_t ev[kHintRing];   // recorded behind the copy of flag i
     int head, queued;           // oldest outcome not yet looked at, and how many are queued
+    int stale;                  // of the queued outcomes, how many belong to the layer the slot stood for before
     int streak, skip_left;
+    unsigned long long used;    // g_hint_clock at the slot's last use: the least recently used slot is given away
 };
 std::mutex g_hint_mu;
 std::vector<HintSlot> g_hints;
+unsigned long long g_hint_clock = 0;
 
 bool capturing(hipStream_t stream) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
@@ -110,22 +119,51 @@ bool capturing(hipStream_t stream) {
     return cap != hipStreamCaptureStatusNone;
 }
 
+// A slot that is handed to another layer keeps its pinned memory and events (copies into them may still be on their
+// way); what is queued at that moment is counted as stale and thrown away when it arrives.
+void hint_rekey(HintSlot& h, int dev, int site, const void* weight, int B, int CO, int CI) {
+    h.dev = dev; h.site = site; h.weight = weight; h.B = B; h.CO = CO; h.CI = CI;
+    h.stale = h.queued;
+    h.streak = h.skip_left = 0;
+}
+
 HintSlot* hint_slot(int site, const void* weight, int B, int CO, int CI, bool create) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-    for (HintSlot& h : g_hints)
-        if (h.dev == dev && h.site == site && h.weight == weight && h.B == B && h.CO == CO && h.CI == CI) return &h;
-    if (!create || g_hints.size() >= 256) return nullptr;
+    HintSlot* same_weight = nullptr;
+    for (HintSlot& h : g_hints) {
+        if (h.dev != dev || h.site != site || h.weight != weight) continue;
+        if (h.B == B && h.CO == CO && h.CI == CI) { h.used = ++g_hint_clock; return &h; }
+        same_weight = &h;
+    }
+    if (!create) return nullptr;
+    // the same address with another shape: the memory holds another layer now, the old one's history is dropped
+    if (same_weight) { hint_rekey(*same_weight, dev, site, weight, B, CO, CI); same_weight->used = ++g_hint_clock; return same_weight; }
+    if (g_hints.size() >= kHintSlots) {
+        HintSlot* oldest = nullptr;
+        for (HintSlot& h : g_hints)
+            if (h.dev == dev && (!oldest || h.used < oldest->used)) oldest = &h;   // events belong to their device
+        if (!oldest) return nullptr;
+        hint_rekey(*oldest, dev, site, weight, B, CO, CI);
+        oldest->used = ++g_hint_clock;
+        return oldest;
+    }
     HintSlot h{};
-    h.dev = dev; h.site = site; h.B = B; h.CO = CO; h.CI = CI; h.weight = weight;
     if (hipHostMalloc(reinterpret_cast<void**>(&h.host), kHintRing * sizeof(unsigned long long), hipHostMallocDefault) != hipSuccess) {
         (void)hipGetLastError();
         return nullptr;
     }
     for (int i = 0; i < kHintRing; i++) {
         h.host[i] = 0;
-        if (hipEventCreateWithFlags(&h.ev[i], hipEventDisableTiming) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+        if (hipEventCreateWithFlags(&h.ev[i], hipEventDisableTiming) != hipSuccess) {
+            (void)hipGetLastError();
+            for (int k = 0; k < i; k++) (void)hipEventDestroy(h.ev[k]);   // nothing has been recorded on them yet
+            (void)hipHostFree(h.host);
+            return nullptr;
+        }
     }
+    hint_rekey(h, dev, site, weight, B, CO, CI);
+    h.used = ++g_hint_clock;
     g_hints.push_back(h);
     return &g_hints.back();
 }
@@ -139,10 +177,13 @@ bool hint_build_tables(int site, const void* weight, int B, int CO, int CI, hipS
     // outcomes that have arrived, oldest first (the host may run several calls ahead of the device)
     while (h->queued > 0) {
         if (hipEventQuery(h->ev[h->head]) != hipSuccess) { (void)hipGetLastError(); break; }   // not ready: next call
-        h->streak = h->host[h->head] != 0ull ? h->streak + 1 : 0;
-        // the streak is long enough (or the probe after a stretch without tables came out the same): no tables
-        // for the next kHintSkip calls, then one call probes again
-        h->skip_left = h->streak >= kHintStreak ? kHintSkip : 0;
+        if (h->stale > 0) h->stale--;   // an outcome of the layer this slot stood for before
+        else {
+            h->streak = h->host[h->head] != 0ull ? h->streak + 1 : 0;
+            // the streak is long enough (or the probe after a stretch without tables came out the same): no tables
+            // for the next kHintSkip calls, then one call probes again
+            h->skip_left = h->streak >= kHintStreak ? kHintSkip : 0;
+        }
         h->head = (h->head + 1) % kHintRing;
         h->queued--;
     }

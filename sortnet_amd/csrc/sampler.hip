@@ -153,6 +153,7 @@ extern "C" int sd_mask_count(uint32_t seed, int C, float q) {
 }
 
 extern "C" int sd_sample_index_lists(uint32_t seed, int S, int G, int C, int count, int* out, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     SD_REQUIRE(S > 0 && G > 0 && C > 0 && C < 65536, "sample_index_lists: need S, G > 0 and 0 < C < 65536");
     SD_REQUIRE(count >= 0 && count <= C, "sample_index_lists: count=%d outside 0..C=%d", count, C);
     if (count == 0) return SD_OK;

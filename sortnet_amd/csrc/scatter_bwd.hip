@@ -334,6 +334,7 @@ using namespace sd;
 
 extern "C" int sd_inf_dist_backward_input(const float* grad_output, const int* pos,
                                           int B, int CO, int CI, int G, int HW, float* grad_input, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     BwdArgs a;
     int rc = make_bwd_args(a, "inf_dist_backward_input", B, CO, CI, G, HW, nullptr, nullptr, 0, 0);
     if (rc) return rc;
@@ -346,6 +347,7 @@ extern "C" int sd_inf_dist_backward_input_weight(const float* grad_output, const
                                                  int B, int CO, int CI, int G, int HW, float* grad_input,
                                                  float* grad_weight, const int* w_index_ci, const int* w_index_co,
                                                  int W_CO, int W_CI, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     BwdArgs a;
     int rc = make_bwd_args(a, "inf_dist_backward_input_weight", B, CO, CI, G, HW, w_index_ci, w_index_co, W_CO, W_CI);
     if (rc) return rc;
@@ -372,12 +374,14 @@ static int sort_bwd(const char* who, const float* grad_output, const int* pos, i
 extern "C" int sd_sort_neuron_backward_input(const float* grad_output, const int* pos,
                                              int B, int CO, int CI, int G, int HW, float* grad_input,
                                              float q, int K, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     return sort_bwd("sort_neuron_backward_input", grad_output, pos, B, CO, CI, G, HW, grad_input, nullptr, q, K, stream);
 }
 
 extern "C" int sd_sort_neuron_backward_input_weight(const float* grad_output, const int* pos,
                                                     int B, int CO, int CI, int G, int HW, float* grad_input,
                                                     float* grad_weight, float q, int K, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     SD_REQUIRE(grad_weight, "sort_neuron_backward_input_weight: null grad_weight");
     return sort_bwd("sort_neuron_backward_input_weight", grad_output, pos, B, CO, CI, G, HW, grad_input, grad_weight,
                     q, K, stream);
@@ -415,6 +419,7 @@ static int bound_bwd(const char* who, const float* gL, const float* gU, const in
 extern "C" int sd_bound_inf_dist_backward_input(const float* grad_outputL, const float* grad_outputU,
                                                 const int* posL, const int* posU, int B, int CO, int CI, int G, int HW,
                                                 float* grad_inputL, float* grad_inputU, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     return bound_bwd("bound_inf_dist_backward_input", grad_outputL, grad_outputU, posL, posU, B, CO, CI, G, HW,
                      grad_inputL, grad_inputU, nullptr, stream);
 }
@@ -423,6 +428,7 @@ extern "C" int sd_bound_inf_dist_backward_input_weight(const float* grad_outputL
                                                        const int* posL, const int* posU, int B, int CO, int CI, int G,
                                                        int HW, float* grad_inputL, float* grad_inputU,
                                                        float* grad_weight, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     SD_REQUIRE(grad_weight, "bound_inf_dist_backward_input_weight: null grad_weight");
     return bound_bwd("bound_inf_dist_backward_input_weight", grad_outputL, grad_outputU, posL, posU, B, CO, CI, G, HW,
                      grad_inputL, grad_inputU, grad_weight, stream);

@@ -3,6 +3,7 @@
 #include "fwd_tile.h"
 #include "fwd_args.h"
 #include "sort_cols.h"
+#include <atomic>
 
 using namespace sd;
 
@@ -133,21 +134,28 @@ static int run_two_level(FwdArgs& a, bool small, int* keys, hipStream_t st) {
 // kernels that evaluate every term, and a count taken on the device decides which of the two runs (at most
 // kSortColsCap of the terms marked: the table kernel).  Negative g_sort_density: built-in limit, and only layers
 // large enough for the tables to pay; 0 never; up to 1: that share, at any size.
-static float g_sort_density = -1.f;
+static std::atomic<float> g_sort_density{-1.f};
 constexpr float kSortColsCap = 0.10f;
 constexpr long long kSortColsMinTerms = 1ll << 24;
 
 // `site`: which entry point asks (with the built-in limit, a layer whose tables have not paid lately is not given
 // any for a while, see hint_build_tables)
 constexpr int kHintSiteSort = 2, kHintSiteBoundSort = 3, kHintSiteSortPos = 6;
-static bool sort_cols_ok(const FwdArgs& a, int site, int B, int CO, int CI, int G, int HW, hipStream_t st) {
-    if (g_sort_density == 0.f || G != 1 || HW != 1 || CI % kSortColsChunk != 0 || !a.fast_x || !a.fast_w) return false;
-    if (g_sort_density > 0.f) return true;
-    return (long long)B * CO * CI >= kSortColsMinTerms && hint_build_tables(site, a.w, B, CO, CI, st);
+// shape and size alone: the workspace is sized by this, so that a call under graph capture (which always builds
+// tables) never needs more than the eager call before it did
+static bool sort_cols_eligible(const FwdArgs& a, int B, int CO, int CI, int G, int HW) {
+    const float density = g_sort_density.load(std::memory_order_relaxed);
+    // the mark lists of the table kernels hold 16-bit input numbers
+    if (density == 0.f || G != 1 || HW != 1 || CI % kSortColsChunk != 0 || CI > 65536 || !a.fast_x || !a.fast_w) return false;
+    return density > 0.f || (long long)B * CO * CI >= kSortColsMinTerms;
+}
+// eligible, and (with the built-in limit) the layer's tables have paid lately
+static bool sort_cols_ok(const FwdArgs& a, int site, int B, int CO, int CI, hipStream_t st) {
+    return g_sort_density.load(std::memory_order_relaxed) > 0.f || hint_build_tables(site, a.w, B, CO, CI, st);
 }
 // after the every-term kernels have been queued behind the table kernel
 static void sort_cols_report(const FwdArgs& a, int site, int B, int CO, int CI, hipStream_t st) {
-    if (g_sort_density < 0.f && a.gate) hint_record(site, a.w, B, CO, CI, a.gate + 1, st);
+    if (g_sort_density.load(std::memory_order_relaxed) < 0.f && a.gate) hint_record(site, a.w, B, CO, CI, a.gate + 1, st);
 }
 
 // `ws`: sort_cols_workspace() bytes.  The gate it leaves in `a` points into `ws`: the kernels queued behind it must
@@ -155,7 +163,8 @@ static void sort_cols_report(const FwdArgs& a, int site, int B, int CO, int CI, 
 // per call, carved by the caller).
 static int queue_sort_cols(FwdArgs& a, const float* xl, const float* xu, const float* w, int B, int CO, int CI, float q,
                            int K, float* outL, float* outU, int* pos, void* ws, hipStream_t st) {
-    const float cap = g_sort_density > 0.f ? g_sort_density : kSortColsCap;
+    const float density = g_sort_density.load(std::memory_order_relaxed);
+    const float cap = density > 0.f ? density : kSortColsCap;
     int rc = sort_cols_forward(xl, xu, w, B, CO, CI, q, K, outL, outU, pos, ws, cap, &a.gate, &a.gate_limit, st);
     a.gate_above = 1;
     return rc;
@@ -176,6 +185,7 @@ static bool few_tiles(const FwdArgs& a, int BB, int BM) {
 extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* weight,
                                              int B, int CO, int CI, int G, int HW, float* output, float q, int K,
                                              sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     FwdArgs a;
     int rc = make_fwd_args(a, "sort_neuron_forward_nograd", input, nullptr, weight, B, CO, CI, G, HW, nullptr, nullptr, 0, 0);
     if (rc) return rc;
@@ -184,12 +194,13 @@ extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* we
     a.y0 = output; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 64);
-    const bool two = K <= 12 && two_level_ok(a, K), cols = sort_cols_ok(a, kHintSiteSort, B, CO, CI, G, HW, st);
+    const bool two = K <= 12 && two_level_ok(a, K), elig = sort_cols_eligible(a, B, CO, CI, G, HW);
+    const bool cols = elig && sort_cols_ok(a, kHintSiteSort, B, CO, CI, st);
     // one request for both users of the workspace: the tables (with the counter the gates read) first, the key
     // lists of the two-level path behind them
-    const size_t tbytes = cols ? (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256 : 0;
+    const size_t tbytes = elig ? (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256 : 0;
     char* base = nullptr;
-    if (cols || two) {
+    if (elig || two) {
         base = static_cast<char*>(workspace(tbytes + (two ? two_level_bytes(a, K) : 0), st));
         if (!base) return SD_ERR_HIP;
     }
@@ -210,6 +221,7 @@ extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* we
 extern "C" int sd_sort_neuron_forward(const float* input, const float* weight,
                                       int B, int CO, int CI, int G, int HW, float* output, int* pos, float q, int K,
                                       sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     FwdArgs a;
     int rc = make_fwd_args(a, "sort_neuron_forward", input, nullptr, weight, B, CO, CI, G, HW, nullptr, nullptr, 0, 0);
     if (rc) return rc;
@@ -220,11 +232,12 @@ extern "C" int sd_sort_neuron_forward(const float* input, const float* weight,
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 32);
     const bool two = K <= 12 && two_level_ok(a, K);
-    const bool cols = sort_cols_ok(a, kHintSiteSortPos, B, CO, CI, G, HW, st);
+    const bool elig = sort_cols_eligible(a, B, CO, CI, G, HW);
+    const bool cols = elig && sort_cols_ok(a, kHintSiteSortPos, B, CO, CI, st);
     // one request for both users of the workspace, as in sd_sort_neuron_forward_nograd
-    const size_t tbytes = cols ? (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256 : 0;
+    const size_t tbytes = elig ? (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256 : 0;
     char* base = nullptr;
-    if (cols || two) {
+    if (elig || two) {
         base = static_cast<char*>(workspace(tbytes + (two ? two_level_bytes(a, K) : 0), st));
         if (!base) return SD_ERR_HIP;
     }
@@ -245,6 +258,7 @@ extern "C" int sd_sort_neuron_forward(const float* input, const float* weight,
 extern "C" int sd_bound_sort_neuron_forward(const float* inputL, const float* inputU, const float* weight,
                                             int B, int CO, int CI, int G, int HW, float* outputL, float* outputU,
                                             float q, int K, sd_stream_t stream) {
+    sd::CallGuard call_guard;   // calls of several host threads reach a stream one after the other, whole
     FwdArgs a;
     SD_REQUIRE(inputU, "bound_sort_neuron_forward: null upper input");
     int rc = make_fwd_args(a, "bound_sort_neuron_forward", inputL, inputU, weight, B, CO, CI, G, HW, nullptr, nullptr, 0, 0);
@@ -254,11 +268,12 @@ extern "C" int sd_bound_sort_neuron_forward(const float* inputL, const float* in
     a.y0 = outputL; a.y1 = outputU; a.q = q;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool small = few_tiles(a, 32, 32);
-    const bool cols = sort_cols_ok(a, kHintSiteBoundSort, B, CO, CI, G, HW, st);
-    if (cols) {
+    const bool elig = sort_cols_eligible(a, B, CO, CI, G, HW);
+    const bool cols = elig && sort_cols_ok(a, kHintSiteBoundSort, B, CO, CI, st);
+    if (elig) {
         void* ws = workspace(sort_cols_workspace(B, CO, CI, K), st);   // the only request of this call
         if (!ws) return SD_ERR_HIP;
-        if ((rc = queue_sort_cols(a, inputL, inputU, weight, B, CO, CI, q, K, outputL, outputU, nullptr, ws, st))) return rc;
+        if (cols && (rc = queue_sort_cols(a, inputL, inputU, weight, B, CO, CI, q, K, outputL, outputU, nullptr, ws, st))) return rc;
     }
     rc = SD_ERR_ARG;
     switch (K) {

@@ -5,8 +5,10 @@ core/norm_dist.py (file:line cited per symbol) so that its layers (core/models/n
 run unmodified on top of this module.  Inputs are 3-D (B, C, HW) fp32 tensors on the GPU,
 weight is (CO, CI / groups); outputs are fp32 on the input's device, positions are int32.
 
-Every function dispatches to the HIP kernels through `sortnet_amd.ext`; there is no pure-torch
-path, so `use_custom_cuda_func=False` (which selects one in the reference) is rejected.
+Every function dispatches to the HIP kernels through `sortnet_amd.ext`.  `use_custom_cuda_func=False`
+selects, as in the reference, a formulation in plain torch ops on the tensors' own device (differentiable
+by autograd, formed for a bounded number of output channels at a time); it is a second, independent
+statement of the same values and nothing in this library calls it on its own.
 """
 import math
 
@@ -29,11 +31,79 @@ def _want_grad(*tensors):
     return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
 
 
-def _no_fallback(flag, name):
-    if not flag:
-        raise NotImplementedError(
-            "%s: use_custom_cuda_func=False selects a pure-torch path in the reference; this library "
-            "only runs its HIP kernels" % name)
+# ---- use_custom_cuda_func=False: the reference's closed forms in torch ops ---------------------------------------
+# The reference forms the whole (B, G, CO/G, CI/G, HW) tensor of differences at once (53.7 GB at B=512,
+# CO=CI=5120); here the output channels go by in blocks whose differences stay below _TORCH_BLOCK_BYTES.
+_TORCH_BLOCK_BYTES = 256 << 20
+
+
+def _blocks_of_differences(inputs, weight, groups):
+    """Yields, group by group and block by block of output channels, the differences
+    d[k][b, m, n, hw] = inputs[k][b, g, n, hw] - weight[g, m, n] for every tensor of `inputs`, in the order in
+    which the outputs are laid out ((B, G * CO/G, HW), group-major)."""
+    B, C, HW = inputs[0].shape
+    cig = C // groups
+    cog = weight.size(0) // groups
+    w = weight.view(groups, cog, cig)
+    step = max(1, _TORCH_BLOCK_BYTES // max(1, 4 * len(inputs) * B * cig * HW))
+    for g in range(groups):
+        xs = [t[:, g * cig:(g + 1) * cig, :].unsqueeze(1) for t in inputs]        # (B, 1, cig, HW)
+        for m0 in range(0, cog, step):
+            wb = w[g, m0:m0 + step].unsqueeze(0).unsqueeze(-1)                    # (1, mc, cig, 1)
+            yield [x - wb for x in xs]
+
+
+def _torch_norm_dist(x, weight, p, groups):
+    """core/norm_dist.py:181-185: the l-p norm of the differences, scaled by their largest magnitude (which is
+    held constant under differentiation) so that large p neither overflows nor underflows."""
+    out = []
+    for (d,) in _blocks_of_differences([x], weight, groups):
+        with torch.no_grad():
+            scale = d.abs().amax(dim=2, keepdim=True)
+        out.append((torch.linalg.vector_norm(d / scale, ord=p, dim=2, keepdim=True) * scale).squeeze(2))
+    return torch.cat(out, dim=1)
+
+
+def _torch_sort_neuron(x, weight, groups, q, truncate):
+    """core/norm_dist.py:226-230: the `truncate` largest magnitudes, weighted q (1 - q)^j from the largest down and
+    normalised by 1 - (1 - q)^truncate (no 1e-10 floor in this form)."""
+    coef = ((1 - q) ** torch.arange(truncate, device=x.device, dtype=x.dtype) * q).view(1, 1, truncate, 1)
+    out = []
+    for (d,) in _blocks_of_differences([x], weight, groups):
+        top = torch.topk(d.abs(), k=truncate, dim=2)[0]                            # (B, mc, truncate, HW), descending
+        out.append((top * coef).sum(dim=2))
+    return torch.cat(out, dim=1) / (1 - (1 - q) ** truncate)
+
+
+def _torch_bound_inf_dist(x_lower, x_upper, weight, groups):
+    """core/norm_dist.py:251-259: per input the two ends w - l and u - w; the upper result is the largest of their
+    maxima and the lower result minus the smallest of their minima, both floored at 1e-10 (this form does not
+    repair inverted intervals)."""
+    lo, up = [], []
+    for dl, du in _blocks_of_differences([x_lower, x_upper], weight, groups):
+        t1, t2 = -dl, du
+        up.append(torch.maximum(t1, t2).clamp(min=1e-10).amax(dim=2))
+        lo.append((-torch.minimum(t1, t2).clamp(max=-1e-10)).amax(dim=2))
+    return torch.cat(lo, dim=1), torch.cat(up, dim=1)
+
+
+def _torch_norm_dist_dropout(x, weight, w_index_ci, w_index_co, p, groups):
+    """core/norm_dist.py:195-213 without the kernels: each 32-sample sub-batch meets the sub-matrix of the weight
+    that its two index lists select (a missing list keeps everything)."""
+    cog, cig = weight.size(0) // groups, weight.size(1)
+    w = weight.view(groups, cog, cig)
+    out = []
+    for s, b0 in enumerate(range(0, x.size(0), 32)):
+        rows = []
+        for g in range(groups):
+            wg = w[g]
+            if w_index_co is not None:
+                wg = wg.index_select(0, w_index_co[s, g].long())
+            if w_index_ci is not None:
+                wg = wg.index_select(1, w_index_ci[s, g].long())
+            rows.append(wg)
+        out.append(_torch_norm_dist(x[b0:b0 + 32], torch.cat(rows, dim=0), p, groups))
+    return torch.cat(out, dim=0)
 
 
 class NormDistF(torch.autograd.Function):
@@ -299,14 +369,16 @@ def mean_shift(x, running_mean=None, momentum=0.1):
 
 def norm_dist(input, weight, p, groups=1, use_custom_cuda_func=True, tag=None):
     """core/norm_dist.py:176-186."""
-    _no_fallback(use_custom_cuda_func, "norm_dist")
+    if not use_custom_cuda_func:
+        return _torch_norm_dist(input, weight, p, groups)
     return NormDistF.apply(input, weight, groups, p, _want_grad(input, weight), tag)
 
 
 def norm_dist_dropout(input, weight, w_index_ci, w_index_co, p, groups=1, use_custom_cuda_func=True, tag=None):
     """core/norm_dist.py:191-214.  `input` is already compacted to the kept channels; `weight` is the
     full tensor; the same index list serves the 32 samples of a sub-batch."""
-    _no_fallback(use_custom_cuda_func, "norm_dist_dropout")
+    if not use_custom_cuda_func:
+        return _torch_norm_dist_dropout(input, weight, w_index_ci, w_index_co, p, groups)
     return NormDistDropoutF.apply(input, weight, w_index_ci, w_index_co, groups, p, tag)
 
 
@@ -315,7 +387,8 @@ def sort_neuron(input, weight, groups=1, q=0.5, truncate=10, use_custom_cuda_fun
     truncate = min(weight.size(-1), truncate)
     if q is None or q == 1.0 or truncate == 1:
         return norm_dist(input, weight, float("inf"), groups, tag=tag)
-    _no_fallback(use_custom_cuda_func, "sort_neuron")
+    if not use_custom_cuda_func:
+        return _torch_sort_neuron(input, weight, groups, q, truncate)
     return SortNeuronF.apply(input, weight, groups, q, truncate, _want_grad(input, weight), tag)
 
 
@@ -333,7 +406,8 @@ def bound_sort_neuron(x_lower, x_upper, weight, groups=1, q=0.5, truncate=10, ta
 
 def bound_inf_dist(x_lower, x_upper, weight, groups=1, use_custom_cuda_func=True, tag=None):
     """core/norm_dist.py:246-260."""
-    _no_fallback(use_custom_cuda_func, "bound_inf_dist")
+    if not use_custom_cuda_func:
+        return _torch_bound_inf_dist(x_lower, x_upper, weight, groups)
     return BoundInfDistF.apply(x_lower, x_upper, weight, groups, _want_grad(x_lower, x_upper, weight), tag)
 
 

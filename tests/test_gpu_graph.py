@@ -270,3 +270,60 @@ def test_graph_replays_of_the_candidate_table_kernels(oracle):
         # the kernels differentiated their own y, which agrees with the oracle's to rel 1e-5: (d/y)^(p-1) moves by p times that
         for got, ref in ((captured["gx"], rgx), (captured["gw"], rgw), (captured["gx2"], rgx)):
             np.testing.assert_allclose(got.cpu().numpy(), ref, rtol=2e-3, atol=2e-3 * float(np.abs(ref).max()))
+
+
+def test_two_host_threads_on_one_stream_leave_results_unchanged():
+    """Two host threads call the same layers at the same time on torch's default stream (which all threads share
+    unless they switch): every entry point that uses the stream's workspace - split-reduction merge buffers, keep bits,
+    candidate tables - must give each thread the results it gets alone, call after call."""
+    import threading
+    from sortnet_amd import ext, _lib
+    dev = _dev()
+    B, CI, CO = 128, 3072, 384
+    _lib.set_bound_candidate_density(0.25)            # tables at this size, the count on the device still decides
+    w = (torch.randn(CO, CI, generator=torch.Generator().manual_seed(40)) * CI ** -0.5).to(dev)
+
+    def inputs(seed):
+        g = torch.Generator().manual_seed(seed)
+        base = torch.randn(1, CI, 1, generator=g) * 0.1
+        return (base + torch.randn(B, CI, 1, generator=g) * (0.01 if seed % 2 else 0.2)).to(dev)
+
+    def run(x, n):
+        outs = []
+        for _ in range(n):
+            y = torch.empty(B, CO, 1, device=dev); pos = torch.empty(B, CO, 1, device=dev, dtype=torch.int32)
+            ym = torch.empty_like(y); pm = torch.empty_like(pos)
+            yl, yu = torch.empty_like(y), torch.empty_like(y)
+            zl, zu, pl, pu = torch.empty_like(y), torch.empty_like(y), torch.empty_like(pos), torch.empty_like(pos)
+            ys = torch.empty_like(y)
+            ext.inf_dist_forward(x, w, y, pos, 1)
+            ext.masked_inf_dist_forward(x, w, ym, pm, 1, 0.3, 5, ext.MASK_FACTORED)
+            ext.bound_inf_dist_forward_nograd(x - 0.02, x + 0.02, w, yl, yu, 1)
+            ext.bound_inf_dist_forward(x - 0.02, x + 0.02, w, zl, zu, pl, pu, 1)
+            ext.sort_neuron_forward_nograd(x, w, ys, 1, 0.5, 6)
+            outs.append((y, pos, ym, pm, yl, yu, zl, zu, pl, pu, ys))
+        return outs
+
+    xs = [inputs(1), inputs(2)]
+    alone = [run(x, 1)[0] for x in xs]
+    torch.cuda.synchronize()
+    got, errors = [None, None], []
+
+    def worker(i):
+        try:
+            torch.cuda.set_device(dev)
+            got[i] = run(xs[i], 12)
+        except Exception as e:      # noqa: BLE001 - reported by the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for i in range(2):
+        for k, outs in enumerate(got[i]):
+            for a, b in zip(outs, alone[i]):
+                assert torch.equal(a, b), "thread %d, call %d" % (i, k)

@@ -124,6 +124,14 @@ def test_sort_candidate_kernels_at_layer_size(density):
             assert torch.equal(a, b), dens
 
 
+def test_rows_longer_than_the_mark_lists_take_the_every_term_kernels(oracle, density):
+    """The table kernels list marked inputs as 16-bit numbers: a dense layer with more than 65536 inputs per row
+    (a multiple of 32, enough terms for the tables, density forced on) must fall back to the every-term kernels
+    instead of being rejected."""
+    x, xl, xu, w = _data(8, 65568, 32, "random", 5)
+    _check(oracle, density, 1.0, x, xl, xu, w, 0.3, 10, "CI=65568")
+
+
 def test_sort_candidate_density_argument(density):
     from sortnet_amd import _lib
     with pytest.raises(RuntimeError):

@@ -1,6 +1,8 @@
 """The entry point that allocates nothing (sd_inf_dist_forward_noalloc) against sd_inf_dist_forward, through
 the C ABI: values and positions bit for bit, on two calls in a row that share the built-in scratch array, the
-second one smaller than the first (stale merge keys of the first call must not leak into it)."""
+second one smaller than the first (stale merge keys of the first call must not leak into it); and the property the
+entry point exists for: a call leaves the device's free memory unchanged, on a stream the library has never seen
+(no workspace of its own), and it can be recorded into a graph and replayed."""
 import pytest
 import torch
 
@@ -71,3 +73,36 @@ def test_noalloc_index_lists_and_limit():
     with pytest.raises(RuntimeError, match="exceed the maximum"):
         _lib.call("sd_inf_dist_forward_noalloc", x.data_ptr(), w.data_ptr(), 4096, 2048, 200, 1, 1,
                   x.data_ptr(), x.data_ptr(), None, None, 0, 0, None)
+
+
+def test_noalloc_allocates_nothing_and_runs_under_capture():
+    dev = _dev()
+    x, w = _pair(128, 3072, 1024, 21, dev)           # split reduction: the merge scratch is in use
+    (y0, p0), _ = _both(x, w)                         # reference result; also warms up code objects and the scratch address
+    y = torch.full_like(y0, -1.0)
+    pos = torch.full_like(p0, -7)
+    fresh = torch.cuda.Stream(device=dev)             # the library holds no workspace for this stream
+    with torch.cuda.stream(fresh):                    # (whatever the runtime sets up at a stream's first launch: now)
+        torch.zeros(8, device=dev).add_(1)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info(dev)
+    with torch.cuda.stream(fresh):
+        _call("sd_inf_dist_forward_noalloc", x, w, y, pos)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info(dev)
+    assert free1 == free0, "the call changed the device's free memory by %d bytes" % (free0 - free1)
+    assert torch.equal(y, y0) and torch.equal(pos, p0)
+    # recorded into a graph (where hipMalloc is not allowed) and replayed, with eager work between the replays
+    y.fill_(-1.0)
+    pos.fill_(-7)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _call("sd_inf_dist_forward_noalloc", x, w, y, pos)
+    for k in range(3):
+        y.fill_(-1.0)
+        pos.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, y0) and torch.equal(pos, p0), "replay %d" % k
+        (e0, q0), _ = _both(x, w)                     # eager calls that share the scratch, between replays
+        assert torch.equal(e0, y0) and torch.equal(q0, p0)
