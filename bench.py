@@ -25,6 +25,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 FP32_VECTOR_PEAK_TFLOPS = 157.3     # MI355X published fp32 vector peak
+NBATCH = 4                          # distinct synthetic batches cycled through the steps of the masked workload
 VALU_LANE_RATE = 78.64e12           # 256 CUs x 4 SIMD x 16 lanes x 2 issue ports x 2.4 GHz lane-instructions/s
 # HBM bytes of one 512x5120x5120 launch come from the committed counter summary (two rocprofv3 --pmc runs,
 # FETCH_SIZE and WRITE_SIZE, scaled by a plain copy of known size): the lines "traffic_bytes_per_launch" (interval
@@ -219,10 +220,14 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     else:
         groups = [model.parameters()]
     opts = [torch.optim.AdamW(g, lr=1e-4, fused=True) for g in groups]
+    # NBATCH distinct synthetic batches, step i takes batch i % NBATCH: the candidate tables and their hints see new
+    # inputs every step, as in training
     g = torch.Generator().manual_seed(0)
-    x = torch.rand(batch, in_features, generator=g).to(dev)
-    targets = torch.randint(0, classes, (batch,), generator=g).to(dev)
-    lower, upper = (x - eps).clamp(min=0), (x + eps).clamp(max=1)
+    batches = []
+    for _ in range(NBATCH):
+        bx = torch.rand(batch, in_features, generator=g).to(dev)
+        bt = torch.randint(0, classes, (batch,), generator=g).to(dev)
+        batches.append((bx, bt, (bx - eps).clamp(min=0), (bx + eps).clamp(max=1)))
 
     ev = lambda: torch.cuda.Event(enable_timing=True)
     phase_ms = {"forward": 0.0, "backward": 0.0, "optimizer": 0.0, "bounds": 0.0}
@@ -231,6 +236,10 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
     probe = []                   # operands of the last width x width interval layer of the last step
     dense_ms = []                # every-term interval kernel, per launch
     fwd_ms, fwd_kernel = [], [None]   # masked l-inf forward tile kernel, per launch
+    # per layer: the share of its terms that the forward / the interval forward formed (1 = every term), read from
+    # the candidate-table counters in the extra one-stream steps
+    fwd_share = [[] for _ in range(model.num_layers)]
+    ibp_share = [[] for _ in range(model.num_layers)]
 
     # The certification pass needs the weights and nothing of the training step, so it is queued on a second stream
     # (default priority) beside forward and backward, on the weights the forward uses and a snapshot of the running
@@ -251,7 +260,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
                 stream.wait_event(updated[i])
         return hook
 
-    def certification(timed, means, before_layer=None):
+    def certification(timed, means, lower, upper, before_layer=None):
         if timed and time_ibp:
             # the pass spelled out, to time every call of the interval forward of a width x width layer with events on
             # the stream it is queued on (torch's current stream)
@@ -264,6 +273,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
                     e0.record()
                     ext.bound_inf_dist_forward_nograd(lo, up, w, ylo, yup, 1)
                     e1.record()
+                    ibp_share[li].append(_lib.last_forward_term_share())
                     if w.size(0) == width and w.size(1) == width:
                         ibp_events.append((e0, e1))
                         probe[:] = [lo, up, w]
@@ -273,6 +283,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
         return model.bounds(lower, upper, means=means, before_layer=before_layer)
 
     def step(i, timed, after_layer=None, concurrent=None):
+        x, targets, lower, upper = batches[i % NBATCH]
         concurrent = overlap if concurrent is None else concurrent
         piped = pipeline and concurrent
         if pipeline and not piped:
@@ -285,7 +296,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
             side.wait_stream(main)                       # the snapshot; without `pipeline` also the previous step's optimizer
             with torch.cuda.stream(side):
                 marks[5].record()
-                lo, up = certification(timed, means, wait_updated(side) if piped else None)
+                lo, up = certification(timed, means, lower, upper, wait_updated(side) if piped else None)
                 marks[6].record()
         dist = model.forward(x, step_seed=i, after_layer=after_layer,
                              before_layer=wait_updated(main) if piped else None)
@@ -319,7 +330,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
             marks[3].record()
         if not concurrent:
             marks[5].record()
-            lo, up = certification(timed, model.running_mean)
+            lo, up = certification(timed, model.running_mean, lower, upper)
             marks[6].record()
         cert = margins(dist.detach(), targets, eps, lo, up)[1]
         marks[4].record()
@@ -347,6 +358,7 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
         # the largest share of the step - the masked l-inf forward with chunk tracking of those layers by the library's
         # events around the tile kernel's launch, read back after every such layer (which makes the host wait).
         def read_timer(i, w):
+            fwd_share[i].append(_lib.last_forward_term_share())
             if i > 0 and tuple(w.shape) == (width, width):
                 ms = _lib.last_forward_kernel_ms()
                 if ms is not None:
@@ -395,7 +407,14 @@ def run_masked(args, mask, q, steps, warmup, batch=None, in_features=None, width
         phase_ms["backward"] += marks[1].elapsed_time(marks[2]) / steps
         phase_ms["optimizer"] += marks[2].elapsed_time(marks[3]) / steps   # with `pipeline`: on its own stream, beside the next step
         phase_ms["bounds"] += marks[5].elapsed_time(marks[6]) / steps      # on its own stream with `overlap`
+    mean = lambda v: sum(v) / len(v) if v else 1.0
+    layer_terms = [w.numel() * batch for w in model.weights]
+    executed = {"forward_terms": sum(t * mean(sh) for t, sh in zip(layer_terms, fwd_share)),
+                "interval_terms": sum(t * mean(sh) for t, sh in zip(layer_terms, ibp_share)),
+                "forward_share_by_layer": [mean(sh) for sh in fwd_share],
+                "interval_share_by_layer": [mean(sh) for sh in ibp_share]} if time_ibp else None
     res = {
+        "executed": executed,
         "ms_per_step": elapsed * 1e3 / steps, "samples_per_s": batch / (elapsed / steps), "steps": steps,
         "host_ms_per_step": queued * 1e3 / steps,      # the host's time to queue a step
         "phase_ms": phase_ms, "terms_per_step": model.terms_per_sample() * batch,
@@ -519,6 +538,8 @@ def main():
                       weight_std=args.weight_std)
     step_s = head["ms_per_step"] * 1e-3
     step_flops = head["terms_per_step"] * (2 + 6)         # forward 2 flops/term, interval bounds 6 flops/term
+    ex = head["executed"]
+    executed_flops = 2.0 * ex["forward_terms"] + 6.0 * ex["interval_terms"] if ex else None
     layer_terms = args.batch * args.width * args.width
     launches, dense, fwd = head["ibp_launch_ms"], head["ibp_every_term_ms"], head["fwd_kernel_ms"]
     step_ms = sum(launches) / max(len(launches), 1)
@@ -585,7 +606,15 @@ def main():
         "config": {"workload": workload_text(args, args.mask, args.q),
                    "batch": args.batch, "width": args.width, "distance_layers": args.depth, "mask": args.mask,
                    "streams": 1 if args.no_overlap else 3},
-        "step_fp32_vector_frac": step_flops / step_s / (FP32_VECTOR_PEAK_TFLOPS * 1e12),
+        # ALGORITHMIC rate: 2 flops per forward term and 6 per interval term for EVERY term of every layer, over the
+        # step time and the fp32 vector peak.  Not a utilisation: the step forms only the terms its candidate tables
+        # mark (`executed`), so this figure can exceed what the vector units deliver.
+        "step_algorithmic_rate_vs_fp32_peak": step_flops / step_s / (FP32_VECTOR_PEAK_TFLOPS * 1e12),
+        # the same from the terms the step actually formed (table marks read back from the device in a few further
+        # one-stream steps): what the vector units really did per second of the step, against their peak
+        "step_executed_rate_vs_fp32_peak": (executed_flops / step_s / (FP32_VECTOR_PEAK_TFLOPS * 1e12)
+                                            if executed_flops else None),
+        "executed": head["executed"],
         "phase_ms": head["phase_ms"],
         "phase_note": ("the certification pass (bounds) is queued on a second stream beside forward and backward, on "
                        "the weights the forward uses; the optimizer, layer by layer on a third stream, waits for both, "
@@ -606,6 +635,19 @@ def main():
             return {"ms_per_step": r["ms_per_step"], "samples_per_s": r["samples_per_s"], "steps": steps,
                     "phase_ms": r["phase_ms"]}
 
+        # the same step with every candidate table switched off: each kernel forms every term, whatever the data
+        from sortnet_amd import _lib
+        setters = (_lib.set_bound_candidate_density, _lib.set_linf_candidate_density, _lib.set_sort_candidate_density,
+                   _lib.set_lp_candidate_density)
+        try:
+            for f in setters:
+                f(0.0)
+            sec["tables_off"] = dict(masked_entry(args.mask, args.q),
+                                     workload=workload_text(args, args.mask, args.q) + "; candidate tables off: every "
+                                     "kernel evaluates every term (the data-independent floor of `value`)")
+        finally:
+            for f in setters:
+                f(-1.0)
         other = "term" if args.mask == "factored" else "factored"
         sec[other + "_mask"] = dict(masked_entry(other, args.q), workload=workload_text(args, other, args.q))
         sec["q1"] = dict(masked_entry(args.mask, 1.0), workload=workload_text(args, args.mask, 1.0))
@@ -620,8 +662,10 @@ def main():
         sec["certification"] = {"ms_per_pass": r["certification_ms"],
                                 "workload": "evaluation-mode pass of the same model: sort neuron (K=10) for the value, "
                                             "interval sort neuron for the bounds, all layers, B=%d" % args.batch}
-        r = run_index_lists(args, 0.75, 8.0, short, warm)
-        sec["index_lists_q0.75_p8"] = {k: r[k] for k in ("ms_per_step", "samples_per_s", "steps", "workload")}
+        # the p-annealing phase of the reference's training (main.py:297-303: p from 8 to 1000 on a logarithmic schedule)
+        for pp in (8.0, 24.0, 256.0):
+            r = run_index_lists(args, 0.75, pp, short, warm)
+            sec["index_lists_q0.75_p%g" % pp] = {k: r[k] for k in ("ms_per_step", "samples_per_s", "steps", "workload")}
         for pp in (8.0, 64.0):
             sec["lp_layer_p%g" % pp] = run_lp_layer(args, pp, short, warm)
         sec["interval_layer_with_pos"] = run_interval_layer(args, short, warm)

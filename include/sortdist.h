@@ -71,6 +71,12 @@ const char* sd_last_forward_kernel(void);
  * recorded on a stream that is being captured. */
 int sd_time_forward_kernels(int on);
 float sd_last_forward_kernel_ms(void);
+/* For benchmarks that must say how much arithmetic a call really did: the share (0..1] of its B * CO * CI / G terms that
+ * the calling thread's last l-inf, masked (factored), interval or sort-neuron forward call formed.  Waits for `stream`
+ * (the one the call was queued on; call this before queueing anything else there) and reads the call's candidate-table
+ * counters: the marked share when a table kernel served the call, 1 when every term was evaluated or no table was
+ * queued (index lists, groups, small layers, l-p calls); -1 on a HIP error.  No reference counterpart. */
+float sd_last_forward_term_share(sd_stream_t stream);
 /* Dense single-group l-p calls at general p queue two kernels for the same result: one that evaluates every term
  * and one that works from a table of the inputs that can hold a term that counts (per output-channel tile and batch
  * row).  The share of marked table entries, counted on the device, decides which of the two runs: the table kernel

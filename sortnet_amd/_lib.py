@@ -48,6 +48,7 @@ _OTHER = {
     "sd_last_forward_kernel": ([], ctypes.c_char_p),
     "sd_time_forward_kernels": ([_i], _i),
     "sd_last_forward_kernel_ms": ([], ctypes.c_float),
+    "sd_last_forward_term_share": ([_S], ctypes.c_float),
     "sd_set_lp_candidate_density": ([_f], _i),
     "sd_set_bound_candidate_density": ([_f], _i),
     "sd_set_bound_candidate_form": ([_i], _i),
@@ -160,3 +161,15 @@ def last_forward_kernel_ms():
     """Duration of the forward tile kernel this thread launched last with timing on (waits for it), or None."""
     ms = load().sd_last_forward_kernel_ms()
     return None if ms < 0 else ms
+
+
+def last_forward_term_share(stream=None):
+    """Share of its terms that this thread's last forward call formed (waits for `stream`, default torch's current
+    one): the marked share when a candidate-table kernel served the call, 1.0 when every term was evaluated."""
+    if stream is None:
+        import torch
+        stream = torch.cuda.current_stream().cuda_stream
+    share = load().sd_last_forward_term_share(stream)
+    if share < 0:
+        raise RuntimeError("sd_last_forward_term_share failed")
+    return share

@@ -898,6 +898,7 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
     // the every-term kernel runs when count[2] > 0
     *gate = c.count + 2;
     *gate_limit = 0ull;
+    note_term_counts(c.count, 2, (double)S * CO * CI, (double)T * B * CI, limit_col);
     // a few workgroups per compute unit over the run: the work of a workgroup follows the marks of its rows
     hipLaunchKernelGGL(xt_kernel, dim3(CI / 16, S), dim3(256), 0, st, xl, xu, B, CI, c.count, limit_col, c.xt);
     if ((rc = check_launch("xt_kernel"))) return rc;

@@ -77,6 +77,14 @@ void note_forward_kernel(const char* kind, int tb, int tm);
 // sd_last_forward_kernel_ms.  Nothing while the stream is being captured.
 void forward_kernel_timer(hipStream_t stream, bool after);
 
+// What sd_last_forward_term_share reads: where the candidate-table counters of the calling thread's last forward
+// call lie on the device and how to turn them into the share of the terms that the call formed.
+//   kind 0: no tables were queued (every term is formed)
+//   kind 1: counts[0] = marked (tile, weight row, input) triples of denom0, counts[1] != 0 when the every-term kernel ran
+//   kind 2: counts[0] / counts[1] = marks of the table per weight row (of denom0) / per batch row (of denom1),
+//           counts[2] != 0 when the every-term kernel ran, else the per-weight-row table served iff counts[0] <= limit0
+void note_term_counts(const unsigned long long* counts, int kind, double denom0, double denom1, unsigned long long limit0);
+
 #define SD_REQUIRE(cond, ...)                                   \
     do {                                                        \
         if (!(cond)) { sd::set_error(__VA_ARGS__); return SD_ERR_ARG; } \

@@ -19,6 +19,7 @@ inline int make_fwd_args(FwdArgs& a, const char* who, const float* x0, const flo
     SD_REQUIRE((long long)B * HW < (1ll << 31) && (long long)B * CO * HW < (1ll << 31) &&
                (long long)B * CI * HW < (1ll << 31), "%s: tensor too large for 32-bit indexing", who);
     a = FwdArgs{};
+    note_term_counts(nullptr, 0, 1.0, 1.0, 0ull);   // until a table kernel is queued for this call
     a.x0 = x0; a.x1 = x1; a.w = w;
     a.ci_idx = ci_idx; a.co_idx = co_idx;
     a.B = B; a.R = B * HW; a.HW = HW; a.G = G;

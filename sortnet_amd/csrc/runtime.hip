@@ -31,6 +31,13 @@ void note_forward_kernel(const char* kind, int tb, int tm) {
     snprintf(g_fwd_kernel, sizeof(g_fwd_kernel), "%s<%d,%d>", kind, tb, tm);
 }
 
+struct TermNote { const unsigned long long* counts; int kind; double denom0, denom1; unsigned long long limit0; };
+static thread_local TermNote g_term_note = {nullptr, 0, 1.0, 1.0, 0ull};
+
+void note_term_counts(const unsigned long long* counts, int kind, double denom0, double denom1, unsigned long long limit0) {
+    g_term_note = TermNote{counts, kind, denom0, denom1, limit0};
+}
+
 // sd_time_forward_kernels / sd_last_forward_kernel_ms: two events per thread, created on first use
 static thread_local bool g_time_kernels = false, g_timed = false, g_time_ev_made = false;
 static thread_local hipEvent_t g_time_ev[2];
@@ -274,6 +281,21 @@ float sd_last_forward_kernel_ms(void) {
         return -1.f;
     }
     return ms;
+}
+
+float sd_last_forward_term_share(sd_stream_t stream) {
+    const sd::TermNote n = sd::g_term_note;
+    if (n.kind == 0 || !n.counts) return 1.f;
+    unsigned long long c[3] = {0ull, 0ull, 0ull};
+    // waits for the stream, so the call that left the counters has run and nothing has overwritten them yet
+    if (hipMemcpyAsync(c, n.counts, sizeof(c), hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)) != hipSuccess ||
+        hipStreamSynchronize(static_cast<hipStream_t>(stream)) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1.f;
+    }
+    if (n.kind == 1) return c[1] != 0ull ? 1.f : (float)((double)c[0] / n.denom0);
+    if (c[2] != 0ull) return 1.f;
+    return c[0] <= n.limit0 ? (float)((double)c[0] / n.denom0) : (float)((double)c[1] / n.denom1);
 }
 
 uint32_t sd_rng_word(uint32_t seed, uint32_t stream_id, uint32_t row, uint32_t col) {

@@ -882,6 +882,7 @@ int sort_cols_forward(const float* xl, const float* xu, const float* w, int B, i
     const unsigned long long limit = (unsigned long long)((double)tiles_b(B) * CO * CI * d);
     *gate = c.count;
     *gate_limit = limit;
+    note_term_counts(c.count, 1, (double)tiles_b(B) * CO * CI, 1.0, 0ull);
     if (K == 1 && xu) return run<1, true, true>(xl, xu, w, B, CO, CI, q, outL, outU, nullptr, c, limit, st);
     switch (K) {
 #define X(k) case k: return xu ? run<k, true>(xl, xu, w, B, CO, CI, q, outL, outU, nullptr, c, limit, st) \
@@ -917,6 +918,7 @@ int max_cols_forward(const float* x, const float* w, const uint32_t* xkeep, cons
     const unsigned long long limit = (unsigned long long)((double)tiles_b(B) * CO * CI * d);
     *gate = c.count;
     *gate_limit = limit;
+    note_term_counts(c.count, 1, (double)tiles_b(B) * CO * CI, 1.0, 0ull);
     if (!xkeep) {
         if (K == 1) return run_max<1, false>(x, w, nullptr, nullptr, B, CO, CI, y, pos, c, limit, st);
     } else switch (K) {
