@@ -31,7 +31,7 @@ def main():
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
     import torch
-    from sortnet_amd import ext
+    from sortnet_amd import ext, _lib
     dev = torch.device("cuda:0")
     B, N, M = args.shape
     g = torch.Generator().manual_seed(0)
@@ -56,6 +56,8 @@ def main():
     def t(name, f, flops_per_term=None, nbytes=None):
         f()
         torch.cuda.synchronize()
+        # the share of its terms that a forward call formed (below 1: a candidate-table kernel served it)
+        share = _lib.last_forward_term_share() if flops_per_term and name.split()[0].endswith(("forward", "forward_nograd", "factored")) else None
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(args.reps):
@@ -69,10 +71,13 @@ def main():
             row["frac_fp32_peak"] = row["tflops"] * 1e12 / PEAK
         if nbytes:
             row["gb_per_s"] = nbytes / (ms * 1e-3) / 1e9
+        if share is not None and share < 1.0:
+            row["terms_formed_share"] = share
         rows.append(row)
         if not args.json:
             extra = "  %6.1f TFLOP/s %5.1f%%" % (row["tflops"], 100 * row["frac_fp32_peak"]) if flops_per_term else ""
             extra += "  %7.1f GB/s" % row["gb_per_s"] if nbytes else ""
+            extra += "  (from tables: %.1f%% of the terms formed)" % (100 * share) if share is not None and share < 1.0 else ""
             print("%-38s %8.3f ms %7.1f fs/term%s" % (name, ms, row["fs_per_term"], extra), flush=True)
 
     on = set(args.ops.split(","))

@@ -83,6 +83,8 @@ void forward_kernel_timer(hipStream_t stream, bool after);
 //   kind 1: counts[0] = marked (tile, weight row, input) triples of denom0, counts[1] != 0 when the every-term kernel ran
 //   kind 2: counts[0] / counts[1] = marks of the table per weight row (of denom0) / per batch row (of denom1),
 //           counts[2] != 0 when the every-term kernel ran, else the per-weight-row table served iff counts[0] <= limit0
+//   kind 3: counts[0] = marks of the table per batch row (of denom0), counts[1] != 0 when the every-term kernels ran,
+//           counts[2] != 0 when the per-batch-row table served, counts[3] = marks of the table per weight row (of denom1)
 void note_term_counts(const unsigned long long* counts, int kind, double denom0, double denom1, unsigned long long limit0);
 
 #define SD_REQUIRE(cond, ...)                                   \

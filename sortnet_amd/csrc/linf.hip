@@ -3,6 +3,7 @@
 #include "fwd_args.h"
 #include "bound_cols.h"
 #include "sort_cols.h"
+#include "row_cands.h"
 #include <atomic>
 #include <mutex>
 #include <type_traits>
@@ -58,18 +59,46 @@ static int max_cols_wanted(const FwdArgs& a, int K, int site, int B, int CO, int
     return hint_build_tables(site, a.w, B, CO, CI, st) ? K : 0;
 }
 
+// Largest share of marked (tile of 128 weight rows, batch row, input) triples at which the l-inf kernel of the tables
+// per batch row runs.  Measured per 512 x 5120 x 5120 layer: 0.10 ms of tables + 0.09 ms of staging + about 4.5 x share
+// ms for the marks (the walk over a row's marks is bound by the latency of its dependent LDS reads and by the scalar
+// unit, about 30 instructions per mark for 2 x 64 terms), against 0.45 ms (0.60 with positions) for every term: at the
+// 6.5 % that inputs in [0, 1] mark against weights ~ N(0, 1/N) the two meet, so the limit sits below that.
+constexpr float kMaxRowsCap = 0.04f;
+
+// bytes of both tables' workspace for one call: per weight row first, per batch row behind it
+static size_t max_tables_bytes(int B, int CO, int CI, int K) {
+    const size_t cols = (max_cols_workspace(B, CO, CI, K) + 255) / 256 * 256;
+    return cols + (row_cands_supported(kRowsMax, K) ? (row_cands_workspace(kRowsMax, B, CO, CI, K) + 255) / 256 * 256 : 0);
+}
+
+// `ws`: max_tables_bytes() bytes.  Afterwards a.gate[0] is non-zero when the every-term kernels are to run.
 static int queue_max_cols(FwdArgs& a, int K, int B, int CO, int CI, void* ws, hipStream_t st) {
     const float density = g_linf_density.load(std::memory_order_relaxed);
     const float cap = density > 0.f ? density : kMaxColsCap;
     // depth 1: the mask keeps everything
-    int rc = max_cols_forward(a.x0, a.w, K == 1 ? nullptr : a.xmask, K == 1 ? nullptr : a.wmask, B, CO, CI, K, a.y0, a.p0,
-                              ws, cap, &a.gate, &a.gate_limit, st);
+    const uint32_t* xkeep = K == 1 ? nullptr : a.xmask;
+    const uint32_t* wkeep = K == 1 ? nullptr : a.wmask;
+    int rc = max_cols_forward(a.x0, a.w, xkeep, wkeep, B, CO, CI, K, a.y0, a.p0, ws, cap, &a.gate, &a.gate_limit, st);
     a.gate_above = 1;
-    return rc;
+    if (rc || !row_cands_supported(kRowsMax, K)) {
+        if (!rc) { a.gate = a.gate + 1; a.gate_limit = 0ull; }   // the flag behind the counter, as with both tables
+        return rc;
+    }
+    const unsigned long long* col_count = a.gate;
+    char* rows_ws = static_cast<char*>(ws) + (max_cols_workspace(B, CO, CI, K) + 255) / 256 * 256;
+    const unsigned long long* every = nullptr;
+    rc = row_cands_forward(kRowsMax, a.x0, nullptr, a.w, xkeep, wkeep, B, CO, CI, 0.f, K, nullptr, a.y0, a.p0, rows_ws,
+                           density > 0.f ? density : kMaxRowsCap, sort_cols_probe_sums(col_count), col_count, &every, st);
+    if (rc) return rc;
+    a.gate = every;
+    a.gate_limit = 0ull;
+    note_term_counts(every - 1, 3, (double)((CO + 127) / 128) * B * CI, (double)((B + 127) / 128) * CO * CI, 0ull);
+    return SD_OK;
 }
 
 static void max_cols_report(const FwdArgs& a, int site, int B, int CO, int CI, hipStream_t st) {
-    if (g_linf_density.load(std::memory_order_relaxed) < 0.f && a.gate) hint_record(site, a.w, B, CO, CI, a.gate + 1, st);
+    if (g_linf_density.load(std::memory_order_relaxed) < 0.f && a.gate) hint_record(site, a.w, B, CO, CI, a.gate, st);
 }
 
 extern "C" int sd_set_linf_candidate_density(float density) {
@@ -163,7 +192,7 @@ extern "C" int sd_inf_dist_forward_nograd(const float* input, const float* weigh
     const int KE = max_cols_eligible(a, 1.f, B, CO, CI, G, HW);
     const int K = max_cols_wanted(a, KE, kHintSiteLinf, B, CO, CI, st);
     if (KE) {
-        void* ws = workspace(max_cols_workspace(B, CO, CI, KE), st);   // the only request of this call
+        void* ws = workspace(max_tables_bytes(B, CO, CI, KE), st);   // the only request of this call
         if (!ws) return SD_ERR_HIP;
         if (K && (rc = queue_max_cols(a, K, B, CO, CI, ws, st))) return rc;
     }
@@ -190,7 +219,7 @@ extern "C" int sd_inf_dist_forward(const float* input, const float* weight,
     // one workspace request for both users: the split-N merge buffer first, the tables (with the counter the gates
     // read) behind it
     const size_t merge = (((size_t)B * CO * 8) + 255) / 256 * 256;
-    char* base = static_cast<char*>(workspace(merge + max_cols_workspace(B, CO, CI, KE), st));
+    char* base = static_cast<char*>(workspace(merge + max_tables_bytes(B, CO, CI, KE), st));
     if (!base) return SD_ERR_HIP;
     if (K && (rc = queue_max_cols(a, K, B, CO, CI, base + merge, st))) return rc;
     rc = run_chunk_pos<LinfChunk>(a, false, st, base, merge);
@@ -287,7 +316,7 @@ extern "C" int sd_masked_inf_dist_forward(const float* input, const float* weigh
         const size_t mask_bytes = ((size_t)(xrows + wrows) * nchunks * 4 + 255) / 256 * 256;
         const int KE = max_cols_eligible(a, (float)a.t16 / 65536.f, B, CO, CI, G, HW);
         K = max_cols_wanted(a, KE, kHintSiteMasked, B, CO, CI, st);
-        char* base = static_cast<char*>(workspace(packed_bytes + mask_bytes + (KE ? max_cols_workspace(B, CO, CI, KE) : 0), st));
+        char* base = static_cast<char*>(workspace(packed_bytes + mask_bytes + (KE ? max_tables_bytes(B, CO, CI, KE) : 0), st));
         if (!base) return SD_ERR_HIP;
         tables = base + packed_bytes + mask_bytes;
         uint32_t* xm = reinterpret_cast<uint32_t*>(base + packed_bytes);

@@ -286,7 +286,7 @@ float sd_last_forward_kernel_ms(void) {
 float sd_last_forward_term_share(sd_stream_t stream) {
     const sd::TermNote n = sd::g_term_note;
     if (n.kind == 0 || !n.counts) return 1.f;
-    unsigned long long c[3] = {0ull, 0ull, 0ull};
+    unsigned long long c[4] = {0ull, 0ull, 0ull, 0ull};
     // waits for the stream, so the call that left the counters has run and nothing has overwritten them yet
     if (hipMemcpyAsync(c, n.counts, sizeof(c), hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)) != hipSuccess ||
         hipStreamSynchronize(static_cast<hipStream_t>(stream)) != hipSuccess) {
@@ -294,6 +294,7 @@ float sd_last_forward_term_share(sd_stream_t stream) {
         return -1.f;
     }
     if (n.kind == 1) return c[1] != 0ull ? 1.f : (float)((double)c[0] / n.denom0);
+    if (n.kind == 3) return c[1] != 0ull ? 1.f : c[2] != 0ull ? (float)((double)c[0] / n.denom0) : (float)((double)c[3] / n.denom1);
     if (c[2] != 0ull) return 1.f;
     return c[0] <= n.limit0 ? (float)((double)c[0] / n.denom0) : (float)((double)c[1] / n.denom1);
 }

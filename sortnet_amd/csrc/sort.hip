@@ -3,6 +3,7 @@
 #include "fwd_tile.h"
 #include "fwd_args.h"
 #include "sort_cols.h"
+#include "row_cands.h"
 #include <atomic>
 
 using namespace sd;
@@ -155,19 +156,46 @@ static bool sort_cols_ok(const FwdArgs& a, int site, int B, int CO, int CI, hipS
 }
 // after the every-term kernels have been queued behind the table kernel
 static void sort_cols_report(const FwdArgs& a, int site, int B, int CO, int CI, hipStream_t st) {
-    if (g_sort_density.load(std::memory_order_relaxed) < 0.f && a.gate) hint_record(site, a.w, B, CO, CI, a.gate + 1, st);
+    if (g_sort_density.load(std::memory_order_relaxed) < 0.f && a.gate) hint_record(site, a.w, B, CO, CI, a.gate, st);
 }
 
-// `ws`: sort_cols_workspace() bytes.  The gate it leaves in `a` points into `ws`: the kernels queued behind it must
+// Largest share of marked (tile of 128 weight rows, batch row, input) triples at which the kernel of the tables per
+// batch row runs.  Measured per 512 x 5120 x 5120 layer at K = 10 on inputs in [0, 1] against weights ~ N(0, 1/N)
+// (7.2 % marked): values 0.83 ms against 1.9 ms for every term, interval bounds 1.35 against 3.3, values with positions
+// 2.1 against 2.6; 0.2 ms of that are tables and staging, the rest grows with the marks.
+constexpr float kSortRowsCap = 0.12f;
+
+// bytes of both tables' workspace for one call: per weight row first (with the probe and the counter the per-batch-row
+// tables read), per batch row behind it
+static size_t sort_tables_bytes(int form, int B, int CO, int CI, int K) {
+    const size_t cols = (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256;
+    return cols + (row_cands_supported(form, K) ? (row_cands_workspace(form, B, CO, CI, K) + 255) / 256 * 256 : 0);
+}
+
+// `ws`: sort_tables_bytes() bytes.  The gate it leaves in `a` points into `ws`: the kernels queued behind it must
 // not be given memory that overlaps it, and `ws` must stay allocated until they have run (one workspace request
-// per call, carved by the caller).
-static int queue_sort_cols(FwdArgs& a, const float* xl, const float* xu, const float* w, int B, int CO, int CI, float q,
-                           int K, float* outL, float* outU, int* pos, void* ws, hipStream_t st) {
+// per call, carved by the caller).  Afterwards a.gate[0] is non-zero when the every-term kernels are to run.
+static int queue_sort_cols(FwdArgs& a, int form, const float* xl, const float* xu, const float* w, int B, int CO, int CI,
+                           float q, int K, float* outL, float* outU, int* pos, void* ws, hipStream_t st) {
     const float density = g_sort_density.load(std::memory_order_relaxed);
     const float cap = density > 0.f ? density : kSortColsCap;
     int rc = sort_cols_forward(xl, xu, w, B, CO, CI, q, K, outL, outU, pos, ws, cap, &a.gate, &a.gate_limit, st);
     a.gate_above = 1;
-    return rc;
+    if (rc || !row_cands_supported(form, K)) {
+        // the every-term kernels read the flag behind the counter, as with both tables
+        if (!rc) { a.gate = a.gate + 1; a.gate_limit = 0ull; }
+        return rc;
+    }
+    const unsigned long long* col_count = a.gate;
+    char* rows_ws = static_cast<char*>(ws) + (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256;
+    const unsigned long long* every = nullptr;
+    rc = row_cands_forward(form, xl, xu, w, nullptr, nullptr, B, CO, CI, q, K, outL, outU, pos, rows_ws,
+                           density > 0.f ? density : kSortRowsCap, sort_cols_probe_sums(col_count), col_count, &every, st);
+    if (rc) return rc;
+    a.gate = every;
+    a.gate_limit = 0ull;
+    note_term_counts(every - 1, 3, (double)((CO + 127) / 128) * B * CI, (double)((B + 127) / 128) * CO * CI, 0ull);
+    return SD_OK;
 }
 
 extern "C" int sd_set_sort_candidate_density(float density) {
@@ -198,14 +226,14 @@ extern "C" int sd_sort_neuron_forward_nograd(const float* input, const float* we
     const bool cols = elig && sort_cols_ok(a, kHintSiteSort, B, CO, CI, st);
     // one request for both users of the workspace: the tables (with the counter the gates read) first, the key
     // lists of the two-level path behind them
-    const size_t tbytes = elig ? (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256 : 0;
+    const size_t tbytes = elig ? sort_tables_bytes(kRowsSortValues, B, CO, CI, K) : 0;
     char* base = nullptr;
     if (elig || two) {
         base = static_cast<char*>(workspace(tbytes + (two ? two_level_bytes(a, K) : 0), st));
         if (!base) return SD_ERR_HIP;
     }
     int* keys = reinterpret_cast<int*>(base + tbytes);
-    if (cols && (rc = queue_sort_cols(a, input, nullptr, weight, B, CO, CI, q, K, nullptr, output, nullptr, base, st))) return rc;
+    if (cols && (rc = queue_sort_cols(a, kRowsSortValues, input, nullptr, weight, B, CO, CI, q, K, nullptr, output, nullptr, base, st))) return rc;
     rc = SD_ERR_ARG;
     switch (K) {
 #define X(k) case k: if (k <= 12 && two) rc = run_two_level<(k <= 12 ? k : 2), true>(a, small, keys, st); \
@@ -235,14 +263,14 @@ extern "C" int sd_sort_neuron_forward(const float* input, const float* weight,
     const bool elig = sort_cols_eligible(a, B, CO, CI, G, HW);
     const bool cols = elig && sort_cols_ok(a, kHintSiteSortPos, B, CO, CI, st);
     // one request for both users of the workspace, as in sd_sort_neuron_forward_nograd
-    const size_t tbytes = elig ? (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256 : 0;
+    const size_t tbytes = elig ? sort_tables_bytes(kRowsSortPos, B, CO, CI, K) : 0;
     char* base = nullptr;
     if (elig || two) {
         base = static_cast<char*>(workspace(tbytes + (two ? two_level_bytes(a, K) : 0), st));
         if (!base) return SD_ERR_HIP;
     }
     int* keys = reinterpret_cast<int*>(base + tbytes);
-    if (cols && (rc = queue_sort_cols(a, input, nullptr, weight, B, CO, CI, q, K, nullptr, output, pos, base, st))) return rc;
+    if (cols && (rc = queue_sort_cols(a, kRowsSortPos, input, nullptr, weight, B, CO, CI, q, K, nullptr, output, pos, base, st))) return rc;
     rc = SD_ERR_ARG;
     switch (K) {
 #define X(k) case k: if (k <= 12 && two) rc = run_two_level<(k <= 12 ? k : 2), false>(a, few_tiles(a, 32, 64), keys, st); \
@@ -271,9 +299,9 @@ extern "C" int sd_bound_sort_neuron_forward(const float* inputL, const float* in
     const bool elig = sort_cols_eligible(a, B, CO, CI, G, HW);
     const bool cols = elig && sort_cols_ok(a, kHintSiteBoundSort, B, CO, CI, st);
     if (elig) {
-        void* ws = workspace(sort_cols_workspace(B, CO, CI, K), st);   // the only request of this call
+        void* ws = workspace(sort_tables_bytes(kRowsSortInterval, B, CO, CI, K), st);   // the only request of this call
         if (!ws) return SD_ERR_HIP;
-        if (cols && (rc = queue_sort_cols(a, inputL, inputU, weight, B, CO, CI, q, K, outputL, outputU, nullptr, ws, st))) return rc;
+        if (cols && (rc = queue_sort_cols(a, kRowsSortInterval, inputL, inputU, weight, B, CO, CI, q, K, outputL, outputU, nullptr, ws, st))) return rc;
     }
     rc = SD_ERR_ARG;
     switch (K) {

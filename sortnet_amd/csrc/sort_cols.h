@@ -30,6 +30,11 @@ int sort_cols_forward(const float* xl, const float* xu, const float* w, int B, i
                       float* outL, float* outU, int* pos, void* ws, float density, const unsigned long long** gate,
                       unsigned long long* gate_limit, hipStream_t st);
 
+// The two sums of the probe that sort_cols_forward / max_cols_forward leave behind the counter words *gate points at
+// (widths of the input columns over all batch tiles; widths of the same columns over 16 weight rows), for the tables
+// of the other orientation (row_cands.h), which are queued behind these and decide from the same sums.
+inline const float* sort_cols_probe_sums(const unsigned long long* gate) { return reinterpret_cast<const float*>(gate + 2); }
+
 // l-inf distance forward (maximum and, if pos is not null, its position) from the same kind of table, optionally
 // under the factored mask (xkeep: one word per (batch row, 32 inputs), wkeep: per (weight row, 32 inputs); both or
 // neither).  K = max_cols_depth(probability that a row keeps an input): how many inputs the bound of a weight row

@@ -7,7 +7,8 @@ the oracle's bits either way (core/cuda/inf_dist_cuda.cu:110-212 semantics: the 
 floor with position 0 when nothing exceeds it): the tests force either side (density 1 / 0) and the built-in limit,
 on batches whose rows are alike against weights of unit scale (the table marks little), on unrelated rows, on grid
 data with many exact ties, and under the mask with a shallow bound so that some outputs are recomputed from every
-input."""
+input.  Inputs in [0, 1] against small weights ("images", "image_ties") are the case of the other table orientation:
+per batch row and tile of 128 weight rows, where the batch row decides which inputs can hold a maximum."""
 import numpy as np
 import pytest
 import torch
@@ -41,6 +42,9 @@ def _data(B, CI, CO, kind, seed):
     elif kind == "images":
         x = torch.rand(B, CI, 1, generator=g)
         w = torch.randn(CO, CI, generator=g) * CI ** -0.5
+    elif kind == "image_ties":      # the batch decides, and many terms are equal: 17 input levels, 9 weight levels
+        x = torch.round(torch.rand(B, CI, 1, generator=g) * 16) / 16
+        w = torch.round(torch.randn(CO, CI, generator=g) * 0.03 * 64) / 64
     elif kind == "ties":
         x = torch.round(torch.randn(B, CI, 1, generator=g) * 0.2 * 4) / 4
         w = torch.round(torch.randn(CO, CI, generator=g) * 4) / 4
@@ -50,7 +54,14 @@ def _data(B, CI, CO, kind, seed):
     return x.contiguous(), w.contiguous()
 
 
-def _check_plain(oracle, x, w, tag):
+def _served_from_tables(expect, tag):
+    """With the limit forced to 1 on data where the batch decides, a table kernel must have served the call."""
+    from sortnet_amd import _lib
+    if expect:
+        assert _lib.last_forward_term_share() < 1.0, tag
+
+
+def _check_plain(oracle, x, w, tag, expect_tables=False):
     from sortnet_amd import ext
     dev = _dev()
     B, CO = x.shape[0], w.shape[0]
@@ -58,14 +69,16 @@ def _check_plain(oracle, x, w, tag):
     y = torch.full((B, CO, 1), float("nan"), device=dev)
     pos = torch.full((B, CO, 1), -7, device=dev, dtype=torch.int32)
     ext.inf_dist_forward(x.to(dev), w.to(dev), y, pos, 1)
+    _served_from_tables(expect_tables, tag)
     assert np.array_equal(y.cpu().numpy(), ry), tag
     assert np.array_equal(pos.cpu().numpy(), rpos), tag
     y2 = torch.full((B, CO, 1), float("nan"), device=dev)
     ext.inf_dist_forward_nograd(x.to(dev), w.to(dev), y2, 1)
+    _served_from_tables(expect_tables, tag)
     assert np.array_equal(y2.cpu().numpy(), ry), tag
 
 
-def _check_masked(oracle, x, w, q, seed, tag):
+def _check_masked(oracle, x, w, q, seed, tag, expect_tables=False):
     from sortnet_amd import ext
     dev = _dev()
     B, CO = x.shape[0], w.shape[0]
@@ -73,6 +86,7 @@ def _check_masked(oracle, x, w, q, seed, tag):
     y = torch.full((B, CO, 1), float("nan"), device=dev)
     pos = torch.full((B, CO, 1), -7, device=dev, dtype=torch.int32)
     ext.masked_inf_dist_forward(x.to(dev), w.to(dev), y, pos, 1, q, seed, ext.MASK_FACTORED)
+    _served_from_tables(expect_tables, tag)
     assert np.array_equal(y.cpu().numpy(), ry), tag
     assert np.array_equal(pos.cpu().numpy(), rpos), tag
     y2 = torch.full((B, CO, 1), float("nan"), device=dev)
@@ -88,9 +102,11 @@ SHAPES = [(70, 96, 64), (33, 2048, 300), (130, 1024, 513), (1, 32, 1), (257, 320
 def test_linf_candidate_kernels_match_oracle(oracle, knobs, dens, B, CI, CO):
     """Ragged batch tiles and weight rows, rows of more than 64 chunks (several loads of table words per row)."""
     knobs(dens)
-    for kind in ("rows_alike", "random", "images", "ties"):
+    for kind in ("rows_alike", "random", "images", "ties", "image_ties"):
         x, w = _data(B, CI, CO, kind, B + CI)
-        _check_plain(oracle, x, w, "dens=%g %s" % (dens, kind))
+        # inputs in [0, 1] against small weights: the tables per batch row serve (rows of at least a few chunks)
+        expect = dens == 1.0 and kind in ("images", "image_ties") and CI >= 160 and B > 1
+        _check_plain(oracle, x, w, "dens=%g %s" % (dens, kind), expect)
 
 
 @pytest.mark.parametrize("dens,depth", [(1.0, 0), (1.0, 8), (0.0, 0), (-1.0, 0)])
@@ -99,10 +115,11 @@ def test_masked_candidate_kernels_match_oracle(oracle, knobs, dens, depth, B, CI
     """Factored mask at q = 0.3, 0.75 and 1.  Depth 8 at q = 0.3: a row keeps none of the eight inputs the bound
     rests on about once in 600 outputs, so many wavefronts walk their weight row a second time over every input."""
     knobs(dens, depth)
-    for kind in ("rows_alike", "random", "ties"):
+    for kind in ("rows_alike", "random", "ties", "images", "image_ties"):
         for q, seed in ((0.3, 5), (0.75, 77), (1.0, 3)):
             x, w = _data(B, CI, CO, kind, B + CI + 1)
-            _check_masked(oracle, x, w, q, seed, "dens=%g depth=%d %s q=%g" % (dens, depth, kind, q))
+            expect = dens == 1.0 and kind in ("images", "image_ties") and CI >= 160 and B > 1
+            _check_masked(oracle, x, w, q, seed, "dens=%g depth=%d %s q=%g" % (dens, depth, kind, q), expect)
 
 
 def test_linf_candidate_kernels_at_layer_size(knobs):

@@ -34,16 +34,23 @@ def _data(B, CI, CO, kind, seed):
     g = torch.Generator().manual_seed(seed)
     if kind == "rows_alike":
         x = torch.randn(1, CI, 1, generator=g) * 0.3 + torch.randn(B, CI, 1, generator=g) * 0.05
-    elif kind == "images":
+    elif kind in ("images", "pixels", "pixel_ties"):
         x = torch.rand(B, CI, 1, generator=g)
     else:
         x = torch.randn(B, CI, 1, generator=g)
-    r = torch.rand(B, CI, 1, generator=g) * 0.05
+    r = torch.rand(B, CI, 1, generator=g) * (0.01 if kind.startswith("pixels") else 0.05)
+    if kind == "pixel_ties":
+        x = torch.round(x * 16) / 16
+        r = torch.full_like(x, 1.0 / 64)
     xl, xu = (x - r).contiguous(), (x + r).contiguous()
     if kind == "inverted":
         m = torch.rand(B, CI, 1, generator=g) < 0.1
         xl, xu = torch.where(m, xu, xl).contiguous(), torch.where(m, xl, xu).contiguous()
     w = torch.randn(CO, CI, generator=g).contiguous()
+    if kind == "pixels":            # inputs in [0, 1] against small weights: the batch row decides where the largest terms sit
+        w = (w * CI ** -0.5).contiguous()
+    if kind == "pixel_ties":        # the same with 17 input levels and a few weight levels: many equal terms
+        w = (torch.round(w * 0.03 * 64) / 64).contiguous()
     if kind == "ties":
         x, w = torch.round(x * 4) / 4, torch.round(w * 4) / 4
         xl, xu = x - 0.25, x + 0.25
@@ -66,12 +73,15 @@ def _run(x, xl, xu, w, q, K):
     return y.cpu().numpy(), yl.cpu().numpy(), yu.cpu().numpy(), yp.cpu().numpy(), pos.cpu().numpy()
 
 
-def _check(oracle, density, dens, x, xl, xu, w, q, K, tag):
+def _check(oracle, density, dens, x, xl, xu, w, q, K, tag, expect_tables=False):
     """Against the oracle at the sort neuron's bar (rel 1e-5), and bit for bit against the every-term kernels."""
     ry, rpos = oracle.sort_neuron_forward(x.numpy(), w.numpy(), q, K)
     rl, ru = oracle.bound_sort_neuron_forward(xl.numpy(), xu.numpy(), w.numpy(), q, K)
     density(dens)
     got = _run(x, xl, xu, w, q, K)
+    if expect_tables:   # (the last call of _run: values with positions)
+        from sortnet_amd import _lib
+        assert _lib.last_forward_term_share() < 1.0, tag
     for g, r in zip(got[:4], (ry, rl, ru, ry)):
         np.testing.assert_allclose(g, r, rtol=RTOL, err_msg=tag)
     assert np.array_equal(got[4], rpos), tag   # positions: exact, ties included
@@ -87,16 +97,27 @@ def _check(oracle, density, dens, x, xl, xu, w, q, K, tag):
 def test_sort_candidate_kernels_match_oracle(oracle, density, dens, B, CI, CO):
     """Ragged batch tiles (B not a multiple of 128) and weight rows (CO not a multiple of 32 / 64 / 128), rows of
     more than 32 chunks (several batches of marks per row), rows shorter than K."""
-    for kind in ("rows_alike", "random", "inverted", "images", "ties"):
+    for kind in ("rows_alike", "random", "inverted", "images", "ties", "pixels", "pixel_ties"):
         for q, K in ((0.3, 10), (0.75, 4)):
             x, xl, xu, w = _data(B, CI, CO, kind, B + CI)
-            _check(oracle, density, dens, x, xl, xu, w, q, K, "dens=%g %s K=%d" % (dens, kind, K))
+            # (the bound of a batch row rests on the K largest of its per-chunk maxima: rows of at least K chunks)
+            expect = dens == 1.0 and kind.startswith("pixel") and CI >= 32 * K and B > 1
+            _check(oracle, density, dens, x, xl, xu, w, q, K, "dens=%g %s K=%d" % (dens, kind, K), expect)
 
 
 @pytest.mark.parametrize("K", [2, 3, 7, 13, 16, 25])
 def test_sort_candidate_kernels_every_k(oracle, density, K):
     x, xl, xu, w = _data(140, 512, 100, "rows_alike", K)
     _check(oracle, density, 1.0, x, xl, xu, w, 0.4, K, "K=%d" % K)
+
+
+@pytest.mark.parametrize("K", [2, 3, 5, 6, 8, 9, 11, 13, 16, 20, 21, 25])
+def test_sort_row_table_kernels_every_k(oracle, density, K):
+    """The tables per batch row: every number of batch rows per wavefront that the top-K lists' size selects, for
+    values, interval bounds and positions (beyond K = 20 only the values have such a kernel)."""
+    for kind in ("pixels", "pixel_ties"):
+        x, xl, xu, w = _data(150, 1024, 200, kind, K)
+        _check(oracle, density, 1.0, x, xl, xu, w, 0.4, K, "%s K=%d" % (kind, K), expect_tables=K <= 12)
 
 
 def test_sort_candidate_kernels_at_layer_size(density):
