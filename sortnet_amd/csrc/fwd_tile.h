@@ -680,6 +680,16 @@ struct LinfChunkPacked : PolicyBase {
     static __device__ __forceinline__ void store(Acc&, const FwdArgs&, size_t, int split = 0) {}
 };
 
+// |d| when the term's random byte is below the threshold (the term is kept), else 0.  Written as arithmetic on the
+// sign of byte - t8 rather than as a compare and a select per term: the compiler still emits compares and selects from
+// it, but schedules them 5 % faster than from the conditional expressions (2.12 -> 2.00 ms per 512 x 5120 x 5120 layer).
+// Measured and not kept: 24-bit multiplies in the hash (full vector rate instead of a quarter: no change, the kernel is
+// not bound by its multiplies) and the same masking forced through inline assembly (3 % slower).
+__device__ __forceinline__ float masked_abs(float d, uint32_t byte, uint32_t t8) {
+    const uint32_t keep = (uint32_t)(((int)byte - (int)t8) >> 31);
+    return __uint_as_float(__float_as_uint(d) & keep & 0x7fffffffu);
+}
+
 // the per-term masked neuron with the same chunk tracking
 struct MaskedTermChunk : PolicyBase {
     static constexpr int PIPE_WAVES = 2;   // hash-bound: timings were flat over 2..4 waves and 4x8 / 4x4 / 2x8 tiles
@@ -690,14 +700,10 @@ struct MaskedTermChunk : PolicyBase {
     }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
                                                  const float4& w, int n, int) {
-        uint32_t word = rng_word(A.key, (uint32_t)n >> 2);
-        float d0 = (word & 0xffu) < a.t8 ? x.x - w.x : 0.f;
-        float d1 = ((word >> 8) & 0xffu) < a.t8 ? x.y - w.y : 0.f;
-        float d2 = ((word >> 16) & 0xffu) < a.t8 ? x.z - w.z : 0.f;
-        float d3 = (word >> 24) < a.t8 ? x.w - w.w : 0.f;
+        const uint32_t word = rng_word(A.key, (uint32_t)n >> 2);
         float v = A.cm;
-        v = fmaxf(fmaxf(v, fabsf(d0)), fabsf(d1));
-        v = fmaxf(fmaxf(v, fabsf(d2)), fabsf(d3));
+        v = fmaxf(fmaxf(v, masked_abs(x.x - w.x, word & 0xffu, a.t8)), masked_abs(x.y - w.y, (word >> 8) & 0xffu, a.t8));
+        v = fmaxf(fmaxf(v, masked_abs(x.z - w.z, (word >> 16) & 0xffu, a.t8)), masked_abs(x.w - w.w, word >> 24, a.t8));
         A.cm = v;
     }
     static __device__ __forceinline__ void chunk_end(Acc& A, const FwdArgs&, int, int k0) {
@@ -718,14 +724,10 @@ struct MaskedTermMax : PolicyBase {
     }
     static __device__ __forceinline__ void step4(Acc& A, const FwdArgs& a, const float4& x, const float4&,
                                                  const float4& w, int n, int) {
-        uint32_t word = rng_word(A.key, (uint32_t)n >> 2);
-        float d0 = (word & 0xffu) < a.t8 ? x.x - w.x : 0.f;
-        float d1 = ((word >> 8) & 0xffu) < a.t8 ? x.y - w.y : 0.f;
-        float d2 = ((word >> 16) & 0xffu) < a.t8 ? x.z - w.z : 0.f;
-        float d3 = (word >> 24) < a.t8 ? x.w - w.w : 0.f;
+        const uint32_t word = rng_word(A.key, (uint32_t)n >> 2);
         float v = A.v;
-        v = fmaxf(fmaxf(v, fabsf(d0)), fabsf(d1));
-        v = fmaxf(fmaxf(v, fabsf(d2)), fabsf(d3));
+        v = fmaxf(fmaxf(v, masked_abs(x.x - w.x, word & 0xffu, a.t8)), masked_abs(x.y - w.y, (word >> 8) & 0xffu, a.t8));
+        v = fmaxf(fmaxf(v, masked_abs(x.z - w.z, (word >> 16) & 0xffu, a.t8)), masked_abs(x.w - w.w, word >> 24, a.t8));
         A.v = v;
     }
     static __device__ __forceinline__ void store(Acc& A, const FwdArgs& a, size_t o, int split = 0) {

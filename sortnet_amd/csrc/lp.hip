@@ -676,8 +676,13 @@ extern "C" int sd_norm_dist_forward(const float* input, const float* weight,
     static const int kTb42[] = {4, 2};
     const bool small = w_index_ci || w_index_co || pick_tb(a, kTb42, 2, 128) == 2;
     const bool online = p > 10.f;   // core/cuda/norm_dist.cpp:4,51-55
-    a.skip_thr = lp_skip_threshold(1e-6f / (float)a.CIg, p, (a.fast_x && a.fast_w && !w_index_co) ? kLpSkipFrom : kLpSkipFromOnline);
-    if (online && a.fast_x && a.fast_w && !w_index_co) return lp_forward_max_first(a, small, st);
+    const bool lists = w_index_ci || w_index_co;
+    // p > 10: the exact maximum per output first, then one pass of sums relative to it.  On the vector path, and with
+    // index lists as well: there the gather kernel's two passes over every LDS chunk (the online form) cost more than
+    // a second launch (index-list training step at keep 0.75: 17.6 -> 13.7 ms at p = 256, 20.4 -> 20.1 at p = 24).
+    const bool max_first = online && ((a.fast_x && a.fast_w && !w_index_co) || (lists && a.HW == 1));
+    a.skip_thr = lp_skip_threshold(1e-6f / (float)a.CIg, p, max_first ? kLpSkipFrom : kLpSkipFromOnline);
+    if (max_first) return lp_forward_max_first(a, small, st);
     if ((rc = lp_split_setup(a, small ? 32 : 64, 128, online, st))) return rc;
     if (!online) {
         int ip = int_power(p);

@@ -391,7 +391,7 @@ def test_norm_dist(oracle, p, B, CI, CO, G, HW):
     np.testing.assert_allclose(y3.cpu().numpy(), ry, rtol=RTOL)
 
 
-@pytest.mark.parametrize("p", [8.0, 20.0, 300.0])
+@pytest.mark.parametrize("p", [8.0, 20.0, 24.0, 64.0, 256.0, 300.0])
 @pytest.mark.parametrize("B,CI,CO,G,ci_n,co_n", [(70, 96, 64, 1, 29, 21), (40, 64, 48, 2, 12, 8), (96, 1024, 300, 1, 701, 150)])
 def test_norm_dist_index_lists(oracle, p, B, CI, CO, G, ci_n, co_n):
     from sortnet_amd import ext
