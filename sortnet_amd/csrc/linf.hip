@@ -89,7 +89,7 @@ static int queue_max_cols(FwdArgs& a, int K, int B, int CO, int CI, void* ws, hi
     char* rows_ws = static_cast<char*>(ws) + (max_cols_workspace(B, CO, CI, K) + 255) / 256 * 256;
     const unsigned long long* every = nullptr;
     rc = row_cands_forward(kRowsMax, a.x0, nullptr, a.w, xkeep, wkeep, B, CO, CI, 0.f, K, nullptr, a.y0, a.p0, rows_ws,
-                           density > 0.f ? density : kMaxRowsCap, sort_cols_probe_sums(col_count), col_count, &every, st);
+                           density > 0.f ? density : kMaxRowsCap, density > 0.f, sort_cols_probe_sums(col_count), col_count, &every, st);
     if (rc) return rc;
     a.gate = every;
     a.gate_limit = 0ull;

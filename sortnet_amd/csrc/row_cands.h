@@ -39,7 +39,9 @@ bool row_cands_supported(int form, int K);
 //   col_stat / col_count: the probe sums and the counter words that sort_cols_forward / max_cols_forward left for
 //     the same call (col_count[1] != 0: the per-weight-row tables are above their limit).  Everything here returns
 //     at once unless the probe says that the batch decides.
-//   density: largest share of marked (tile of weight rows, batch row, input) triples at which the main kernel runs.
+//   density: largest share of marked (tile of weight rows, batch row, input) triples at which the main kernel runs;
+//     forced: the caller's limit was set by hand (then the l-inf form builds its tables whenever the batch decides,
+//     instead of only where the probe promises very few marks).
 //   *every: device word that is non-zero when neither table serves the call, i.e. when the kernels that evaluate
 //     every term are to run (their gate: run when *every > 0); (*every)[-1] holds the marks of this table,
 //     (*every)[1] is non-zero when this table's kernel runs, (*every)[2] the marks per weight row (copied).
@@ -47,7 +49,7 @@ bool row_cands_supported(int form, int K);
 //   outL / outU / pos as in sort_cols_forward / max_cols_forward (values go to outU).
 int row_cands_forward(int form, const float* xl, const float* xu, const float* w, const uint32_t* xkeep,
                       const uint32_t* wkeep, int B, int CO, int CI, float q, int K, float* outL, float* outU, int* pos,
-                      void* ws, float density, const float* col_stat, const unsigned long long* col_count,
+                      void* ws, float density, bool forced, const float* col_stat, const unsigned long long* col_count,
                       const unsigned long long** every, hipStream_t st);
 
 }  // namespace sd

@@ -73,9 +73,12 @@ __device__ __forceinline__ void repair(float& l, float& u) {
 // The probe of sort_cols.hip (same constant): the batch rows of a tile differ by more than 2.5 times what 16 entries
 // of a weight column do.  stat[0] = widths of the input columns over all batch tiles, stat[1] = widths of the same
 // columns over 16 weight rows.
-constexpr float kProbeRatio = 2.5f;
-__device__ __forceinline__ bool rows_decide(const float* stat, int S) {
-    return stat[0] > kProbeRatio * (float)S * stat[1];
+// `ratio` is kProbeRatio for the sort-neuron forms.  The l-inf form asks for more (kProbeRatioMax): its kernel only pays
+// below about 4 % of marks, and on inputs spread evenly over their range the marked share is about 1.5 / (that ratio), so
+// its tables are not even built unless the probe promises that few.
+constexpr float kProbeRatio = 2.5f, kProbeRatioMax = 40.f;
+__device__ __forceinline__ bool rows_decide(const float* stat, int S, float ratio) {
+    return stat[0] > ratio * (float)S * stat[1];
 }
 
 // Top-K lists hold their values ascending (res[K-1] largest) and start at 0: new[k] = max(res[k], min(res[k+1], v))
@@ -100,8 +103,8 @@ __device__ __forceinline__ void static_for(F&& f, std::integer_sequence<int, R..
 template <bool WMASK>
 __global__ void __launch_bounds__(256) rc_range_kernel(const float* __restrict__ w, const uint32_t* __restrict__ wkeep,
                                                        int M, int N, int S, float* __restrict__ wr,
-                                                       const float* __restrict__ stat) {
-    if (!rows_decide(stat, S)) return;
+                                                       const float* __restrict__ stat, float ratio) {
+    if (!rows_decide(stat, S, ratio)) return;
     __shared__ float part[4][3][64];
     const int nl = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int n = blockIdx.x * 64 + nl, t = blockIdx.y;
@@ -144,8 +147,8 @@ template <int K, bool IV, bool XMASK>
 __global__ void __launch_bounds__(256) rc_low_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
                                                      const uint32_t* __restrict__ xkeep, const float* __restrict__ wr,
                                                      int B, int N, int T, int Bp, int S, float* __restrict__ lists,
-                                                     const float* __restrict__ stat) {
-    if (!rows_decide(stat, S)) return;
+                                                     const float* __restrict__ stat, float ratio) {
+    if (!rows_decide(stat, S, ratio)) return;
     __shared__ __attribute__((aligned(16))) float lt[64][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float ut[IV ? 64 : 1][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float ws[4][2][kChunk];
@@ -230,8 +233,8 @@ __global__ void __launch_bounds__(256) rc_low_kernel(const float* __restrict__ x
 // K-th largest of the slices' lists (0 when fewer than K lower bounds are positive); grid.y = T * nw
 template <int K>
 __global__ void __launch_bounds__(256) rc_merge_kernel(const float* __restrict__ lists, int slices, int Bp, int nw, int S,
-                                                       float* __restrict__ low, const float* __restrict__ stat) {
-    if (!rows_decide(stat, S)) return;
+                                                       float* __restrict__ low, const float* __restrict__ stat, float ratio) {
+    if (!rows_decide(stat, S, ratio)) return;
     const int b = blockIdx.x * 256 + threadIdx.x;
     if (b >= Bp) return;
     const int t = blockIdx.y / nw, which = blockIdx.y % nw;
@@ -255,8 +258,8 @@ __global__ void __launch_bounds__(256) rc_bits_kernel(const float* __restrict__ 
                                                       const uint32_t* __restrict__ xkeep, const float* __restrict__ wr,
                                                       const float* __restrict__ low, int B, int N, int T, int Bp, int S,
                                                       uint32_t* __restrict__ bits, uint32_t* __restrict__ partial,
-                                                      const float* __restrict__ stat) {
-    if (!rows_decide(stat, S)) return;
+                                                      const float* __restrict__ stat, float ratio) {
+    if (!rows_decide(stat, S, ratio)) return;
     __shared__ __attribute__((aligned(16))) float lt[64][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float ut[IV ? 64 : 1][kChunk + 4];
     __shared__ __attribute__((aligned(16))) float ws[4][2][kChunk];
@@ -344,9 +347,10 @@ __global__ void __launch_bounds__(256) rc_bits_kernel(const float* __restrict__ 
 __global__ void __launch_bounds__(1024) rc_sum_kernel(const uint32_t* __restrict__ partial, size_t n,
                                                       unsigned long long* __restrict__ count,
                                                       const unsigned long long* __restrict__ col_count,
-                                                      const float* __restrict__ stat, int S, unsigned long long limit) {
+                                                      const float* __restrict__ stat, int S, unsigned long long limit,
+                                                      float ratio) {
     __shared__ unsigned long long acc[1024];
-    const bool rows = rows_decide(stat, S);
+    const bool rows = rows_decide(stat, S, ratio);
     unsigned long long s0 = 0;
     if (rows) for (size_t i = threadIdx.x; i < n; i += 1024) s0 += partial[i];
     acc[threadIdx.x] = s0;
@@ -401,8 +405,10 @@ __global__ void __launch_bounds__(64 * kWaves, 1) rc_main_kernel(MainArgs a) {
     uint32_t* wb = reinterpret_cast<uint32_t*>(smem + 2 * TILE);   // [kSeg][ROWS]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // this wavefront's list of the marked inputs of one row and stage: (input within the stage, value[, upper value], -)
-    float4* marks = reinterpret_cast<float4*>(wb + kSeg * ROWS) + wave * kStage;
+    // this wavefront's lists of the marked inputs of its rows in one stage (two entries past a full list are read)
+    struct Entry { int i; float l, u; };
+    constexpr int kMarkRow = kStage + 2;
+    Entry* marks = reinterpret_cast<Entry*>(wb + kSeg * ROWS) + wave * (TR * kMarkRow);
     const int B = a.B, Bp = a.Bp, M = a.M, N = a.N, NCH = N / kChunk;
     const int rows = a.rows, BG = (B + rows - 1) / rows;
     // Workgroups go to the chip's eight dies in turn, each with a cache of its own: consecutive (tile, batch rows)
@@ -534,41 +540,44 @@ __global__ void __launch_bounds__(64 * kWaves, 1) rc_main_kernel(MainArgs a) {
             }
         }
     };
-    // A row's marks of the stage are first compacted by the lanes themselves: lane i, which holds input i, finds its
-    // place among the marked lanes with a bit count and posts (i, value) in the wavefront's list.  The walk over the
-    // list then costs one broadcast read per four marks and no bit scanning: the scalar unit, which all sixteen
-    // wavefronts share, only keeps the loop's count.
+    // The marks of the wavefront's rows in the stage are first compacted by the lanes themselves: lane i, which holds
+    // input i, finds its place among the marked lanes of a row with a bit count and posts (i, value) in that row's
+    // list.  The walk over a list then costs one broadcast read per mark and no bit scanning (the scalar unit, which
+    // all sixteen wavefronts share, only keeps the loop's count), and it is software-pipelined: while the terms of
+    // mark k are formed, the weights of mark k + 1 and the entry of mark k + 2 are on their way (an entry must have
+    // arrived before its weights can be asked for: two dependent LDS reads per mark otherwise).
     auto compute = [&](int buf, int st, const float (&xl_)[TR], const float (&xu_)[IV ? TR : 1]) __attribute__((always_inline)) {
         const char* W = reinterpret_cast<const char*>(wt(buf) + 2 * lane);
         const uint32_t* words = wb + (2 * st - seg_lo) * ROWS + r_lo;
         uint32_t wa[TR], wc[TR];
         #pragma unroll
         for (int r = 0; r < TR; r++) { wa[r] = words[r < nr ? r : 0]; wc[r] = words[ROWS + (r < nr ? r : 0)]; }
-        static_for([&](auto R) __attribute__((always_inline)) {
-            constexpr int r = decltype(R)::value;
+        int cnt[TR];
+        __builtin_amdgcn_wave_barrier();                 // the walks of the stage before this one have read their entries
+        #pragma unroll
+        for (int r = 0; r < TR; r++) {
             uint32_t mlo = 0u, mhi = 0u;
             if (r < nr) { mlo = (uint32_t)__builtin_amdgcn_readfirstlane(wa[r]); mhi = (uint32_t)__builtin_amdgcn_readfirstlane(wc[r]); }
-            const int cnt = __builtin_popcount(mlo) + __builtin_popcount(mhi);
-            if (cnt == 0) return;
+            cnt[r] = __builtin_popcount(mlo) + __builtin_popcount(mhi);
             const uint32_t mine = ((lane < 32 ? mlo : mhi) >> (lane & 31)) & 1u;
             const int rank = (int)__builtin_amdgcn_mbcnt_hi(mhi, __builtin_amdgcn_mbcnt_lo(mlo, 0u));
-            __builtin_amdgcn_wave_barrier();                 // the walk over the row before this one has read its entries
-            if (mine) marks[rank] = make_float4(__int_as_float(lane), xl_[r], IV ? xu_[IV ? r : 0] : 0.f, 0.f);
-            __builtin_amdgcn_wave_barrier();                 // LDS operations of one wavefront complete in order
-            const int n0 = st * kStage;
-            for (int k = 0; k < cnt; k += 4) {
-                // four marks at a time: their entries, then their weights, all requested before the first term is formed
-                const float4 e0 = marks[k], e1 = marks[k + 1 < cnt ? k + 1 : k], e2 = marks[k + 2 < cnt ? k + 2 : k],
-                             e3 = marks[k + 3 < cnt ? k + 3 : k];
-                const int i0 = __float_as_int(e0.x), i1 = __float_as_int(e1.x), i2 = __float_as_int(e2.x), i3 = __float_as_int(e3.x);
-                const float2 w0 = *reinterpret_cast<const float2*>(W + i0 * (kWRow * 4));
-                const float2 w1 = *reinterpret_cast<const float2*>(W + i1 * (kWRow * 4));
-                const float2 w2 = *reinterpret_cast<const float2*>(W + i2 * (kWRow * 4));
-                const float2 w3 = *reinterpret_cast<const float2*>(W + i3 * (kWRow * 4));
-                term(R, w0, e0.y, e0.z, n0 + i0);
-                if (k + 1 < cnt) term(R, w1, e1.y, e1.z, n0 + i1);
-                if (k + 2 < cnt) term(R, w2, e2.y, e2.z, n0 + i2);
-                if (k + 3 < cnt) term(R, w3, e3.y, e3.z, n0 + i3);
+            if (mine) marks[r * kMarkRow + rank] = Entry{lane, xl_[r], IV ? xu_[IV ? r : 0] : 0.f};
+        }
+        __builtin_amdgcn_wave_barrier();                 // LDS operations of one wavefront complete in order
+        const int n0 = st * kStage;
+        static_for([&](auto R) __attribute__((always_inline)) {
+            constexpr int r = decltype(R)::value;
+            const int total = cnt[r];
+            if (total == 0) return;
+            const Entry* list = marks + r * kMarkRow;
+            // (past the end of the list the entries are stale: their input numbers are masked into the stage, not used)
+            Entry e = list[0], e1 = list[1];
+            float2 ww = *reinterpret_cast<const float2*>(W + (e.i & (kStage - 1)) * (kWRow * 4));
+            for (int k = 0; k < total; k++) {
+                const float2 w1 = *reinterpret_cast<const float2*>(W + (e1.i & (kStage - 1)) * (kWRow * 4));
+                const Entry e2 = list[k + 2];
+                term(R, ww, e.l, e.u, n0 + e.i);
+                e = e1; ww = w1; e1 = e2;
             }
         }, std::make_integer_sequence<int, TR>{});
     };
@@ -704,7 +713,7 @@ inline int rows_per_group(int B, int T, int cap) {
 template <int FORM, int K, int TR, bool POS, bool MASKED>
 int launch_main(MainArgs a, hipStream_t st) {
     constexpr int ROWS = kWaves * TR;
-    constexpr size_t lds = (size_t)(2 * kStage * kWRow + kSeg * ROWS) * 4 + (size_t)kWaves * kStage * 16;
+    constexpr size_t lds = (size_t)(2 * kStage * kWRow + kSeg * ROWS) * 4 + (size_t)kWaves * TR * (kStage + 2) * 12;
     static_assert(lds <= 160 * 1024, "LDS of the main kernel");
     auto kern = rc_main_kernel<FORM, K, TR, POS, MASKED>;
     static bool attr_done = false;   // once per instantiation (benign if two threads both set it)
@@ -740,17 +749,17 @@ int run(const float* xl, const float* xu, const float* w, int B, int M, int N, f
     constexpr bool IV = FORM == kRowsSortInterval;
     const int T = tiles_w(M), Bp = bpad_of(B), NCH = N / kChunk, slices = slices_of(NCH), S = (B + 127) / 128;
     int rc;
-    hipLaunchKernelGGL((rc_range_kernel<false>), dim3((N + 63) / 64, T), dim3(256), 0, st, w, nullptr, M, N, S, c.wr, col_stat);
+    hipLaunchKernelGGL((rc_range_kernel<false>), dim3((N + 63) / 64, T), dim3(256), 0, st, w, nullptr, M, N, S, c.wr, col_stat, kProbeRatio);
     if ((rc = check_launch("rc_range_kernel"))) return rc;
     const dim3 tgrid(Bp / 64, slices, (T + 3) / 4);
-    hipLaunchKernelGGL((rc_low_kernel<K, IV, false>), tgrid, dim3(256), 0, st, xl, xu, nullptr, c.wr, B, N, T, Bp, S, c.lists, col_stat);
+    hipLaunchKernelGGL((rc_low_kernel<K, IV, false>), tgrid, dim3(256), 0, st, xl, xu, nullptr, c.wr, B, N, T, Bp, S, c.lists, col_stat, kProbeRatio);
     if ((rc = check_launch("rc_low_kernel"))) return rc;
     constexpr int nw = IV ? 2 : 1;
-    hipLaunchKernelGGL((rc_merge_kernel<K>), dim3((Bp + 255) / 256, T * nw), dim3(256), 0, st, c.lists, slices, Bp, nw, S, c.low, col_stat);
+    hipLaunchKernelGGL((rc_merge_kernel<K>), dim3((Bp + 255) / 256, T * nw), dim3(256), 0, st, c.lists, slices, Bp, nw, S, c.low, col_stat, kProbeRatio);
     if ((rc = check_launch("rc_merge_kernel"))) return rc;
-    hipLaunchKernelGGL((rc_bits_kernel<IV, false>), tgrid, dim3(256), 0, st, xl, xu, nullptr, c.wr, c.low, B, N, T, Bp, S, c.bits, c.partial, col_stat);
+    hipLaunchKernelGGL((rc_bits_kernel<IV, false>), tgrid, dim3(256), 0, st, xl, xu, nullptr, c.wr, c.low, B, N, T, Bp, S, c.bits, c.partial, col_stat, kProbeRatio);
     if ((rc = check_launch("rc_bits_kernel"))) return rc;
-    hipLaunchKernelGGL(rc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)tgrid.x * tgrid.y * tgrid.z * 4, c.count, col_count, col_stat, S, limit);
+    hipLaunchKernelGGL(rc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)tgrid.x * tgrid.y * tgrid.z * 4, c.count, col_count, col_stat, S, limit, kProbeRatio);
     if ((rc = check_launch("rc_sum_kernel"))) return rc;
     MainArgs a{xl, xu, w, nullptr, nullptr, c.bits, c.low, c.count, c.fix, B, Bp, M, N, 0, q, outL, outU, pos};
     return launch_main<FORM, K, tr_for(FORM, K), false, false>(a, st);
@@ -759,24 +768,24 @@ int run(const float* xl, const float* xu, const float* w, int B, int M, int N, f
 template <int K, bool MASKED>
 int run_max(const float* x, const float* w, const uint32_t* xkeep, const uint32_t* wkeep, int B, int M, int N, float* y,
             int* pos, const Carve& c, unsigned long long limit, const float* col_stat, const unsigned long long* col_count,
-            hipStream_t st) {
+            float ratio, hipStream_t st) {
     const int T = tiles_w(M), Bp = bpad_of(B), NCH = N / kChunk, slices = slices_of(NCH), S = (B + 127) / 128;
     int rc;
-    hipLaunchKernelGGL((rc_range_kernel<MASKED>), dim3((N + 63) / 64, T), dim3(256), 0, st, w, wkeep, M, N, S, c.wr, col_stat);
+    hipLaunchKernelGGL((rc_range_kernel<MASKED>), dim3((N + 63) / 64, T), dim3(256), 0, st, w, wkeep, M, N, S, c.wr, col_stat, ratio);
     if ((rc = check_launch("rc_range_kernel"))) return rc;
     const dim3 tgrid(Bp / 64, slices, (T + 3) / 4);
-    hipLaunchKernelGGL((rc_low_kernel<K, false, MASKED>), tgrid, dim3(256), 0, st, x, nullptr, xkeep, c.wr, B, N, T, Bp, S, c.lists, col_stat);
+    hipLaunchKernelGGL((rc_low_kernel<K, false, MASKED>), tgrid, dim3(256), 0, st, x, nullptr, xkeep, c.wr, B, N, T, Bp, S, c.lists, col_stat, ratio);
     if ((rc = check_launch("rc_low_kernel"))) return rc;
-    hipLaunchKernelGGL((rc_merge_kernel<K>), dim3((Bp + 255) / 256, T), dim3(256), 0, st, c.lists, slices, Bp, 1, S, c.low, col_stat);
+    hipLaunchKernelGGL((rc_merge_kernel<K>), dim3((Bp + 255) / 256, T), dim3(256), 0, st, c.lists, slices, Bp, 1, S, c.low, col_stat, ratio);
     if ((rc = check_launch("rc_merge_kernel"))) return rc;
-    hipLaunchKernelGGL((rc_bits_kernel<false, MASKED>), tgrid, dim3(256), 0, st, x, nullptr, xkeep, c.wr, c.low, B, N, T, Bp, S, c.bits, c.partial, col_stat);
+    hipLaunchKernelGGL((rc_bits_kernel<false, MASKED>), tgrid, dim3(256), 0, st, x, nullptr, xkeep, c.wr, c.low, B, N, T, Bp, S, c.bits, c.partial, col_stat, ratio);
     if ((rc = check_launch("rc_bits_kernel"))) return rc;
-    hipLaunchKernelGGL(rc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)tgrid.x * tgrid.y * tgrid.z * 4, c.count, col_count, col_stat, S, limit);
+    hipLaunchKernelGGL(rc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)tgrid.x * tgrid.y * tgrid.z * 4, c.count, col_count, col_stat, S, limit, ratio);
     if ((rc = check_launch("rc_sum_kernel"))) return rc;
     MainArgs a{x, nullptr, w, xkeep, wkeep, c.bits, c.low, c.count, c.fix, B, Bp, M, N, 0, 0.f, nullptr, y, pos};
-    // (eight rows per wavefront; six under the mask, whose keep words take registers too)
-    if (pos) rc = launch_main<kRowsMax, 1, MASKED ? 6 : 8, true, MASKED>(a, st);
-    else rc = launch_main<kRowsMax, 1, MASKED ? 6 : 8, false, MASKED>(a, st);
+    // (four rows per wavefront: their mark lists share the LDS with the weight tiles)
+    if (pos) rc = launch_main<kRowsMax, 1, 4, true, MASKED>(a, st);
+    else rc = launch_main<kRowsMax, 1, 4, false, MASKED>(a, st);
     if (rc || !MASKED) return rc;
     if (pos) hipLaunchKernelGGL((rc_fix_kernel<true>), dim3(256), dim3(256), 0, st, a);
     else hipLaunchKernelGGL((rc_fix_kernel<false>), dim3(256), dim3(256), 0, st, a);
@@ -806,8 +815,9 @@ bool row_cands_supported(int form, int K) {
 
 int row_cands_forward(int form, const float* xl, const float* xu, const float* w, const uint32_t* xkeep,
                       const uint32_t* wkeep, int B, int CO, int CI, float q, int K, float* outL, float* outU, int* pos,
-                      void* ws, float density, const float* col_stat, const unsigned long long* col_count,
+                      void* ws, float density, bool forced, const float* col_stat, const unsigned long long* col_count,
                       const unsigned long long** every, hipStream_t st) {
+    const float ratio_max = forced ? kProbeRatio : kProbeRatioMax;
     if (CI % kChunk != 0 || B < 1 || CO < 1 || !row_cands_supported(form, K) || (xkeep == nullptr) != (wkeep == nullptr) ||
         (long long)B * CO >= (1ll << 32)) {
         set_error("row_cands_forward: shape or form not supported");
@@ -840,9 +850,9 @@ int row_cands_forward(int form, const float* xl, const float* xu, const float* w
             }
             break;
         case kRowsMax:
-            if (!xkeep) return run_max<1, false>(xl, w, nullptr, nullptr, B, CO, CI, outU, pos, c, limit, col_stat, col_count, st);
+            if (!xkeep) return run_max<1, false>(xl, w, nullptr, nullptr, B, CO, CI, outU, pos, c, limit, col_stat, col_count, ratio_max, st);
             switch (K) {
-#define X(k) case k: return run_max<k, true>(xl, w, xkeep, wkeep, B, CO, CI, outU, pos, c, limit, col_stat, col_count, st);
+#define X(k) case k: return run_max<k, true>(xl, w, xkeep, wkeep, B, CO, CI, outU, pos, c, limit, col_stat, col_count, ratio_max, st);
                 X(8) X(12) X(16) X(20) X(24)
 #undef X
             }

@@ -190,7 +190,7 @@ static int queue_sort_cols(FwdArgs& a, int form, const float* xl, const float* x
     char* rows_ws = static_cast<char*>(ws) + (sort_cols_workspace(B, CO, CI, K) + 255) / 256 * 256;
     const unsigned long long* every = nullptr;
     rc = row_cands_forward(form, xl, xu, w, nullptr, nullptr, B, CO, CI, q, K, outL, outU, pos, rows_ws,
-                           density > 0.f ? density : kSortRowsCap, sort_cols_probe_sums(col_count), col_count, &every, st);
+                           density > 0.f ? density : kSortRowsCap, density > 0.f, sort_cols_probe_sums(col_count), col_count, &every, st);
     if (rc) return rc;
     a.gate = every;
     a.gate_limit = 0ull;
