@@ -799,6 +799,57 @@ struct BoundChunk : PolicyBase {
     }
 };
 
+// BoundChunk for the LDS-direct kernel: the numbers of the winning chunks inside the slice kept in 8 bits each, the
+// lower and the upper bound's side by side (two outputs to a register; at most 254 chunks per slice, 255 = none), so
+// that 4 x 4 outputs cost 64 + 8 registers and the tile fits four waves per SIMD next to no staging registers.  Same
+// (value, chunk) pairs as BoundChunk, so the same resolve pass follows.
+struct BoundChunkPacked : PolicyBase {
+    static constexpr bool GATED = true;   // one of two queued for a result when FwdArgs::gate is set
+    static constexpr bool DIRECT = true;
+    static constexpr bool HAS_TSTATE = true;
+    static constexpr int NX = 2;
+    static constexpr int MAX_CHUNKS = 254;      // per slice
+    struct Acc { float lo, hi, cl, ch; };
+    template <int N> struct TState { uint32_t cids[(N + 1) / 2]; };   // per output: byte 0 lower, byte 1 upper (of its half word)
+    template <int N> static __device__ __forceinline__ void tinit(TState<N>& S) {
+        #pragma unroll
+        for (int k = 0; k < (N + 1) / 2; k++) S.cids[k] = 0xffffffffu;
+    }
+    static __device__ __forceinline__ void init(Acc& A, const FwdArgs&, size_t, bool, int split = 0) {
+        A.lo = -kEps; A.hi = kEps; A.cl = 0.f; A.ch = 0.f;
+    }
+    static __device__ __forceinline__ void term(Acc& A, float l, float u, float w) {
+        float t1 = w - l, t2 = u - w;
+        A.cl = fminf(fminf(A.cl, t1), t2);
+        A.ch = fmaxf(fmaxf(A.ch, t1), t2);
+    }
+    static __device__ __forceinline__ void step4(Acc& A, const FwdArgs&, const float4& l, const float4& u,
+                                                 const float4& w, int, int) {
+        term(A, l.x, u.x, w.x); term(A, l.y, u.y, w.y); term(A, l.z, u.z, w.z); term(A, l.w, u.w, w.w);
+    }
+    template <int N>
+    static __device__ __forceinline__ void chunk_end_t(Acc& A, TState<N>& S, const FwdArgs&, int idx, int, int kl) {
+        const bool wl = A.cl < A.lo, wh = A.ch > A.hi;   // strictly better: the lowest chunk attaining a bound survives
+        const int sh = 16 * (idx & 1);
+        uint32_t f = S.cids[idx >> 1];
+        A.lo = wl ? A.cl : A.lo;
+        A.hi = wh ? A.ch : A.hi;
+        f = wl ? ((f & ~(0xffu << sh)) | ((uint32_t)kl << sh)) : f;
+        f = wh ? ((f & ~(0xffu << (sh + 8))) | ((uint32_t)kl << (sh + 8))) : f;
+        S.cids[idx >> 1] = f;
+        A.cl = 0.f; A.ch = 0.f;
+    }
+    template <int N>
+    static __device__ __forceinline__ void store_t(Acc& A, TState<N>& S, const FwdArgs& a, size_t o, int, int idx, int c0) {
+        const uint32_t f = S.cids[idx >> 1] >> (16 * (idx & 1));
+        const uint32_t kl = f & 0xffu, kh = (f >> 8) & 0xffu;
+        store_chunk_winner(a, o, -A.lo, kl == 0xffu ? -1 : c0 + (int)kl, false);
+        store_chunk_winner(a, o, A.hi, kh == 0xffu ? -1 : c0 + (int)kh, true);
+    }
+    static __device__ __forceinline__ void chunk_end(Acc&, const FwdArgs&, int, int) {}
+    static __device__ __forceinline__ void store(Acc&, const FwdArgs&, size_t, int split = 0) {}
+};
+
 // ---- sort neuron -------------------------------------------------------------------------
 // res[] ascending (res[K-1] largest), slots start at 0.  A value v > res[0] is inserted above
 // equal values: new[k] = clamp(v, res[k], res[k+1]), new[K-1] = max(res[K-1], v); the index

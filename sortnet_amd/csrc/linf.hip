@@ -467,7 +467,10 @@ extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* input
             a.gate_above = 1;
         }
     }
-    rc = TB == 2 ? launch_fwd<BoundChunk, 2, 4>(a, st) : launch_fwd<BoundChunk, 4, 4>(a, st);
+    // exact dense tiles: the LDS-direct kernel with the chunk numbers packed (same (value, chunk) pairs, same resolve)
+    if (TB == 4 && a.nsplit > 1 && direct_ok<4, 4>(a) && (a.CIg / KT + a.nsplit - 1) / a.nsplit <= BoundChunkPacked::MAX_CHUNKS)
+        rc = launch_fwd_direct<BoundChunkPacked, 4, 4>(a, st);
+    else rc = TB == 2 ? launch_fwd<BoundChunk, 2, 4>(a, st) : launch_fwd<BoundChunk, 4, 4>(a, st);
     if (rc) return rc;
     if (hinted && cols) hint_record(kHintSiteBoundPos, weight, B, CO, CI, a.gate, st);   // the gate is 1 when every term ran
     return launch_resolve_bound(a, st);

@@ -407,8 +407,7 @@ __global__ void __launch_bounds__(64 * kWaves, 1) rc_main_kernel(MainArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // this wavefront's lists of the marked inputs of its rows in one stage (two entries past a full list are read)
     struct Entry { int i; float l, u; };
-    constexpr int kMarkRow = kStage + 2;
-    Entry* marks = reinterpret_cast<Entry*>(wb + kSeg * ROWS) + wave * (TR * kMarkRow);
+    Entry* marks = reinterpret_cast<Entry*>(wb + kSeg * ROWS) + wave * (TR * kStage + 2);
     const int B = a.B, Bp = a.Bp, M = a.M, N = a.N, NCH = N / kChunk;
     const int rows = a.rows, BG = (B + rows - 1) / rows;
     // Workgroups go to the chip's eight dies in turn, each with a cache of its own: consecutive (tile, batch rows)
@@ -545,37 +544,39 @@ __global__ void __launch_bounds__(64 * kWaves, 1) rc_main_kernel(MainArgs a) {
     // list.  The walk over a list then costs one broadcast read per mark and no bit scanning (the scalar unit, which
     // all sixteen wavefronts share, only keeps the loop's count), and it is software-pipelined: while the terms of
     // mark k are formed, the weights of mark k + 1 and the entry of mark k + 2 are on their way (an entry must have
-    // arrived before its weights can be asked for: two dependent LDS reads per mark otherwise).
+    // arrived before its weights can be asked for: two dependent LDS reads per mark otherwise).  The rows' lists lie
+    // end to end, so the pipeline is filled once per stage and runs on across the rows.
     auto compute = [&](int buf, int st, const float (&xl_)[TR], const float (&xu_)[IV ? TR : 1]) __attribute__((always_inline)) {
         const char* W = reinterpret_cast<const char*>(wt(buf) + 2 * lane);
         const uint32_t* words = wb + (2 * st - seg_lo) * ROWS + r_lo;
         uint32_t wa[TR], wc[TR];
         #pragma unroll
         for (int r = 0; r < TR; r++) { wa[r] = words[r < nr ? r : 0]; wc[r] = words[ROWS + (r < nr ? r : 0)]; }
-        int cnt[TR];
-        __builtin_amdgcn_wave_barrier();                 // the walks of the stage before this one have read their entries
+        int end[TR];                                      // one past row r's last entry in the wavefront's list
+        __builtin_amdgcn_wave_barrier();                 // the walk of the stage before this one has read its entries
+        int filled = 0;
         #pragma unroll
         for (int r = 0; r < TR; r++) {
             uint32_t mlo = 0u, mhi = 0u;
             if (r < nr) { mlo = (uint32_t)__builtin_amdgcn_readfirstlane(wa[r]); mhi = (uint32_t)__builtin_amdgcn_readfirstlane(wc[r]); }
-            cnt[r] = __builtin_popcount(mlo) + __builtin_popcount(mhi);
             const uint32_t mine = ((lane < 32 ? mlo : mhi) >> (lane & 31)) & 1u;
             const int rank = (int)__builtin_amdgcn_mbcnt_hi(mhi, __builtin_amdgcn_mbcnt_lo(mlo, 0u));
-            if (mine) marks[r * kMarkRow + rank] = Entry{lane, xl_[r], IV ? xu_[IV ? r : 0] : 0.f};
+            if (mine) marks[filled + rank] = Entry{lane, xl_[r], IV ? xu_[IV ? r : 0] : 0.f};
+            filled += __builtin_popcount(mlo) + __builtin_popcount(mhi);
+            end[r] = filled;
         }
         __builtin_amdgcn_wave_barrier();                 // LDS operations of one wavefront complete in order
+        if (filled == 0) return;
         const int n0 = st * kStage;
+        // (past the end of the list the entries are stale: their input numbers are masked into the stage, not used)
+        Entry e = marks[0], e1 = marks[1];
+        float2 ww = *reinterpret_cast<const float2*>(W + (e.i & (kStage - 1)) * (kWRow * 4));
+        int k = 0;
         static_for([&](auto R) __attribute__((always_inline)) {
             constexpr int r = decltype(R)::value;
-            const int total = cnt[r];
-            if (total == 0) return;
-            const Entry* list = marks + r * kMarkRow;
-            // (past the end of the list the entries are stale: their input numbers are masked into the stage, not used)
-            Entry e = list[0], e1 = list[1];
-            float2 ww = *reinterpret_cast<const float2*>(W + (e.i & (kStage - 1)) * (kWRow * 4));
-            for (int k = 0; k < total; k++) {
+            for (; k < end[r]; k++) {
                 const float2 w1 = *reinterpret_cast<const float2*>(W + (e1.i & (kStage - 1)) * (kWRow * 4));
-                const Entry e2 = list[k + 2];
+                const Entry e2 = marks[k + 2];
                 term(R, ww, e.l, e.u, n0 + e.i);
                 e = e1; ww = w1; e1 = e2;
             }
@@ -739,7 +740,8 @@ int launch_main(MainArgs a, hipStream_t st) {
 constexpr int tr_for(int form, int K) {
     const int per = (form == kRowsSortValues ? 2 : 4) * K;
     // (the ordered insertion with positions needs the most temporaries, the two-list form a few more than the values)
-    const int tr = (form == kRowsSortValues ? 64 : form == kRowsSortInterval ? 44 : 40) / per;
+    const int tr = (form == kRowsSortValues ? 64 : form == kRowsSortInterval ? 80 : 40) / per;
+    if (form == kRowsSortInterval && tr >= 4) return tr > 5 ? 4 : 3;   // (four and five rows of two lists spill)
     return tr > 5 ? 5 : tr < 1 ? 1 : tr;
 }
 

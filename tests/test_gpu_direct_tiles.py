@@ -103,6 +103,21 @@ def test_interval_bounds_with_inverted_intervals(oracle, B, CI, CO, G):
     _served_by((B, CI, CO, G))
     assert np.array_equal(yl.cpu().numpy(), rl)
     assert np.array_equal(yu.cpu().numpy(), ru)
+    # with positions: the chunk-tracking form (4 x 4 outputs, chunk numbers packed two outputs to a register), also on
+    # coarse-grid data where many terms tie for a bound inside a chunk and across chunks
+    for grid in (None, 8):
+        if grid:
+            xl, xu, wq = (xl * grid).round() / grid, (xu * grid).round() / grid, (w * grid).round() / grid
+        else:
+            wq = w
+        rl, ru, rpl, rpu = oracle.bound_inf_dist_forward(xl.numpy(), xu.numpy(), wq.numpy(), G)
+        zl, zu = torch.empty(B, CO, 1, device=dev), torch.empty(B, CO, 1, device=dev)
+        pl = torch.empty(B, CO, 1, device=dev, dtype=torch.int32)
+        pu = torch.empty_like(pl)
+        ext.bound_inf_dist_forward(xl.to(dev), xu.to(dev), wq.to(dev), zl, zu, pl, pu, G)
+        _served_by((B, CI, CO, G), "fwd_kernel_direct<4,4>")
+        assert np.array_equal(zl.cpu().numpy(), rl) and np.array_equal(zu.cpu().numpy(), ru), grid
+        assert np.array_equal(pl.cpu().numpy(), rpl) and np.array_equal(pu.cpu().numpy(), rpu), grid
 
 
 @pytest.mark.parametrize("B,CI,CO,G", [EXACT[0], EXACT[2], EXACT[3]])
