@@ -90,6 +90,14 @@ __device__ __forceinline__ void insert_value(float (&res)[K], float v) {
     for (int k = 0; k < K - 1; k++) res[k] = __builtin_amdgcn_fmed3f(res[k], v, res[k + 1]);
     res[K - 1] = __builtin_amdgcn_fmed3f(res[K - 1], v, __builtin_inff());
 }
+// The same with +infinity held in a register the compiler cannot see through: with the literal it rewrites the last
+// median as a maximum and adds an instruction that quiets res[K - 1] first (two instructions per list and mark).
+template <int K>
+__device__ __forceinline__ void insert_value(float (&res)[K], float v, float inf) {
+    #pragma unroll
+    for (int k = 0; k < K - 1; k++) res[k] = __builtin_amdgcn_fmed3f(res[k], v, res[k + 1]);
+    res[K - 1] = __builtin_amdgcn_fmed3f(res[K - 1], v, inf);
+}
 
 template <class F, int... R>
 __device__ __forceinline__ void static_for(F&& f, std::integer_sequence<int, R...>) {
@@ -406,7 +414,9 @@ __global__ void __launch_bounds__(64 * kWaves, 1) rc_main_kernel(MainArgs a) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // this wavefront's lists of the marked inputs of its rows in one stage (two entries past a full list are read)
-    struct Entry { int i; float l, u; };
+    // (off: byte offset of the input's weights in the tile; un: the row's upper end in the interval form, the input's
+    // number within the stage, as bits, in the others)
+    struct Entry { int off; float l, un; };
     Entry* marks = reinterpret_cast<Entry*>(wb + kSeg * ROWS) + wave * (TR * kStage + 2);
     const int B = a.B, Bp = a.Bp, M = a.M, N = a.N, NCH = N / kChunk;
     const int rows = a.rows, BG = (B + rows - 1) / rows;
@@ -419,6 +429,11 @@ __global__ void __launch_bounds__(64 * kWaves, 1) rc_main_kernel(MainArgs a) {
     // this wavefront's rows of the group: r_lo .. r_lo + nr - 1 (nr <= TR)
     const int r_lo = wave * rows / kWaves, nr = (wave + 1) * rows / kWaves - r_lo;
     auto wt = [&](int buf) { return smem + buf * TILE; };
+
+    // the lists of marks start as zeros: entries past the end of a list are read (and not used)
+    for (int i = lane; i < (TR * kStage + 2) * 3; i += 64) reinterpret_cast<uint32_t*>(marks)[i] = 0u;
+    float inf = __builtin_inff();
+    asm volatile("" : "+v"(inf));                     // (see insert_value)
 
     // state of the wavefront's rows x the lane's two weight rows
     constexpr bool LISTS = FORM != kRowsMax;
@@ -507,20 +522,22 @@ __global__ void __launch_bounds__(64 * kWaves, 1) rc_main_kernel(MainArgs a) {
             xl_[r] = l;
         }
     };
-    // one marked input of row r: ww = the lane's two weights, (xa, xb) = the row's value (or its l and u), n = its number
-    auto term = [&](auto R, const float2& ww, float xa, float xb, int n) __attribute__((always_inline)) {
+    // one marked input of row r: ww = the lane's two weights, (xa, xb) = the row's value and the input's number within
+    // the stage as bits (or its l and u), n0 = the first input of the stage
+    auto term = [&](auto R, const float2& ww, float xa, float xb, int n0) __attribute__((always_inline)) {
         constexpr int r = decltype(R)::value;
+        [[maybe_unused]] const int n = n0 + __float_as_int(xb);   // (forms without an interval)
         if constexpr (IV) {
             const float a1 = ww.x - xa, a2 = xb - ww.x, b1 = ww.y - xa, b2 = xb - ww.y;
-            insert_value<K>(lo[r][0], -fminf(a1, a2));
-            insert_value<K>(hi[r][0], fmaxf(a1, a2));
-            insert_value<K>(lo[r][1], -fminf(b1, b2));
-            insert_value<K>(hi[r][1], fmaxf(b1, b2));
+            insert_value<K>(lo[r][0], -fminf(a1, a2), inf);
+            insert_value<K>(hi[r][0], fmaxf(a1, a2), inf);
+            insert_value<K>(lo[r][1], -fminf(b1, b2), inf);
+            insert_value<K>(hi[r][1], fmaxf(b1, b2), inf);
         } else {
             const float d0 = xa - ww.x, d1 = xa - ww.y;
             if constexpr (FORM == kRowsSortValues) {
-                insert_value<K>(hi[r][0], fabsf(d0));
-                insert_value<K>(hi[r][1], fabsf(d1));
+                insert_value<K>(hi[r][0], fabsf(d0), inf);
+                insert_value<K>(hi[r][1], fabsf(d1), inf);
             } else if constexpr (FORM == kRowsSortPos) {
                 // the marks of a row go by in ascending input order: the ordered insertion of the scan over
                 // all inputs (core/cuda/sort_neuron.cu:108-113, 176-185), ties included
@@ -561,23 +578,24 @@ __global__ void __launch_bounds__(64 * kWaves, 1) rc_main_kernel(MainArgs a) {
             if (r < nr) { mlo = (uint32_t)__builtin_amdgcn_readfirstlane(wa[r]); mhi = (uint32_t)__builtin_amdgcn_readfirstlane(wc[r]); }
             const uint32_t mine = ((lane < 32 ? mlo : mhi) >> (lane & 31)) & 1u;
             const int rank = (int)__builtin_amdgcn_mbcnt_hi(mhi, __builtin_amdgcn_mbcnt_lo(mlo, 0u));
-            if (mine) marks[filled + rank] = Entry{lane, xl_[r], IV ? xu_[IV ? r : 0] : 0.f};
+            if (mine) marks[filled + rank] = Entry{lane * (kWRow * 4), xl_[r], IV ? xu_[IV ? r : 0] : __int_as_float(lane)};
             filled += __builtin_popcount(mlo) + __builtin_popcount(mhi);
             end[r] = filled;
         }
         __builtin_amdgcn_wave_barrier();                 // LDS operations of one wavefront complete in order
         if (filled == 0) return;
         const int n0 = st * kStage;
-        // (past the end of the list the entries are stale: their input numbers are masked into the stage, not used)
+        // (past the end of the list the entries are stale, from an earlier stage or the zeros the lists start with:
+        // their offsets lie in the tile and what is read through them is not used)
         Entry e = marks[0], e1 = marks[1];
-        float2 ww = *reinterpret_cast<const float2*>(W + (e.i & (kStage - 1)) * (kWRow * 4));
+        float2 ww = *reinterpret_cast<const float2*>(W + e.off);
         int k = 0;
         static_for([&](auto R) __attribute__((always_inline)) {
             constexpr int r = decltype(R)::value;
             for (; k < end[r]; k++) {
-                const float2 w1 = *reinterpret_cast<const float2*>(W + (e1.i & (kStage - 1)) * (kWRow * 4));
+                const float2 w1 = *reinterpret_cast<const float2*>(W + e1.off);
                 const Entry e2 = marks[k + 2];
-                term(R, ww, e.l, e.u, n0 + e.i);
+                term(R, ww, e.l, e.un, n0);
                 e = e1; ww = w1; e1 = e2;
             }
         }, std::make_integer_sequence<int, TR>{});
