@@ -862,15 +862,18 @@ __device__ __forceinline__ void topk_insert_values(float (&res)[K], float v) {
 }
 template <int K>
 __device__ __forceinline__ void topk_insert(float (&res)[K], int (&idx)[K], float v, int p) {
+    // (v and the entries are defined numbers here, so "v < res[k + 1]" of slot k is "not v >= res[k + 1]" of slot
+    // k + 1: one comparison per slot serves both, and the values move as the median of (res[k], v, res[k + 1]))
+    bool ge[K];
+    #pragma unroll
+    for (int k = 0; k < K; k++) ge[k] = v >= res[k];
     #pragma unroll
     for (int k = 0; k < K - 1; k++) {
-        bool below_next = v < res[k + 1], above_cur = v >= res[k];
-        idx[k] = below_next ? (above_cur ? p : idx[k]) : idx[k + 1];
-        res[k] = below_next ? (above_cur ? v : res[k]) : res[k + 1];
+        idx[k] = ge[k + 1] ? idx[k + 1] : (ge[k] ? p : idx[k]);
+        res[k] = __builtin_amdgcn_fmed3f(res[k], v, res[k + 1]);   // = ge[k + 1] ? res[k + 1] : (ge[k] ? v : res[k])
     }
-    bool top = v >= res[K - 1];
-    idx[K - 1] = top ? p : idx[K - 1];
-    res[K - 1] = top ? v : res[K - 1];
+    idx[K - 1] = ge[K - 1] ? p : idx[K - 1];
+    res[K - 1] = ge[K - 1] ? v : res[K - 1];
 }
 // y = (init + sum_j t_j c_j q) / (1 - c_K), largest first, every product rounded separately
 template <int K>

@@ -25,6 +25,11 @@ inline int slices_of(int NCH) {
     return s < NCH ? s : NCH;
 }
 
+// The value and interval forms of the sort neuron walk a transposed copy of the weights, wavefront by wavefront,
+// without LDS tiles or barriers (rt_main_kernel); the forms with positions and the l-inf forms stage tiles
+// (rc_main_kernel).
+constexpr bool walks_transposed(int form) { return form == kRowsSortValues || form == kRowsSortInterval; }
+
 struct Carve {
     float* wr;        // [T][2][N]  per tile of weight rows and input: min w, max w over the rows that keep the input
     float* lists;     // [T][slices][nw][K][Bp]  K largest chunk maxima of the lower bounds of a batch row's terms within a slice
@@ -33,9 +38,10 @@ struct Carve {
     uint32_t* partial;            // marks per wavefront of the table kernel
     unsigned long long* count;    // [0] marks, [1] every-term kernels run, [2] this table's kernel runs, [3] marks per weight row (copy), [4] outputs to recompute
     uint32_t* fix;    // [B * M] outputs of the masked l-inf form whose bound did not hold (recomputed from every input)
+    float* wt;        // [T][N][128] the weights of a tile, one 512-byte row per input (forms walked without LDS tiles)
 };
 
-size_t carve_sizes(int form, int B, int M, int N, int K, size_t (&sz)[7]) {
+size_t carve_sizes(int form, int B, int M, int N, int K, size_t (&sz)[8]) {
     const size_t T = tiles_w(M), Bp = bpad_of(B), NCH = N / kChunk, slices = slices_of((int)NCH);
     const size_t nw = form == kRowsSortInterval ? 2 : 1;
     sz[0] = align256(T * 2 * N * 4);
@@ -45,13 +51,14 @@ size_t carve_sizes(int form, int B, int M, int N, int K, size_t (&sz)[7]) {
     sz[4] = align256(Bp / 64 * slices * ((T + 3) / 4) * 4 * 4);
     sz[5] = 256;
     sz[6] = form == kRowsMax ? align256((size_t)B * M * 4) : 0;
+    sz[7] = walks_transposed(form) ? align256(T * N * kTileW * 4) : 0;
     size_t t = 0;
     for (size_t v : sz) t += v;
     return t;
 }
 
 Carve carve(void* ws, int form, int B, int M, int N, int K) {
-    size_t sz[7];
+    size_t sz[8];
     carve_sizes(form, B, M, N, K, sz);
     char* p = static_cast<char*>(ws);
     Carve c;
@@ -61,7 +68,8 @@ Carve carve(void* ws, int form, int B, int M, int N, int K) {
     c.bits = reinterpret_cast<uint32_t*>(p); p += sz[3];
     c.partial = reinterpret_cast<uint32_t*>(p); p += sz[4];
     c.count = reinterpret_cast<unsigned long long*>(p); p += sz[5];
-    c.fix = reinterpret_cast<uint32_t*>(p);
+    c.fix = reinterpret_cast<uint32_t*>(p); p += sz[6];
+    c.wt = reinterpret_cast<float*>(p);
     return c;
 }
 
@@ -108,10 +116,11 @@ __device__ __forceinline__ void static_for(F&& f, std::integer_sequence<int, R..
 // Column ranges of the weights over a tile of 128 weight rows (WMASK: over the rows that keep the input; a column
 // that no row keeps, or that holds an undefined or infinite weight, becomes (-inf, +inf): no lower bound, always a
 // candidate).  64 inputs x 4 groups of 32 rows per workgroup.
-template <bool WMASK>
+template <bool WMASK, bool WT = false>
 __global__ void __launch_bounds__(256) rc_range_kernel(const float* __restrict__ w, const uint32_t* __restrict__ wkeep,
                                                        int M, int N, int S, float* __restrict__ wr,
-                                                       const float* __restrict__ stat, float ratio) {
+                                                       const float* __restrict__ stat, float ratio,
+                                                       float* __restrict__ wt = nullptr) {
     if (!rows_decide(stat, S, ratio)) return;
     __shared__ float part[4][3][64];
     const int nl = threadIdx.x & 63, grp = threadIdx.x >> 6;
@@ -119,7 +128,22 @@ __global__ void __launch_bounds__(256) rc_range_kernel(const float* __restrict__
     const int r0 = t * kTileW + grp * (kTileW / 4);
     const int r1 = r0 + kTileW / 4 < M ? r0 + kTileW / 4 : M;
     float lo = __builtin_inff(), hi = -__builtin_inff(), odd = 0.f;
-    if (n < N) {
+    if constexpr (WT) {
+        // WT: also the transposed copy, wt[(t N + n) 128 + row of the tile] (rows past the last: zero, not used)
+        static_assert(!WMASK, "the transposed copy is for the forms without a mask");
+        if (n < N) {
+            float v[kTileW / 4];
+            #pragma unroll
+            for (int i = 0; i < kTileW / 4; i++) v[i] = r0 + i < M ? w[(size_t)(r0 + i) * N + n] : 0.f;
+            #pragma unroll
+            for (int i = 0; i < kTileW / 4; i++) {
+                if (r0 + i < M) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); odd += v[i] - v[i]; }
+            }
+            float4* dst = reinterpret_cast<float4*>(wt + ((size_t)t * N + n) * kTileW + grp * (kTileW / 4));
+            #pragma unroll
+            for (int i = 0; i < kTileW / 16; i++) dst[i] = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+        }
+    } else if (n < N) {
         #pragma unroll 4
         for (int m = r0; m < r1; m++) {
             bool kept = true;
@@ -261,7 +285,9 @@ __global__ void __launch_bounds__(256) rc_merge_kernel(const float* __restrict__
 // rows of the tile reaches the bound of its list and is positive (the lists start at 0 and take larger values only;
 // an undefined bound or term compares false: an undefined term is left out of every list).  Marks counted per
 // wavefront.
-template <bool IV, bool XMASK>
+// BYROW: the words of a (tile, batch row) lie side by side over the chunks, bits[(t Bp + b) NCH + c] (rt_main_kernel
+// reads a row's words 64 at a time); otherwise those of a (tile, chunk) over the batch rows, bits[(t NCH + c) Bp + b].
+template <bool IV, bool XMASK, bool BYROW = false>
 __global__ void __launch_bounds__(256) rc_bits_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
                                                       const uint32_t* __restrict__ xkeep, const float* __restrict__ wr,
                                                       const float* __restrict__ low, int B, int N, int T, int Bp, int S,
@@ -339,7 +365,8 @@ __global__ void __launch_bounds__(256) rc_bits_kernel(const float* __restrict__ 
             }
             if (!valid) word = 0u;
             if constexpr (XMASK) word &= xkeep[(size_t)brow * NCH + c];
-            bits[((size_t)t * NCH + c) * Bp + b0 + r] = word;
+            if constexpr (BYROW) bits[((size_t)t * Bp + b0 + r) * NCH + c] = word;
+            else bits[((size_t)t * NCH + c) * Bp + b0 + r] = word;
             marks += __builtin_popcount(word);
         }
         __syncthreads();
@@ -674,6 +701,150 @@ __global__ void __launch_bounds__(64 * kWaves, 1) rc_main_kernel(MainArgs a) {
     }, std::make_integer_sequence<int, TR>{});
 }
 
+// ---- main kernel without tiles -------------------------------------------------------------------
+// Values and interval bounds of the sort neuron.  A wavefront takes one batch row at a time against the tile's 128
+// weight rows (lane l holds the rows l and l + 64): it reads the row's table words 64 chunks at a time, lists the
+// marked inputs in LDS and walks the list four marks at a time with the loads of the next four in flight: lane l
+// fetches the number and the row's value(s) of mark l % 4 (read back lane by lane, so they are scalar operands of the
+// terms), every lane its two weights from the transposed copy (two coalesced 256-byte loads per mark).  No tile is
+// staged and no barrier is met, so a wavefront with many marks holds nobody up; the tile's transposed weights
+// (2.6 MB at 5120 inputs) stay in the cache of the die its workgroups are dealt to.  Every load is issued
+// unconditionally (groups past the end of the list repeat its last mark and are not used), so that the waits the
+// compiler places cover exactly the group that is used next.
+constexpr int kRtWaves = 8;          // wavefronts of a workgroup
+constexpr int kRtRows = 1;           // batch rows a wavefront takes, one after the other
+constexpr int kRtBatch = 64;         // chunks whose table words a wavefront reads at a time, one per lane
+constexpr int kRtListCap = 2304;     // entries of a wavefront's list of marked inputs (16-bit input numbers)
+
+struct RtArgs {
+    const float* xl; const float* xu; const float* wt;
+    const uint32_t* bits;
+    const unsigned long long* count;
+    int B, Bp, M, N;
+    float q;
+    float* outL; float* outU;
+};
+
+template <int K, bool IV>
+__global__ void __launch_bounds__(64 * kRtWaves) rt_main_kernel(RtArgs a) {
+    if (a.count[2] == 0ull) return;
+    __shared__ uint16_t list[kRtWaves][kRtListCap];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int B = a.B, M = a.M, N = a.N, NCH = N / kChunk;
+    const int BG = (B + kRtWaves * kRtRows - 1) / (kRtWaves * kRtRows);
+    // consecutive (tile, batch rows) pairs are dealt out so that the workgroups of a tile share a die and its cache
+    int item = blockIdx.x;
+    if (gridDim.x % 8 == 0) item = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int bg = item % BG, t = item / BG;
+    const float* __restrict__ wcol = a.wt + (size_t)t * N * kTileW + lane;
+    uint16_t* mine = list[wave];
+    float inf = __builtin_inff();
+    asm volatile("" : "+v"(inf));                     // (see insert_value)
+
+    for (int rr = 0; rr < kRtRows; rr++) {
+        const int b = (bg * kRtWaves + wave) * kRtRows + rr;
+        if (b >= B) break;   // wave-uniform; the rows of a wavefront ascend
+        float hi[2][K], lo[IV ? 2 : 1][IV ? K : 1];
+        #pragma unroll
+        for (int k = 0; k < K; k++) {
+            hi[0][k] = hi[1][k] = 0.f;
+            if constexpr (IV) lo[0][k] = lo[1][k] = 0.f;
+        }
+        const uint32_t* __restrict__ rowbits = a.bits + ((size_t)t * a.Bp + b) * NCH;
+        const float* __restrict__ xlrow = a.xl + (size_t)b * N;
+        const float* __restrict__ xurow = IV ? a.xu + (size_t)b * N : nullptr;
+        int cnt = 0;   // marks in the list
+        float xreg[2], ureg[IV ? 2 : 1];
+        float wa[2][4], wb[2][4];
+        auto load = [&](int buf, int k0, int total) __attribute__((always_inline)) {
+            int k = k0 + (lane & 3);
+            k = k < total ? k : total - 1;
+            const int nn = (int)mine[k];
+            float l = xlrow[nn];
+            if constexpr (IV) {
+                float u = xurow[nn];
+                repair(l, u);
+                ureg[buf] = u;
+            }
+            xreg[buf] = l;
+            #pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int n = __builtin_amdgcn_readlane(nn, i);
+                wa[buf][i] = wcol[(size_t)n * kTileW];
+                wb[buf][i] = wcol[(size_t)n * kTileW + 64];
+            }
+        };
+        auto compute = [&](int buf, int k0, int total) __attribute__((always_inline)) {
+            #pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if (k0 + i < total) {   // wave-uniform
+                    const float xi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xreg[buf]), i));
+                    if constexpr (IV) {
+                        const float ui = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ureg[buf]), i));
+                        const float a1 = wa[buf][i] - xi, a2 = ui - wa[buf][i];
+                        const float b1 = wb[buf][i] - xi, b2 = ui - wb[buf][i];
+                        insert_value<K>(lo[0], -fminf(a1, a2), inf);
+                        insert_value<K>(hi[0], fmaxf(a1, a2), inf);
+                        insert_value<K>(lo[1], -fminf(b1, b2), inf);
+                        insert_value<K>(hi[1], fmaxf(b1, b2), inf);
+                    } else {
+                        insert_value<K>(hi[0], fabsf(xi - wa[buf][i]), inf);
+                        insert_value<K>(hi[1], fabsf(xi - wb[buf][i]), inf);
+                    }
+                }
+            }
+        };
+        // walks the list, the loads of a group in flight while the group before it is used
+        auto walk = [&](int total) __attribute__((always_inline)) {
+            if (total == 0) return;
+            load(0, 0, total);
+            for (int k0 = 0; k0 < total; k0 += 8) {
+                load(1, k0 + 4, total);
+                compute(0, k0, total);
+                load(0, k0 + 8, total);
+                compute(1, k0 + 4, total);
+            }
+        };
+        uint32_t next = lane < NCH ? rowbits[lane] : 0u;
+        for (int c0 = 0; c0 < NCH; c0 += kRtBatch) {
+            uint32_t word = next;
+            if (c0 + kRtBatch < NCH) next = c0 + kRtBatch + lane < NCH ? rowbits[c0 + kRtBatch + lane] : 0u;
+            // every lane appends the marks of its word behind those of the lanes before it
+            const int mine_n = __builtin_popcount(word);
+            int incl = mine_n;
+            #pragma unroll
+            for (int o = 1; o < kRtBatch; o <<= 1) {
+                const int v = __shfl_up(incl, o);
+                if (lane >= o) incl += v;
+            }
+            int off = cnt + incl - mine_n;
+            cnt += __builtin_amdgcn_readlane(incl, kRtBatch - 1);
+            while (word) {
+                const int i = __builtin_ctz(word);
+                word &= word - 1;
+                mine[off++] = (uint16_t)(((c0 + lane) << 5) | i);   // the input's number (rows of at most 65536 inputs)
+            }
+            // a row's marks are walked in one go unless the list could overflow with the next chunks
+            if (cnt > kRtListCap - kRtBatch * kChunk || c0 + kRtBatch >= NCH) {
+                __builtin_amdgcn_wave_barrier();
+                walk(cnt);
+                cnt = 0;
+                __builtin_amdgcn_wave_barrier();   // the reads of the list come before the next marks
+            }
+        }
+        #pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int col = t * kTileW + lane + 64 * j;
+            if (col < M) {
+                const size_t o = (size_t)b * M + col;
+                a.outU[o] = geo_sum<K>(hi[j], a.q);
+                if constexpr (IV) a.outL[o] = geo_sum<K>(lo[j], a.q);
+            }
+        }
+    }
+}
+
 // Outputs of the masked l-inf form whose maximum stayed below the bound their marks were taken against: one
 // wavefront per output over every input that both rows keep, lowest input first among equal terms.
 template <bool POS>
@@ -767,9 +938,11 @@ template <int FORM, int K>
 int run(const float* xl, const float* xu, const float* w, int B, int M, int N, float q, float* outL, float* outU, int* pos,
         const Carve& c, unsigned long long limit, const float* col_stat, const unsigned long long* col_count, hipStream_t st) {
     constexpr bool IV = FORM == kRowsSortInterval;
+    constexpr bool WT = walks_transposed(FORM);
     const int T = tiles_w(M), Bp = bpad_of(B), NCH = N / kChunk, slices = slices_of(NCH), S = (B + 127) / 128;
     int rc;
-    hipLaunchKernelGGL((rc_range_kernel<false>), dim3((N + 63) / 64, T), dim3(256), 0, st, w, nullptr, M, N, S, c.wr, col_stat, kProbeRatio);
+    hipLaunchKernelGGL((rc_range_kernel<false, WT>), dim3((N + 63) / 64, T), dim3(256), 0, st, w, nullptr, M, N, S, c.wr, col_stat,
+                       kProbeRatio, WT ? c.wt : nullptr);
     if ((rc = check_launch("rc_range_kernel"))) return rc;
     const dim3 tgrid(Bp / 64, slices, (T + 3) / 4);
     hipLaunchKernelGGL((rc_low_kernel<K, IV, false>), tgrid, dim3(256), 0, st, xl, xu, nullptr, c.wr, B, N, T, Bp, S, c.lists, col_stat, kProbeRatio);
@@ -777,12 +950,19 @@ int run(const float* xl, const float* xu, const float* w, int B, int M, int N, f
     constexpr int nw = IV ? 2 : 1;
     hipLaunchKernelGGL((rc_merge_kernel<K>), dim3((Bp + 255) / 256, T * nw), dim3(256), 0, st, c.lists, slices, Bp, nw, S, c.low, col_stat, kProbeRatio);
     if ((rc = check_launch("rc_merge_kernel"))) return rc;
-    hipLaunchKernelGGL((rc_bits_kernel<IV, false>), tgrid, dim3(256), 0, st, xl, xu, nullptr, c.wr, c.low, B, N, T, Bp, S, c.bits, c.partial, col_stat, kProbeRatio);
+    hipLaunchKernelGGL((rc_bits_kernel<IV, false, WT>), tgrid, dim3(256), 0, st, xl, xu, nullptr, c.wr, c.low, B, N, T, Bp, S, c.bits, c.partial, col_stat, kProbeRatio);
     if ((rc = check_launch("rc_bits_kernel"))) return rc;
     hipLaunchKernelGGL(rc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)tgrid.x * tgrid.y * tgrid.z * 4, c.count, col_count, col_stat, S, limit, kProbeRatio);
     if ((rc = check_launch("rc_sum_kernel"))) return rc;
-    MainArgs a{xl, xu, w, nullptr, nullptr, c.bits, c.low, c.count, c.fix, B, Bp, M, N, 0, q, outL, outU, pos};
-    return launch_main<FORM, K, tr_for(FORM, K), false, false>(a, st);
+    if constexpr (WT) {
+        RtArgs a{xl, xu, c.wt, c.bits, c.count, B, Bp, M, N, q, outL, outU};
+        const int BG = (B + kRtWaves * kRtRows - 1) / (kRtWaves * kRtRows);
+        hipLaunchKernelGGL((rt_main_kernel<K, IV>), dim3((unsigned)(T * BG)), dim3(64 * kRtWaves), 0, st, a);
+        return check_launch("rt_main_kernel");
+    } else {
+        MainArgs a{xl, xu, w, nullptr, nullptr, c.bits, c.low, c.count, c.fix, B, Bp, M, N, 0, q, outL, outU, pos};
+        return launch_main<FORM, K, tr_for(FORM, K), false, false>(a, st);
+    }
 }
 
 template <int K, bool MASKED>
@@ -815,7 +995,7 @@ int run_max(const float* x, const float* w, const uint32_t* xkeep, const uint32_
 }  // namespace
 
 size_t row_cands_workspace(int form, int B, int CO, int CI, int K) {
-    size_t sz[7];
+    size_t sz[8];
     return carve_sizes(form, B, CO, CI, K, sz);
 }
 
@@ -841,6 +1021,10 @@ int row_cands_forward(int form, const float* xl, const float* xu, const float* w
     if (CI % kChunk != 0 || B < 1 || CO < 1 || !row_cands_supported(form, K) || (xkeep == nullptr) != (wkeep == nullptr) ||
         (long long)B * CO >= (1ll << 32)) {
         set_error("row_cands_forward: shape or form not supported");
+        return SD_ERR_ARG;
+    }
+    if (walks_transposed(form) && CI > 65536) {   // (16-bit input numbers in the lists of marks)
+        set_error("row_cands_forward: rows of more than 65536 inputs");
         return SD_ERR_ARG;
     }
     const Carve c = carve(ws, form, B, CO, CI, K);
