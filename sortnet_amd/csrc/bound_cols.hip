@@ -9,7 +9,6 @@ constexpr int kChunk = kColsChunk;   // inputs per table word
 constexpr int kTileB = 128;          // batch rows of a tile: 64 lanes x 2
 constexpr int kTileW = 128;          // weight rows of a workgroup of the main kernel: 16 wavefronts x 8
 constexpr int kLowSlices = 8;        // slices of the input range in the two table kernels
-constexpr int kSegChunks = 64;       // chunks whose table words the per-batch-row main kernel keeps in LDS at a time
 constexpr int kStage = 64;           // inputs of one LDS stage of the per-weight-row main kernel (two table words)
 
 inline size_t align256(size_t b) { return (b + 255) / 256 * 256; }
@@ -22,16 +21,17 @@ struct Carve {
     float* low;       // [S][2][Mp] (or [T][2][Bp]) lower bounds of the upper / lower result of every output of the table's rows
     float* stat;      // two sums of col_range_kernel's probe, directly behind `low` (one fill clears both)
     unsigned long long* count;   // [0] marks of the per-weight-row table, [1] of the per-batch-row table, [2] every-term kernel's turn
-    uint32_t* bits;   // [S][NCH][Mp] (or [T][NCH][Bp]): bit i of a word = input 32 c + i may hold a maximum of that row in that tile
+    uint32_t* bits;   // [S][NCH][Mp] (or [T][Bp][NCH]): bit i of a word = input 32 c + i may hold a maximum of that row in that tile
     uint32_t* partial;   // marks per wavefront of the table kernel
     uint32_t* order;  // [S][Mp] per batch tile and block of 128 weight rows: the row (0..127) at each place of the block
     float* xt;        // [S][N][64][4] per batch tile and input: (l, l', u, u') of the tile's rows i and i + 64, repaired
+    float* wt;        // [T][N][128] per weight tile and input: the weights of the tile's rows (the per-batch-row kernel walks these)
 };
 
 inline int bpad_of(int B) { return (B + kTileB - 1) / kTileB * kTileB; }
 inline size_t maxz(size_t a, size_t b) { return a > b ? a : b; }
 
-size_t carve_sizes(int B, int M, int N, size_t (&sz)[8]) {
+size_t carve_sizes(int B, int M, int N, size_t (&sz)[9]) {
     const size_t S = tiles_b(B), Mp = mpad_of(M), Bp = bpad_of(B), T = Mp / kTileW, NCH = N / kChunk;
     sz[0] = align256(S * 4 * N * 4);                               // xr
     sz[1] = align256(T * 2 * N * 4);                               // wr
@@ -41,11 +41,12 @@ size_t carve_sizes(int B, int M, int N, size_t (&sz)[8]) {
     sz[5] = align256(maxz(Mp / 64, Bp / 64 * ((T + 3) / 4)) * kLowSlices * 4 * 4);   // partial
     sz[6] = align256(S * N * 1024);                                // xt
     sz[7] = align256(S * Mp * 4);                                  // order
-    return sz[0] + sz[1] + sz[2] + sz[3] + sz[4] + sz[5] + sz[6] + sz[7];
+    sz[8] = align256(Mp * N * 4);                                  // wt
+    return sz[0] + sz[1] + sz[2] + sz[3] + sz[4] + sz[5] + sz[6] + sz[7] + sz[8];
 }
 
 Carve carve(void* ws, int B, int M, int N) {
-    size_t sz[8];
+    size_t sz[9];
     carve_sizes(B, M, N, sz);
     const size_t S = tiles_b(B), Mp = mpad_of(M), Bp = bpad_of(B), T = Mp / kTileW;
     char* p = static_cast<char*>(ws);
@@ -59,7 +60,8 @@ Carve carve(void* ws, int B, int M, int N) {
     c.bits = reinterpret_cast<uint32_t*>(p); p += sz[4];
     c.partial = reinterpret_cast<uint32_t*>(p); p += sz[5];
     c.xt = reinterpret_cast<float*>(p); p += sz[6];
-    c.order = reinterpret_cast<uint32_t*>(p);
+    c.order = reinterpret_cast<uint32_t*>(p); p += sz[7];
+    c.wt = reinterpret_cast<float*>(p);
     return c;
 }
 
@@ -281,10 +283,8 @@ __device__ __forceinline__ void col_table_body(const float* __restrict__ w, cons
 // current one is used.  The results leave through an LDS transpose (coalesced along the weight rows) and merge over
 // the slices by atomic maximum.
 constexpr int kStageFloats = kStage * 256;   // (l, l', u, u') of 64 lanes per input
-constexpr int kMainTileFloats = kChunk * (2 * kTileB + 4 + 2 * 64 + 4);   // per-batch-row main kernel: l/u tile + weight tile of one chunk
-constexpr int kMainWords = kSegChunks * kTileB;                            // and its table words
-constexpr int kLdsWords = 2 * kMainTileFloats + kMainWords > 2 * kStageFloats ? 2 * kMainTileFloats + kMainWords
-                                                                              : 2 * kStageFloats;
+// (two stages of inputs; with positions the results leave through two planes of 128 x 129 words)
+constexpr int kLdsWords = 2 * kStageFloats > 2 * kTileB * (kTileW + 1) ? 2 * kStageFloats : 2 * kTileB * (kTileW + 1);
 
 // (l, l', u, u') of the batch rows i and i + 64 of every tile, per input, repaired: the layout the main kernel keeps
 // in LDS, so that it stages a tile with 16-byte copies.  16 inputs per workgroup.
@@ -517,20 +517,26 @@ __device__ __forceinline__ void bound_cols_body(const float* __restrict__ xT, co
 // Same three steps with the roles exchanged: ranges of W per (tile, input), lower bounds of the results per
 // (tile, batch row), marks per (tile, chunk, batch row).  All of them return at once unless rows_decide().
 __global__ void __launch_bounds__(256) row_range_kernel(const float* __restrict__ w, int M, int N, int S,
-                                                        float* __restrict__ wr, const float* __restrict__ stat) {
+                                                        float* __restrict__ wr, float* __restrict__ wt,
+                                                        const float* __restrict__ stat) {
     if (!rows_decide(stat, S)) return;
     __shared__ float part[4][3][64];
     const int nl = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int n = blockIdx.x * 64 + nl, t = blockIdx.y;
     const int r0 = t * kTileW + grp * (kTileW / 4);
-    const int r1 = r0 + kTileW / 4 < M ? r0 + kTileW / 4 : M;
     float lo = __builtin_inff(), hi = -__builtin_inff(), odd = 0.f;
     if (n < N) {
-        #pragma unroll 4
-        for (int m = r0; m < r1; m++) {
-            const float v = w[(size_t)m * N + n];
-            lo = fminf(lo, v); hi = fmaxf(hi, v); odd += v - v;
+        // also the transposed copy the main kernel walks: wt[(t N + n) 128 + row of the tile] (rows past the last: 0)
+        float v[kTileW / 4];
+        #pragma unroll
+        for (int i = 0; i < kTileW / 4; i++) v[i] = r0 + i < M ? w[(size_t)(r0 + i) * N + n] : 0.f;
+        #pragma unroll
+        for (int i = 0; i < kTileW / 4; i++) {
+            if (r0 + i < M) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); odd += v[i] - v[i]; }
         }
+        float4* dst = reinterpret_cast<float4*>(wt + ((size_t)t * N + n) * kTileW + grp * (kTileW / 4));
+        #pragma unroll
+        for (int i = 0; i < kTileW / 16; i++) dst[i] = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
     }
     part[grp][0][nl] = lo; part[grp][1][nl] = hi; part[grp][2][nl] = odd;
     __syncthreads();
@@ -619,7 +625,7 @@ __device__ __forceinline__ void row_table_body(const float* __restrict__ xl, con
                 }
                 if (!LOW) {
                     if (!valid) word = 0u;
-                    bits[((size_t)t * NCH + c) * Bp + b0 + r] = word;
+                    bits[((size_t)t * Bp + b0 + r) * NCH + c] = word;   // a row's words side by side
                     marks += __builtin_popcount(word);
                 }
             }
@@ -687,179 +693,155 @@ __global__ void __launch_bounds__(1024) sum_tables_kernel(const uint32_t* __rest
     }
 }
 
-// Main kernel of this orientation, same tile with the roles exchanged: lane l holds the weight rows l and l + 64
-// of the tile, wavefront v the batch rows 8 v .. 8 v + 7.  The inputs go by in chunks of 32; the l, u and weight
-// tiles (128 x 32 each) of the next-but-one chunk are in flight while the current one is used from LDS, where an
-// input's (w, w') of a lane is one 8-byte word and the (l, u) of a batch row one 8-byte broadcast.  The table words
-// of 64 chunks at a time are copied to LDS ahead of the loop over them; a chunk nobody marks is not staged.  One
-// loop per batch row over that row's own marks (find-first-set, clear, branch); the results are written along the
-// weight rows as they are.
-// POS as in bound_cols_body: a batch row's marks go by in input order as well.
+// Main kernel of this orientation.  A wavefront takes one batch row against the tile's 128 weight rows (lane l holds the
+// rows l and l + 64): it reads the row's table words 64 chunks at a time, lists the marked inputs in LDS and walks the
+// list four marks at a time with the loads of the next four in flight: lane l fetches the number and the (l, u) of mark
+// l % 4 (read back lane by lane, so they are scalar operands of the terms), every lane its two weights from the
+// transposed copy (two coalesced 256-byte loads per mark).  No tile is staged and no barrier is met; the workgroups of a
+// tile (eight wavefronts = eight batch rows each) are dealt to one die, whose cache then holds the tile's transposed
+// weights.  Every load is issued unconditionally (groups past the end of the list repeat its last mark and are not
+// used).  One wavefront sees every input of its outputs, so the results are stored, not merged.
+// POS: the chunk of the mark that last improved a bound strictly is the chunk of the first input attaining it (the
+// marks go by in input order, and every input that attains a bound is marked); the (value bits << 32 | ~chunk) pairs
+// are left as the every-term kernel with chunk tracking leaves them, for resolve_bound_kernel.
+constexpr int kWalkWaves = 8;        // wavefronts of a workgroup
+constexpr int kWalkBatch = 64;       // chunks whose table words a wavefront reads at a time, one per lane
+constexpr int kWalkListCap = 2304;   // entries of a wavefront's list of marked inputs (16-bit input numbers)
+
 template <bool POS>
-__device__ __forceinline__ void bound_rows_body(const float* __restrict__ xl, const float* __restrict__ xu,
-                                                const float* __restrict__ w, const uint32_t* __restrict__ bits, int B,
-                                                int Bp, int M, int N, int nsplit, float* __restrict__ yL,
-                                                float* __restrict__ yU, unsigned long long* __restrict__ packedL,
-                                                unsigned long long* __restrict__ packedU, float* smem, uint32_t* wb) {
-    constexpr int TR = 8;
-    constexpr int WROW = 2 * 64 + 4;      // floats per input in the weight tile: 64 lanes x (w, w')
-    constexpr int XROW = 2 * kTileB + 4;  // floats per input in the l/u tile: 128 batch rows x (l, u)
-    constexpr int kTileFloats = kChunk * (XROW + WROW);
-    static_assert(kTileFloats == kMainTileFloats && kSegChunks * kTileB == kMainWords, "LDS of the shared kernel");
+__global__ void __launch_bounds__(64 * kWalkWaves)
+bound_rows_walk_kernel(const float* __restrict__ xl, const float* __restrict__ xu, const float* __restrict__ wt,
+                       const uint32_t* __restrict__ bits, const unsigned long long* __restrict__ count,
+                       unsigned long long limit_col, unsigned long long limit_row, int B, int Bp, int M, int N,
+                       float* __restrict__ yL, float* __restrict__ yU, unsigned long long* __restrict__ packedL,
+                       unsigned long long* __restrict__ packedU) {
+    if (count[0] <= limit_col || count[1] > limit_row) return;   // the other table's turn, or the every-term kernel's
+    __shared__ uint16_t list[kWalkWaves][kWalkListCap];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int TM = (M + kTileW - 1) / kTileW, SB = Bp / kTileB, NCH = N / kChunk;
-    const int bt = blockIdx.x % SB, t = (blockIdx.x / SB) % TM, split = blockIdx.x / (TM * SB);
-    const int m0 = t * kTileW, b0 = bt * kTileB;
-    const int per = (NCH + nsplit - 1) / nsplit;
-    const int c_lo = split * per, c_hi = c_lo + per < NCH ? c_lo + per : NCH;
-    auto xt = [&](int buf) { return smem + buf * kTileFloats; };
-    auto wt = [&](int buf) { return smem + buf * kTileFloats + kChunk * XROW; };
-
-    float lo[TR][2], hi[TR][2];
-    uint32_t cw[TR];   // POS: chunk numbers of (lower, lower', upper, upper') of a batch row, one byte each, 255 = none
-    #pragma unroll
-    for (int r = 0; r < TR; r++) { lo[r][0] = lo[r][1] = -kEps; hi[r][0] = hi[r][1] = kEps; cw[r] = 0xffffffffu; }
-
-    // word of (chunk c, batch row b0 + i): bw[c * Bp + i]; rows past the batch, up to the padded count, hold zero
-    const uint32_t* __restrict__ bw = bits + (size_t)t * NCH * Bp + b0;
-    int seg_lo = c_lo;
-    auto marked = [&](int c) {
-        const uint32_t* q = wb + (c - seg_lo) * kTileB;
-        return __builtin_amdgcn_ballot_w64((q[lane] | q[lane + 64]) != 0u) != 0ull;
-    };
-    const int frow = tid >> 3, fq = tid & 7;
-    const int fb = b0 + frow < B ? b0 + frow : B - 1, fm = m0 + frow < M ? m0 + frow : M - 1;
-    auto fetch = [&](int c, bool need, float4& l4, float4& u4, float4& w4) {
-        const size_t off = (size_t)c * kChunk + 4 * fq;
-        l4 = *reinterpret_cast<const float4*>(need ? xl + (size_t)fb * N + off : xl);
-        u4 = *reinterpret_cast<const float4*>(need ? xu + (size_t)fb * N + off : xu);
-        w4 = *reinterpret_cast<const float4*>(need ? w + (size_t)fm * N + off : w);
-    };
-    auto stash = [&](int buf, float4 l4, float4 u4, const float4& w4) {
-        repair(l4.x, u4.x); repair(l4.y, u4.y); repair(l4.z, u4.z); repair(l4.w, u4.w);
-        float* dx = xt(buf) + (4 * fq) * XROW + 2 * frow;
-        *reinterpret_cast<float2*>(dx) = make_float2(l4.x, u4.x);
-        *reinterpret_cast<float2*>(dx + XROW) = make_float2(l4.y, u4.y);
-        *reinterpret_cast<float2*>(dx + 2 * XROW) = make_float2(l4.z, u4.z);
-        *reinterpret_cast<float2*>(dx + 3 * XROW) = make_float2(l4.w, u4.w);
-        // weight row frow belongs to lane frow % 64, slot frow / 64
-        float* dw = wt(buf) + (4 * fq) * WROW + 2 * (frow & 63) + (frow >> 6);
-        dw[0] = w4.x; dw[WROW] = w4.y; dw[2 * WROW] = w4.z; dw[3 * WROW] = w4.w;
-    };
-    auto compute = [&](int buf, int c) {
-        const float* X = xt(buf) + 2 * (wave * TR), *W = wt(buf) + 2 * lane;
-        const uint4* rowwords = reinterpret_cast<const uint4*>(wb + (c - seg_lo) * kTileB + wave * TR);
-        const uint4 q0 = rowwords[0], q1 = rowwords[1];
-        const uint32_t words[TR] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    const int NCH = N / kChunk, BG = (B + kWalkWaves - 1) / kWalkWaves;
+    int item = blockIdx.x;
+    if (gridDim.x % 8 == 0) item = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int bg = item % BG, t = item / BG;
+    const int b = bg * kWalkWaves + wave;
+    if (b >= B) return;   // wave-uniform
+    const float* __restrict__ wcol = wt + (size_t)t * N * kTileW + lane;
+    uint16_t* mine = list[wave];
+    const uint32_t* __restrict__ rowbits = bits + ((size_t)t * Bp + b) * NCH;
+    const float* __restrict__ xlrow = xl + (size_t)b * N;
+    const float* __restrict__ xurow = xu + (size_t)b * N;
+    float lo[2] = {-kEps, -kEps}, hi[2] = {kEps, kEps};
+    int cl[2] = {-1, -1}, cu[2] = {-1, -1};   // POS: chunk of the input that last improved the bound (-1: none)
+    int cnt = 0;   // marks in the list
+    float lreg[2], ureg[2];
+    int nreg[2];
+    float wa[2][4], wb[2][4];
+    auto load = [&](int buf, int k0, int total) __attribute__((always_inline)) {
+        int k = k0 + (lane & 3);
+        k = k < total ? k : total - 1;
+        const int nn = (int)mine[k];
+        float l = xlrow[nn], u = xurow[nn];
+        repair(l, u);
+        lreg[buf] = l; ureg[buf] = u; nreg[buf] = nn;
         #pragma unroll
-        for (int r = 0; r < TR; r++) {
-            uint32_t bm = __builtin_amdgcn_readfirstlane(words[r]);
-            while (bm) {
-                const int n = __builtin_ctz(bm);
-                bm &= bm - 1;
-                const float2 ww = *reinterpret_cast<const float2*>(W + n * WROW);        // the lane's two weights
-                const float2 lu = *reinterpret_cast<const float2*>(X + n * XROW + 2 * r);   // l, u of the row
-                const float a1 = ww.x - lu.x, a2 = lu.y - ww.x, b1 = ww.y - lu.x, b2 = lu.y - ww.y;
-                if (POS) {
-                    const uint32_t kl4 = (uint32_t)(c - c_lo) * 0x01010101u;
+        for (int i = 0; i < 4; i++) {
+            const int n = __builtin_amdgcn_readlane(nn, i);
+            wa[buf][i] = wcol[(size_t)n * kTileW];
+            wb[buf][i] = wcol[(size_t)n * kTileW + 64];
+        }
+    };
+    auto compute = [&](int buf, int k0, int total) __attribute__((always_inline)) {
+        #pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (k0 + i < total) {   // wave-uniform
+                const float li = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lreg[buf]), i));
+                const float ui = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ureg[buf]), i));
+                const float a1 = wa[buf][i] - li, a2 = ui - wa[buf][i], b1 = wb[buf][i] - li, b2 = ui - wb[buf][i];
+                if constexpr (POS) {
+                    const int c = __builtin_amdgcn_readlane(nreg[buf], i) >> 5;
                     const float v0 = fminf(a1, a2), V0 = fmaxf(a1, a2), v1 = fminf(b1, b2), V1 = fmaxf(b1, b2);
-                    const bool w0 = v0 < lo[r][0], w1 = v1 < lo[r][1], w2 = V0 > hi[r][0], w3 = V1 > hi[r][1];
-                    lo[r][0] = w0 ? v0 : lo[r][0]; lo[r][1] = w1 ? v1 : lo[r][1];
-                    hi[r][0] = w2 ? V0 : hi[r][0]; hi[r][1] = w3 ? V1 : hi[r][1];
-                    uint32_t c4 = cw[r];
-                    c4 = w0 ? ((c4 & 0xffffff00u) | (kl4 & 0x000000ffu)) : c4;
-                    c4 = w1 ? ((c4 & 0xffff00ffu) | (kl4 & 0x0000ff00u)) : c4;
-                    c4 = w2 ? ((c4 & 0xff00ffffu) | (kl4 & 0x00ff0000u)) : c4;
-                    c4 = w3 ? ((c4 & 0x00ffffffu) | (kl4 & 0xff000000u)) : c4;
-                    cw[r] = c4;
+                    const bool w0 = v0 < lo[0], w1 = v1 < lo[1], w2 = V0 > hi[0], w3 = V1 > hi[1];
+                    lo[0] = w0 ? v0 : lo[0]; lo[1] = w1 ? v1 : lo[1];
+                    hi[0] = w2 ? V0 : hi[0]; hi[1] = w3 ? V1 : hi[1];
+                    cl[0] = w0 ? c : cl[0]; cl[1] = w1 ? c : cl[1];
+                    cu[0] = w2 ? c : cu[0]; cu[1] = w3 ? c : cu[1];
                 } else {
-                    lo[r][0] = fminf(fminf(lo[r][0], a1), a2);
-                    hi[r][0] = fmaxf(fmaxf(hi[r][0], a1), a2);
-                    lo[r][1] = fminf(fminf(lo[r][1], b1), b2);
-                    hi[r][1] = fmaxf(fmaxf(hi[r][1], b1), b2);
+                    lo[0] = fminf(fminf(lo[0], a1), a2);
+                    hi[0] = fmaxf(fmaxf(hi[0], a1), a2);
+                    lo[1] = fminf(fminf(lo[1], b1), b2);
+                    hi[1] = fmaxf(fmaxf(hi[1], b1), b2);
                 }
             }
         }
     };
-
-    for (; seg_lo < c_hi; seg_lo += kSegChunks) {
-        const int seg_hi = seg_lo + kSegChunks < c_hi ? seg_lo + kSegChunks : c_hi;
-        __syncthreads();
-        for (int e = tid; e < (seg_hi - seg_lo) * kTileB; e += 1024)
-            wb[e] = bw[(size_t)(seg_lo + (e >> 7)) * Bp + (e & (kTileB - 1))];
-        __syncthreads();
-        float4 la, ua, wa, lb, ub, wc;
-        bool n0 = marked(seg_lo), n1 = seg_lo + 1 < seg_hi ? marked(seg_lo + 1) : false;
-        fetch(seg_lo, n0, la, ua, wa);
-        fetch(seg_lo + 1 < seg_hi ? seg_lo + 1 : seg_lo, n1, lb, ub, wc);
-        if (n0) stash(0, la, ua, wa);
-        __syncthreads();
-        for (int c = seg_lo; c < seg_hi; c += 2) {
-            const bool n2 = c + 2 < seg_hi ? marked(c + 2) : false;
-            fetch(c + 2 < seg_hi ? c + 2 : c, n2, la, ua, wa);
-            if (n0) compute(0, c);
-            if (n1) stash(1, lb, ub, wc);
-            __syncthreads();
-            if (c + 1 >= seg_hi) break;
-            const bool n3 = c + 3 < seg_hi ? marked(c + 3) : false;
-            fetch(c + 3 < seg_hi ? c + 3 : c, n3, lb, ub, wc);
-            if (n1) compute(1, c + 1);
-            if (n2) stash(0, la, ua, wa);
-            __syncthreads();
-            n0 = n2; n1 = n3;
+    auto walk = [&](int total) __attribute__((always_inline)) {
+        if (total == 0) return;
+        load(0, 0, total);
+        for (int k0 = 0; k0 < total; k0 += 8) {
+            load(1, k0 + 4, total);
+            compute(0, k0, total);
+            load(0, k0 + 8, total);
+            compute(1, k0 + 4, total);
+        }
+    };
+    uint32_t next = lane < NCH ? rowbits[lane] : 0u;
+    for (int c0 = 0; c0 < NCH; c0 += kWalkBatch) {
+        uint32_t word = next;
+        if (c0 + kWalkBatch < NCH) next = c0 + kWalkBatch + lane < NCH ? rowbits[c0 + kWalkBatch + lane] : 0u;
+        // every lane appends the marks of its word behind those of the lanes before it
+        const int mine_n = __builtin_popcount(word);
+        int incl = mine_n;
+        #pragma unroll
+        for (int o = 1; o < kWalkBatch; o <<= 1) {
+            const int v = __shfl_up(incl, o);
+            if (lane >= o) incl += v;
+        }
+        int off = cnt + incl - mine_n;
+        cnt += __builtin_amdgcn_readlane(incl, kWalkBatch - 1);
+        while (word) {
+            const int i = __builtin_ctz(word);
+            word &= word - 1;
+            mine[off++] = (uint16_t)(((c0 + lane) << 5) | i);   // the input's number (rows of at most 65536 inputs)
+        }
+        // a row's marks are walked in one go unless the list could overflow with the next chunks
+        if (cnt > kWalkListCap - kWalkBatch * kChunk || c0 + kWalkBatch >= NCH) {
+            __builtin_amdgcn_wave_barrier();
+            walk(cnt);
+            cnt = 0;
+            __builtin_amdgcn_wave_barrier();   // the reads of the list come before the next marks
         }
     }
-
     #pragma unroll
-    for (int r = 0; r < TR; r++) {
-        const int row = b0 + wave * TR + r;
-        #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int col = m0 + lane + 64 * j;
-            if (row < B && col < M) {
-                const size_t o = (size_t)row * M + col;
-                if (POS) {
-                    const uint32_t kL = (cw[r] >> (8 * j)) & 0xffu, kU = (cw[r] >> (16 + 8 * j)) & 0xffu;
-                    if (kL != 0xffu)
-                        atomicMax(packedL + o, ((unsigned long long)__float_as_uint(-lo[r][j]) << 32) |
-                                                   (unsigned long long)(0xffffffffu - (uint32_t)(c_lo + (int)kL)));
-                    if (kU != 0xffu)
-                        atomicMax(packedU + o, ((unsigned long long)__float_as_uint(hi[r][j]) << 32) |
-                                                   (unsigned long long)(0xffffffffu - (uint32_t)(c_lo + (int)kU)));
-                    continue;
-                }
-                // both results are >= 1e-10 > 0, so their bit patterns order like integers
-                if (nsplit > 1) {
-                    atomicMax(reinterpret_cast<int*>(yL + o), __float_as_int(-lo[r][j]));
-                    atomicMax(reinterpret_cast<int*>(yU + o), __float_as_int(hi[r][j]));
-                } else { yL[o] = -lo[r][j]; yU[o] = hi[r][j]; }
-            }
+    for (int j = 0; j < 2; j++) {
+        const int col = t * kTileW + lane + 64 * j;
+        if (col < M) {
+            const size_t o = (size_t)b * M + col;
+            if constexpr (POS) {
+                if (cl[j] >= 0)
+                    packedL[o] = ((unsigned long long)__float_as_uint(-lo[j]) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)cl[j]);
+                if (cu[j] >= 0)
+                    packedU[o] = ((unsigned long long)__float_as_uint(hi[j]) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)cu[j]);
+            } else { yL[o] = -lo[j]; yU[o] = hi[j]; }
         }
     }
 }
 
-// One launch for both orientations (same grid, same LDS): whichever table is below its limit is used
+// The kernel of the tables per weight row (the tables per batch row have bound_rows_walk_kernel)
 template <bool POS>
 __global__ void __launch_bounds__(1024, 1)
-bound_table_kernel(const float* __restrict__ xl, const float* __restrict__ xu, const float* __restrict__ w,
-                   const float* __restrict__ xT, const uint32_t* __restrict__ bits, const uint32_t* __restrict__ order,
-                   const unsigned long long* __restrict__ count, unsigned long long limit_col,
-                   unsigned long long limit_row, int B, int Bp, int M, int Mp, int N, int nsplit,
-                   float* __restrict__ yL, float* __restrict__ yU, unsigned long long* __restrict__ packedL,
+bound_table_kernel(const float* __restrict__ w, const float* __restrict__ xT, const uint32_t* __restrict__ bits,
+                   const uint32_t* __restrict__ order, const unsigned long long* __restrict__ count,
+                   unsigned long long limit_col, int B, int M, int Mp, int N, int nsplit, float* __restrict__ yL,
+                   float* __restrict__ yU, unsigned long long* __restrict__ packedL,
                    unsigned long long* __restrict__ packedU) {
     __shared__ __attribute__((aligned(16))) float lds[kLdsWords];
-    if (count[0] <= limit_col)
-        bound_cols_body<POS>(xT, w, bits, order, B, M, Mp, N, nsplit, yL, yU, packedL, packedU, lds);
-    else if (count[1] <= limit_row)
-        bound_rows_body<POS>(xl, xu, w, bits, B, Bp, M, N, nsplit, yL, yU, packedL, packedU, lds,
-                             reinterpret_cast<uint32_t*>(lds + 2 * kMainTileFloats));
+    if (count[0] <= limit_col) bound_cols_body<POS>(xT, w, bits, order, B, M, Mp, N, nsplit, yL, yU, packedL, packedU, lds);
 }
 
 }  // namespace
 
 size_t bound_cols_workspace(int B, int CO, int CI) {
-    size_t sz[8];
+    size_t sz[9];
     return carve_sizes(B, CO, CI, sz);
 }
 
@@ -880,9 +862,10 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
     const float d = density < 0.f ? 0.f : density > 1.f ? 1.f : density;
     const float dr = density_rows < 0.f ? 0.f : density_rows > 1.f ? 1.f : density_rows;
     const unsigned long long limit_col = (unsigned long long)((double)S * CO * CI * d);
-    const unsigned long long limit_row = (unsigned long long)((double)T * B * CI * dr);
-    // ranges of W per tile of weight rows: only when the probe picks the tables per batch row
-    hipLaunchKernelGGL(row_range_kernel, dim3((CI + 63) / 64, T), dim3(256), 0, st, w, CO, CI, S, c.wr, c.stat);
+    // (the kernel of the tables per batch row lists 16-bit input numbers)
+    const unsigned long long limit_row = CI <= 65536 ? (unsigned long long)((double)T * B * CI * dr) : 0ull;
+    // ranges of W per tile of weight rows and the transposed copy: only when the probe picks the tables per batch row
+    hipLaunchKernelGGL(row_range_kernel, dim3((CI + 63) / 64, T), dim3(256), 0, st, w, CO, CI, S, c.wr, c.wt, c.stat);
     if ((rc = check_launch("row_range_kernel"))) return rc;
     const int wg_col = (Mp / 64) * slices, wg_row = (Bp / 64) * slices * ((T + 3) / 4);
     const int wg_tab = wg_col > wg_row ? wg_col : wg_row;
@@ -912,17 +895,23 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
         const double cost = (double)((wgs * n + cus - 1) / cus) / n * (1.0 + 0.04 * n);
         if (n == 1 || cost < best) { best = cost; nsplit = n; }
     }
+    const int BG = (B + kWalkWaves - 1) / kWalkWaves;
     if (with_pos) {
-        // chunk numbers within a slice take 8 bits (255 = none), in either orientation
-        while ((((NCH + 1) / 2 + nsplit - 1) / nsplit) * 2 > 254 || (NCH + nsplit - 1) / nsplit > 254) nsplit++;
-        hipLaunchKernelGGL(bound_table_kernel<true>, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.xt,
-                           c.bits, c.order, c.count, limit_col, limit_row, B, Bp, CO, Mp, CI, nsplit, outL, outU, packedL,
-                           packedU);
-        return check_launch("bound_table_kernel");
+        // chunk numbers within a slice take 8 bits (255 = none)
+        while ((((NCH + 1) / 2 + nsplit - 1) / nsplit) * 2 > 254) nsplit++;
+        hipLaunchKernelGGL(bound_table_kernel<true>, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, w, c.xt, c.bits,
+                           c.order, c.count, limit_col, B, CO, Mp, CI, nsplit, outL, outU, packedL, packedU);
+        if ((rc = check_launch("bound_table_kernel"))) return rc;
+        hipLaunchKernelGGL(bound_rows_walk_kernel<true>, dim3((unsigned)(T * BG)), dim3(64 * kWalkWaves), 0, st, xl, xu, c.wt,
+                           c.bits, c.count, limit_col, limit_row, B, Bp, CO, CI, outL, outU, packedL, packedU);
+        return check_launch("bound_rows_walk_kernel");
     }
-    hipLaunchKernelGGL(bound_table_kernel<false>, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, xl, xu, w, c.xt, c.bits,
-                       c.order, c.count, limit_col, limit_row, B, Bp, CO, Mp, CI, nsplit, outL, outU, nullptr, nullptr);
-    return check_launch("bound_table_kernel");
+    hipLaunchKernelGGL(bound_table_kernel<false>, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, w, c.xt, c.bits, c.order,
+                       c.count, limit_col, B, CO, Mp, CI, nsplit, outL, outU, nullptr, nullptr);
+    if ((rc = check_launch("bound_table_kernel"))) return rc;
+    hipLaunchKernelGGL(bound_rows_walk_kernel<false>, dim3((unsigned)(T * BG)), dim3(64 * kWalkWaves), 0, st, xl, xu, c.wt, c.bits,
+                       c.count, limit_col, limit_row, B, Bp, CO, CI, outL, outU, nullptr, nullptr);
+    return check_launch("bound_rows_walk_kernel");
 }
 
 }  // namespace sd

@@ -60,11 +60,13 @@ static int max_cols_wanted(const FwdArgs& a, int K, int site, int B, int CO, int
 }
 
 // Largest share of marked (tile of 128 weight rows, batch row, input) triples at which the l-inf kernel of the tables
-// per batch row runs.  Measured per 512 x 5120 x 5120 layer: 0.10 ms of tables + 0.09 ms of staging + about 4.5 x share
-// ms for the marks (the walk over a row's marks is bound by the latency of its dependent LDS reads and by the scalar
-// unit, about 30 instructions per mark for 2 x 64 terms), against 0.45 ms (0.60 with positions) for every term: at the
-// 6.5 % that inputs in [0, 1] mark against weights ~ N(0, 1/N) the two meet, so the limit sits below that.
-constexpr float kMaxRowsCap = 0.04f;
+// per batch row runs, and the smallest layer (in terms) given such tables under the built-in limit.  Measured on inputs
+// in [0, 1] against weights ~ N(0, 1/N) (6.5 to 8.4 % marked): 512 x 5120 x 5120 0.34 ms (0.36 with positions; 0.15 ms
+// of it tables and the transposed copy of the weights) against 0.49 (0.61) for every term, 512 x 3072 x 5120 0.26 (0.27)
+// against 0.27 (0.43), 256 x 4096 x 2048 0.13 (0.13) against 0.09 (0.12): the main kernel's time grows with the marks,
+// so the limit sits where the two would meet at the large sizes.
+constexpr float kMaxRowsCap = 0.10f;
+constexpr long long kMaxRowsMinTerms = 1ll << 32;
 
 // bytes of both tables' workspace for one call: per weight row first, per batch row behind it
 static size_t max_tables_bytes(int B, int CO, int CI, int K) {
@@ -81,7 +83,8 @@ static int queue_max_cols(FwdArgs& a, int K, int B, int CO, int CI, void* ws, hi
     const uint32_t* wkeep = K == 1 ? nullptr : a.wmask;
     int rc = max_cols_forward(a.x0, a.w, xkeep, wkeep, B, CO, CI, K, a.y0, a.p0, ws, cap, &a.gate, &a.gate_limit, st);
     a.gate_above = 1;
-    if (rc || !row_cands_supported(kRowsMax, K)) {
+    const bool rows = row_cands_supported(kRowsMax, K) && (density > 0.f || (long long)B * CO * CI >= kMaxRowsMinTerms);
+    if (rc || !rows) {
         if (!rc) { a.gate = a.gate + 1; a.gate_limit = 0ull; }   // the flag behind the counter, as with both tables
         return rc;
     }

@@ -4,10 +4,10 @@
 //
 // Over a tile of weight rows the term |x[b,n] - w[m,n]| is bracketed by the column minimum and maximum of the
 // weights, so the K largest terms of (b, m) sit, for every m of the tile, at the few inputs where x[b, .] is
-// extreme.  A bit table (tile, 32 inputs, batch row) marks the inputs whose term can reach a lower bound of the
-// K-th largest; the main kernel stages tiles of inputs and weights through LDS, gives a wavefront a few batch rows
-// (lane l holds the weight rows l and l + 64 of the tile) and walks each row's own marks with scalar instructions,
-// so an unmarked input costs nothing.  Same bits as the kernels that evaluate every term
+// extreme.  A bit table (tile, batch row, 32 inputs) marks the inputs whose term can reach a lower bound of the
+// K-th largest; the main kernel gives a wavefront one batch row (lane l holds the weight rows l and l + 64 of the
+// tile), lists the row's marks and walks them against a transposed copy of the tile's weights, so an unmarked input
+// costs nothing.  Same bits as the kernels that evaluate every term
 // (core/cuda/sort_neuron.cu:16-314, core/cuda/inf_dist_cuda.cu:110-212 semantics).
 //
 // This orientation is queued behind the per-weight-row tables of sort_cols.h and shares their probe: its kernels
@@ -30,9 +30,8 @@ enum RowCandsForm {
 // bytes of workspace row_cands_forward needs
 size_t row_cands_workspace(int form, int B, int CO, int CI, int K);
 
-// True when this build has a main kernel for (form, K): values for every K, interval bounds for K <= 18, positions
-// for K <= 12 (beyond, the top-K lists of a wavefront's row do not fit its registers), the l-inf form for the depths
-// of max_cols_depth.
+// True when this build has a main kernel for (form, K): the sort-neuron forms for K = 2 .. 25, the l-inf form for the
+// depths of max_cols_depth.
 bool row_cands_supported(int form, int K);
 
 // Queues the tables per batch row and the main kernel that works from them.

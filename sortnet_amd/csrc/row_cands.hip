@@ -12,9 +12,6 @@ constexpr int kChunk = kRowCandsChunk;
 constexpr int kTileW = 128;          // weight rows of a tile: 64 lanes x 2
 constexpr int kBPad = 128;           // batch rows are padded to a multiple of this in the tables
 constexpr int kMaxPer = 32;          // most chunks a slice of the table kernels covers
-constexpr int kWaves = 16;           // wavefronts of a workgroup of the main kernel
-constexpr int kSeg = 64;             // chunks whose table words the main kernel keeps in LDS at a time
-constexpr int kWRow = 2 * 64 + 4;    // floats per input in the staged weight tile: 64 lanes x (w, w')
 
 inline size_t align256(size_t b) { return (b + 255) / 256 * 256; }
 inline int tiles_w(int M) { return (M + kTileW - 1) / kTileW; }
@@ -25,20 +22,15 @@ inline int slices_of(int NCH) {
     return s < NCH ? s : NCH;
 }
 
-// The value and interval forms of the sort neuron walk a transposed copy of the weights, wavefront by wavefront,
-// without LDS tiles or barriers (rt_main_kernel); the forms with positions and the l-inf forms stage tiles
-// (rc_main_kernel).
-constexpr bool walks_transposed(int form) { return form == kRowsSortValues || form == kRowsSortInterval; }
-
 struct Carve {
     float* wr;        // [T][2][N]  per tile of weight rows and input: min w, max w over the rows that keep the input
     float* lists;     // [T][slices][nw][K][Bp]  K largest chunk maxima of the lower bounds of a batch row's terms within a slice
     float* low;       // [T][nw][Bp]  K-th largest of them over all slices: upper list, lower list
-    uint32_t* bits;   // [T][NCH][Bp] bit i of a word = input 32 c + i may be among the K largest of that batch row in that tile
+    uint32_t* bits;   // [T][Bp][NCH] bit i of a word = input 32 c + i may be among the K largest of that batch row in that tile
     uint32_t* partial;            // marks per wavefront of the table kernel
     unsigned long long* count;    // [0] marks, [1] every-term kernels run, [2] this table's kernel runs, [3] marks per weight row (copy), [4] outputs to recompute
     uint32_t* fix;    // [B * M] outputs of the masked l-inf form whose bound did not hold (recomputed from every input)
-    float* wt;        // [T][N][128] the weights of a tile, one 512-byte row per input (forms walked without LDS tiles)
+    float* wt;        // [T][N][128] the weights of a tile, one 512-byte row per input (dropped weights undefined)
 };
 
 size_t carve_sizes(int form, int B, int M, int N, int K, size_t (&sz)[8]) {
@@ -51,7 +43,7 @@ size_t carve_sizes(int form, int B, int M, int N, int K, size_t (&sz)[8]) {
     sz[4] = align256(Bp / 64 * slices * ((T + 3) / 4) * 4 * 4);
     sz[5] = 256;
     sz[6] = form == kRowsMax ? align256((size_t)B * M * 4) : 0;
-    sz[7] = walks_transposed(form) ? align256(T * N * kTileW * 4) : 0;
+    sz[7] = align256(T * N * kTileW * 4);
     size_t t = 0;
     for (size_t v : sz) t += v;
     return t;
@@ -82,9 +74,9 @@ __device__ __forceinline__ void repair(float& l, float& u) {
 // of a weight column do.  stat[0] = widths of the input columns over all batch tiles, stat[1] = widths of the same
 // columns over 16 weight rows.
 // `ratio` is kProbeRatio for the sort-neuron forms.  The l-inf form asks for more (kProbeRatioMax): its kernel only pays
-// below about 4 % of marks, and on inputs spread evenly over their range the marked share is about 1.5 / (that ratio), so
+// below about 10 % of marks, and on inputs spread evenly over their range the marked share is about 1 / (that ratio), so
 // its tables are not even built unless the probe promises that few.
-constexpr float kProbeRatio = 2.5f, kProbeRatioMax = 40.f;
+constexpr float kProbeRatio = 2.5f, kProbeRatioMax = 10.f;
 __device__ __forceinline__ bool rows_decide(const float* stat, int S, float ratio) {
     return stat[0] > ratio * (float)S * stat[1];
 }
@@ -116,43 +108,32 @@ __device__ __forceinline__ void static_for(F&& f, std::integer_sequence<int, R..
 // Column ranges of the weights over a tile of 128 weight rows (WMASK: over the rows that keep the input; a column
 // that no row keeps, or that holds an undefined or infinite weight, becomes (-inf, +inf): no lower bound, always a
 // candidate).  64 inputs x 4 groups of 32 rows per workgroup.
-template <bool WMASK, bool WT = false>
+template <bool WMASK>
 __global__ void __launch_bounds__(256) rc_range_kernel(const float* __restrict__ w, const uint32_t* __restrict__ wkeep,
-                                                       int M, int N, int S, float* __restrict__ wr,
-                                                       const float* __restrict__ stat, float ratio,
-                                                       float* __restrict__ wt = nullptr) {
+                                                       int M, int N, int S, float* __restrict__ wr, float* __restrict__ wt,
+                                                       const float* __restrict__ stat, float ratio) {
     if (!rows_decide(stat, S, ratio)) return;
     __shared__ float part[4][3][64];
     const int nl = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int n = blockIdx.x * 64 + nl, t = blockIdx.y;
     const int r0 = t * kTileW + grp * (kTileW / 4);
-    const int r1 = r0 + kTileW / 4 < M ? r0 + kTileW / 4 : M;
     float lo = __builtin_inff(), hi = -__builtin_inff(), odd = 0.f;
-    if constexpr (WT) {
-        // WT: also the transposed copy, wt[(t N + n) 128 + row of the tile] (rows past the last: zero, not used)
-        static_assert(!WMASK, "the transposed copy is for the forms without a mask");
-        if (n < N) {
-            float v[kTileW / 4];
-            #pragma unroll
-            for (int i = 0; i < kTileW / 4; i++) v[i] = r0 + i < M ? w[(size_t)(r0 + i) * N + n] : 0.f;
-            #pragma unroll
-            for (int i = 0; i < kTileW / 4; i++) {
-                if (r0 + i < M) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); odd += v[i] - v[i]; }
+    if (n < N) {
+        float v[kTileW / 4];
+        #pragma unroll
+        for (int i = 0; i < kTileW / 4; i++) v[i] = r0 + i < M ? w[(size_t)(r0 + i) * N + n] : 0.f;
+        #pragma unroll
+        for (int i = 0; i < kTileW / 4; i++) {
+            bool kept = r0 + i < M;
+            if constexpr (WMASK) {
+                if (kept) kept = (wkeep[(size_t)(r0 + i) * (N / kChunk) + (n >> 5)] >> (n & 31)) & 1u;
             }
-            float4* dst = reinterpret_cast<float4*>(wt + ((size_t)t * N + n) * kTileW + grp * (kTileW / 4));
-            #pragma unroll
-            for (int i = 0; i < kTileW / 16; i++) dst[i] = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+            if (kept) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); odd += v[i] - v[i]; }
+            else if (WMASK) v[i] = __builtin_nanf("");
         }
-    } else if (n < N) {
-        #pragma unroll 4
-        for (int m = r0; m < r1; m++) {
-            bool kept = true;
-            if constexpr (WMASK) kept = (wkeep[(size_t)m * (N / kChunk) + (n >> 5)] >> (n & 31)) & 1u;
-            if (kept) {
-                const float v = w[(size_t)m * N + n];
-                lo = fminf(lo, v); hi = fmaxf(hi, v); odd += v - v;
-            }
-        }
+        float4* dst = reinterpret_cast<float4*>(wt + ((size_t)t * N + n) * kTileW + grp * (kTileW / 4));
+        #pragma unroll
+        for (int i = 0; i < kTileW / 16; i++) dst[i] = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
     }
     part[grp][0][nl] = lo; part[grp][1][nl] = hi; part[grp][2][nl] = odd;
     __syncthreads();
@@ -285,9 +266,9 @@ __global__ void __launch_bounds__(256) rc_merge_kernel(const float* __restrict__
 // rows of the tile reaches the bound of its list and is positive (the lists start at 0 and take larger values only;
 // an undefined bound or term compares false: an undefined term is left out of every list).  Marks counted per
 // wavefront.
-// BYROW: the words of a (tile, batch row) lie side by side over the chunks, bits[(t Bp + b) NCH + c] (rt_main_kernel
-// reads a row's words 64 at a time); otherwise those of a (tile, chunk) over the batch rows, bits[(t NCH + c) Bp + b].
-template <bool IV, bool XMASK, bool BYROW = false>
+// The words of a (tile, batch row) lie side by side over the chunks, bits[(t Bp + b) NCH + c]: the main kernel reads a
+// row's words 64 at a time.
+template <bool IV, bool XMASK>
 __global__ void __launch_bounds__(256) rc_bits_kernel(const float* __restrict__ xl, const float* __restrict__ xu,
                                                       const uint32_t* __restrict__ xkeep, const float* __restrict__ wr,
                                                       const float* __restrict__ low, int B, int N, int T, int Bp, int S,
@@ -365,8 +346,7 @@ __global__ void __launch_bounds__(256) rc_bits_kernel(const float* __restrict__ 
             }
             if (!valid) word = 0u;
             if constexpr (XMASK) word &= xkeep[(size_t)brow * NCH + c];
-            if constexpr (BYROW) bits[((size_t)t * Bp + b0 + r) * NCH + c] = word;
-            else bits[((size_t)t * NCH + c) * Bp + b0 + r] = word;
+            bits[((size_t)t * Bp + b0 + r) * NCH + c] = word;
             marks += __builtin_popcount(word);
         }
         __syncthreads();
@@ -405,312 +385,20 @@ __global__ void __launch_bounds__(1024) rc_sum_kernel(const uint32_t* __restrict
 }
 
 // ---- main kernel -------------------------------------------------------------------------------
-// A workgroup of 16 wavefronts owns 128 weight rows (lane l holds the rows l and l + 64 of the tile) and a group of
-// `rows` <= 16 TR batch rows, dealt evenly to its wavefronts (at most TR each).  The group size is chosen on the host
-// so that the workgroups fill whole rounds of the chip's compute units.  The inputs go by in stages of 64.  The
-// weight tile of a stage (128 x 64) goes through LDS, where an input's (w, w') of a lane is one 8-byte word; the
-// tiles of the next two stages are on their way while the current one is used.  A wavefront keeps the inputs of its
-// own rows in registers (lane i holds input i of the stage; the next stage's are fetched a stage ahead), so a marked
-// input's value reaches the terms as a lane read and no barrier stands between a wavefront and its inputs.  The table
-// words of 32 stages at a time are copied to LDS ahead of the loop over them; a stage nobody marks is not staged.  One
-// loop per batch row over that row's own marks, so that the top-K lists are only ever indexed with constants; the
-// marks are taken four at a time, the weights of all four requested before the first term is formed (the walk is
-// bound by the latency of its LDS reads otherwise).  The results are written along the weight rows as they are.
-constexpr int kStage = 2 * kChunk;   // inputs of a stage: two table words per batch row
-
-struct MainArgs {
-    const float* xl; const float* xu; const float* w;
-    const uint32_t* xkeep; const uint32_t* wkeep;   // factored mask (l-inf form), or null
-    const uint32_t* bits; const float* low;
-    unsigned long long* count;
-    uint32_t* fix;
-    int B, Bp, M, N;
-    int rows;                                        // batch rows of a workgroup
-    float q;
-    float* outL; float* outU; int* pos;
-};
-
-template <int FORM, int K, int TR, bool POS, bool MASKED>
-__global__ void __launch_bounds__(64 * kWaves, 1) rc_main_kernel(MainArgs a) {
-    if (a.count[2] == 0ull) return;
-    constexpr bool IV = FORM == kRowsSortInterval;
-    constexpr int ROWS = kWaves * TR;                 // most batch rows of a workgroup
-    constexpr int TILE = kStage * kWRow;              // floats of one buffer
-    extern __shared__ __attribute__((aligned(16))) float smem[];
-    uint32_t* wb = reinterpret_cast<uint32_t*>(smem + 2 * TILE);   // [kSeg][ROWS]
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // this wavefront's lists of the marked inputs of its rows in one stage (two entries past a full list are read)
-    // (off: byte offset of the input's weights in the tile; un: the row's upper end in the interval form, the input's
-    // number within the stage, as bits, in the others)
-    struct Entry { int off; float l, un; };
-    Entry* marks = reinterpret_cast<Entry*>(wb + kSeg * ROWS) + wave * (TR * kStage + 2);
-    const int B = a.B, Bp = a.Bp, M = a.M, N = a.N, NCH = N / kChunk;
-    const int rows = a.rows, BG = (B + rows - 1) / rows;
-    // Workgroups go to the chip's eight dies in turn, each with a cache of its own: consecutive (tile, batch rows)
-    // pairs are dealt out so that the workgroups of a tile of weight rows, which all stream that tile, share a die
-    int item = blockIdx.x;
-    if (gridDim.x % 8 == 0) item = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-    const int bg = item % BG, t = item / BG;
-    const int m0 = t * kTileW, b0 = bg * rows;
-    // this wavefront's rows of the group: r_lo .. r_lo + nr - 1 (nr <= TR)
-    const int r_lo = wave * rows / kWaves, nr = (wave + 1) * rows / kWaves - r_lo;
-    auto wt = [&](int buf) { return smem + buf * TILE; };
-
-    // the lists of marks start as zeros: entries past the end of a list are read (and not used)
-    for (int i = lane; i < (TR * kStage + 2) * 3; i += 64) reinterpret_cast<uint32_t*>(marks)[i] = 0u;
-    float inf = __builtin_inff();
-    asm volatile("" : "+v"(inf));                     // (see insert_value)
-
-    // state of the wavefront's rows x the lane's two weight rows
-    constexpr bool LISTS = FORM != kRowsMax;
-    float hi[TR][2][LISTS ? K : 1];
-    float lo[IV ? TR : 1][2][IV ? K : 1];
-    int idx[(FORM == kRowsSortPos || (FORM == kRowsMax && POS)) ? TR : 1][2][FORM == kRowsSortPos ? K : 1];
-    #pragma unroll
-    for (int r = 0; r < TR; r++) {
-        #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            if constexpr (LISTS) {
-                #pragma unroll
-                for (int k = 0; k < K; k++) {
-                    hi[r][j][k] = 0.f;
-                    if constexpr (IV) lo[r][j][k] = 0.f;
-                    if constexpr (FORM == kRowsSortPos) idx[r][j][k] = 0;
-                }
-            } else {
-                hi[r][j][0] = kEps;
-                if constexpr (POS) idx[r][j][0] = 0;
-            }
-        }
-    }
-
-    // word of (chunk c, batch row b0 + i): bw[c * Bp + i]; rows past the batch, up to the padded count, hold zero
-    const uint32_t* __restrict__ bw = a.bits + (size_t)t * NCH * Bp + b0;
-    int seg_lo = 0;                                   // first chunk (of 32 inputs) whose words are in LDS
-    auto marked = [&](int st) {
-        const uint32_t* q = wb + (2 * st - seg_lo) * ROWS;
-        uint32_t v = lane < rows ? (q[lane] | q[ROWS + lane]) : 0u;
-        if constexpr (ROWS > 64) v |= lane + 64 < rows ? (q[lane + 64] | q[ROWS + lane + 64]) : 0u;
-        return __builtin_amdgcn_ballot_w64(v != 0u) != 0ull;
-    };
-    // weight tile: work-item (frow, fq) carries inputs 4 fq .. + 3 and 32 + 4 fq .. + 3 of weight row frow of the stage
-    const int frow = tid >> 3, fq = tid & 7;
-    const int fm = m0 + frow < M ? m0 + frow : M - 1;
-    struct Piece { float4 a, b; uint32_t ka, kb; };
-    auto fetch = [&](int st, bool need, Piece& p) __attribute__((always_inline)) {
-        const int c0 = 2 * st, c1 = 2 * st + 1 < NCH ? 2 * st + 1 : 2 * st;   // the last stage may be half a stage
-        const float* src = a.w + (size_t)fm * N + 4 * fq;
-        p.a = *reinterpret_cast<const float4*>(need ? src + (size_t)c0 * kChunk : a.w);
-        p.b = *reinterpret_cast<const float4*>(need ? src + (size_t)c1 * kChunk : a.w);
-        if constexpr (MASKED) {
-            p.ka = need ? a.wkeep[(size_t)fm * NCH + c0] : 0u;
-            p.kb = need ? a.wkeep[(size_t)fm * NCH + c1] : 0u;
-        }
-    };
-    auto stash = [&](int buf, const Piece& p) __attribute__((always_inline)) {
-        float4 u = p.a, v = p.b;
-        if constexpr (MASKED) {
-            // dropped weights become undefined: their terms never compare greater
-            const float qn = __builtin_nanf("");
-            const uint32_t ba = p.ka >> (4 * fq), bb = p.kb >> (4 * fq);
-            u.x = (ba & 1u) ? u.x : qn; u.y = (ba & 2u) ? u.y : qn; u.z = (ba & 4u) ? u.z : qn; u.w = (ba & 8u) ? u.w : qn;
-            v.x = (bb & 1u) ? v.x : qn; v.y = (bb & 2u) ? v.y : qn; v.z = (bb & 4u) ? v.z : qn; v.w = (bb & 8u) ? v.w : qn;
-        }
-        // weight row frow belongs to lane frow % 64, slot frow / 64
-        float* dw = wt(buf) + (4 * fq) * kWRow + 2 * (frow & 63) + (frow >> 6);
-        dw[0] = u.x; dw[kWRow] = u.y; dw[2 * kWRow] = u.z; dw[3 * kWRow] = u.w;
-        dw += kChunk * kWRow;
-        dw[0] = v.x; dw[kWRow] = v.y; dw[2 * kWRow] = v.z; dw[3 * kWRow] = v.w;
-    };
-    // inputs of the wavefront's rows: lane i holds input i of the stage (repaired, dropped inputs undefined)
-    uint32_t xoff[TR];   // (B x N stays below 2^31 elements)
-    #pragma unroll
-    for (int r = 0; r < TR; r++) {
-        const int row = b0 + r_lo + (r < nr ? r : 0);
-        xoff[r] = (uint32_t)(row < B ? row : B - 1) * (uint32_t)N;
-    }
-    auto load_x = [&](int st, float (&xl_)[TR], float (&xu_)[IV ? TR : 1]) __attribute__((always_inline)) {
-        int n = st * kStage + lane;
-        const bool in = n < N;
-        n = in ? n : N - 1;
-        #pragma unroll
-        for (int r = 0; r < TR; r++) {
-            float l = a.xl[xoff[r] + n];
-            if constexpr (IV) {
-                float u = a.xu[xoff[r] + n];
-                repair(l, u);
-                xu_[r] = u;
-            }
-            if constexpr (MASKED) {
-                const uint32_t kx = a.xkeep[xoff[r] / (uint32_t)kChunk + (uint32_t)(n >> 5)];   // (N is a multiple of 32)
-                l = ((kx >> (n & 31)) & 1u) ? l : __builtin_nanf("");
-            }
-            xl_[r] = l;
-        }
-    };
-    // one marked input of row r: ww = the lane's two weights, (xa, xb) = the row's value and the input's number within
-    // the stage as bits (or its l and u), n0 = the first input of the stage
-    auto term = [&](auto R, const float2& ww, float xa, float xb, int n0) __attribute__((always_inline)) {
-        constexpr int r = decltype(R)::value;
-        [[maybe_unused]] const int n = n0 + __float_as_int(xb);   // (forms without an interval)
-        if constexpr (IV) {
-            const float a1 = ww.x - xa, a2 = xb - ww.x, b1 = ww.y - xa, b2 = xb - ww.y;
-            insert_value<K>(lo[r][0], -fminf(a1, a2), inf);
-            insert_value<K>(hi[r][0], fmaxf(a1, a2), inf);
-            insert_value<K>(lo[r][1], -fminf(b1, b2), inf);
-            insert_value<K>(hi[r][1], fmaxf(b1, b2), inf);
-        } else {
-            const float d0 = xa - ww.x, d1 = xa - ww.y;
-            if constexpr (FORM == kRowsSortValues) {
-                insert_value<K>(hi[r][0], fabsf(d0), inf);
-                insert_value<K>(hi[r][1], fabsf(d1), inf);
-            } else if constexpr (FORM == kRowsSortPos) {
-                // the marks of a row go by in ascending input order: the ordered insertion of the scan over
-                // all inputs (core/cuda/sort_neuron.cu:108-113, 176-185), ties included
-                if (fabsf(d0) > hi[r][0][0]) topk_insert<K>(hi[r][0], idx[r][0], fabsf(d0), n | (d0 >= 0.f ? 0 : (int)kSign));
-                if (fabsf(d1) > hi[r][1][0]) topk_insert<K>(hi[r][1], idx[r][1], fabsf(d1), n | (d1 >= 0.f ? 0 : (int)kSign));
-            } else {
-                // running maximum; only a larger term replaces it, so the first of equal terms keeps the
-                // position (core/cuda/inf_dist_cuda.cu:176-190); an undefined term never compares greater
-                const bool g0 = fabsf(d0) > hi[r][0][0], g1 = fabsf(d1) > hi[r][1][0];
-                hi[r][0][0] = g0 ? fabsf(d0) : hi[r][0][0];
-                hi[r][1][0] = g1 ? fabsf(d1) : hi[r][1][0];
-                if constexpr (POS) {
-                    idx[r][0][0] = g0 ? (n | (d0 >= 0.f ? 0 : (int)kSign)) : idx[r][0][0];
-                    idx[r][1][0] = g1 ? (n | (d1 >= 0.f ? 0 : (int)kSign)) : idx[r][1][0];
-                }
-            }
-        }
-    };
-    // The marks of the wavefront's rows in the stage are first compacted by the lanes themselves: lane i, which holds
-    // input i, finds its place among the marked lanes of a row with a bit count and posts (i, value) in that row's
-    // list.  The walk over a list then costs one broadcast read per mark and no bit scanning (the scalar unit, which
-    // all sixteen wavefronts share, only keeps the loop's count), and it is software-pipelined: while the terms of
-    // mark k are formed, the weights of mark k + 1 and the entry of mark k + 2 are on their way (an entry must have
-    // arrived before its weights can be asked for: two dependent LDS reads per mark otherwise).  The rows' lists lie
-    // end to end, so the pipeline is filled once per stage and runs on across the rows.
-    auto compute = [&](int buf, int st, const float (&xl_)[TR], const float (&xu_)[IV ? TR : 1]) __attribute__((always_inline)) {
-        const char* W = reinterpret_cast<const char*>(wt(buf) + 2 * lane);
-        const uint32_t* words = wb + (2 * st - seg_lo) * ROWS + r_lo;
-        uint32_t wa[TR], wc[TR];
-        #pragma unroll
-        for (int r = 0; r < TR; r++) { wa[r] = words[r < nr ? r : 0]; wc[r] = words[ROWS + (r < nr ? r : 0)]; }
-        int end[TR];                                      // one past row r's last entry in the wavefront's list
-        __builtin_amdgcn_wave_barrier();                 // the walk of the stage before this one has read its entries
-        int filled = 0;
-        #pragma unroll
-        for (int r = 0; r < TR; r++) {
-            uint32_t mlo = 0u, mhi = 0u;
-            if (r < nr) { mlo = (uint32_t)__builtin_amdgcn_readfirstlane(wa[r]); mhi = (uint32_t)__builtin_amdgcn_readfirstlane(wc[r]); }
-            const uint32_t mine = ((lane < 32 ? mlo : mhi) >> (lane & 31)) & 1u;
-            const int rank = (int)__builtin_amdgcn_mbcnt_hi(mhi, __builtin_amdgcn_mbcnt_lo(mlo, 0u));
-            if (mine) marks[filled + rank] = Entry{lane * (kWRow * 4), xl_[r], IV ? xu_[IV ? r : 0] : __int_as_float(lane)};
-            filled += __builtin_popcount(mlo) + __builtin_popcount(mhi);
-            end[r] = filled;
-        }
-        __builtin_amdgcn_wave_barrier();                 // LDS operations of one wavefront complete in order
-        if (filled == 0) return;
-        const int n0 = st * kStage;
-        // (past the end of the list the entries are stale, from an earlier stage or the zeros the lists start with:
-        // their offsets lie in the tile and what is read through them is not used)
-        Entry e = marks[0], e1 = marks[1];
-        float2 ww = *reinterpret_cast<const float2*>(W + e.off);
-        int k = 0;
-        static_for([&](auto R) __attribute__((always_inline)) {
-            constexpr int r = decltype(R)::value;
-            for (; k < end[r]; k++) {
-                const float2 w1 = *reinterpret_cast<const float2*>(W + e1.off);
-                const Entry e2 = marks[k + 2];
-                term(R, ww, e.l, e.un, n0);
-                e = e1; ww = w1; e1 = e2;
-            }
-        }, std::make_integer_sequence<int, TR>{});
-    };
-
-    float xc[TR], xcu[IV ? TR : 1], xn[TR], xnu[IV ? TR : 1];
-    for (; seg_lo < NCH; seg_lo += kSeg) {
-        const int seg_hi = seg_lo + kSeg < NCH ? seg_lo + kSeg : NCH;      // chunks [seg_lo, seg_hi), seg_lo even
-        const int st_lo = seg_lo / 2, st_hi = (seg_hi + 1) / 2;
-        __syncthreads();
-        for (int e = tid; e < kSeg * ROWS; e += 64 * kWaves) {
-            const int i = e % ROWS, c = seg_lo + e / ROWS;
-            wb[e] = (i < rows && c < seg_hi) ? bw[(size_t)c * Bp + i] : 0u;
-        }
-        __syncthreads();
-        // stage st is used from LDS while the pieces of stages st + 1 and st + 2 are on their way
-        Piece pa, pb;
-        pa.ka = pa.kb = pb.ka = pb.kb = 0u;
-        bool n0 = marked(st_lo), n1 = st_lo + 1 < st_hi ? marked(st_lo + 1) : false;
-        fetch(st_lo, n0, pa);
-        fetch(st_lo + 1 < st_hi ? st_lo + 1 : st_lo, n1, pb);
-        load_x(st_lo, xc, xcu);
-        if (n0) stash(0, pa);
-        __syncthreads();
-        for (int st = st_lo; st < st_hi; st += 2) {
-            const bool n2 = st + 2 < st_hi ? marked(st + 2) : false;
-            fetch(st + 2 < st_hi ? st + 2 : st, n2, pa);
-            load_x(st + 1 < st_hi ? st + 1 : st, xn, xnu);
-            if (n0) compute(0, st, xc, xcu);
-            if (n1) stash(1, pb);
-            __syncthreads();
-            if (st + 1 >= st_hi) break;
-            const bool n3 = st + 3 < st_hi ? marked(st + 3) : false;
-            fetch(st + 3 < st_hi ? st + 3 : st, n3, pb);
-            load_x(st + 2 < st_hi ? st + 2 : st, xc, xcu);
-            if (n1) compute(1, st + 1, xn, xnu);
-            if (n2) stash(0, pa);
-            __syncthreads();
-            n0 = n2; n1 = n3;
-        }
-    }
-
-    const size_t plane = (size_t)B * M;
-    static_for([&](auto R) __attribute__((always_inline)) {
-        constexpr int r = decltype(R)::value;
-        const int row = b0 + r_lo + r;
-        if (r < nr && row < B) {
-            float bound = 0.f;
-            if constexpr (MASKED) bound = a.low[(size_t)t * Bp + row];   // wave-uniform
-            #pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const int col = m0 + lane + 64 * j;
-                if (col < M) {
-                    const size_t o = (size_t)row * M + col;
-                    if constexpr (FORM == kRowsSortValues) {
-                        a.outU[o] = geo_sum<K>(hi[r][j], a.q);
-                    } else if constexpr (IV) {
-                        a.outL[o] = geo_sum<K>(lo[r][j], a.q);
-                        a.outU[o] = geo_sum<K>(hi[r][j], a.q);
-                    } else if constexpr (FORM == kRowsSortPos) {
-                        a.outU[o] = geo_sum<K>(hi[r][j], a.q);
-                        #pragma unroll
-                        for (int k = 0; k < K; k++) a.pos[(size_t)(K - 1 - k) * plane + o] = idx[r][j][k];   // plane 0 = largest
-                    } else {
-                        a.outU[o] = hi[r][j][0];
-                        if constexpr (POS) a.pos[o] = idx[r][j][0];
-                        if constexpr (MASKED) {
-                            // The bound rests on K inputs that the batch row keeps; a weight row that keeps none of them
-                            // may have its maximum at an unmarked input: such an output is recomputed from every input.
-                            if (!(hi[r][j][0] >= bound)) a.fix[atomicAdd(a.count + 4, 1ull)] = (uint32_t)o;
-                        }
-                    }
-                }
-            }
-        }
-    }, std::make_integer_sequence<int, TR>{});
-}
-
-// ---- main kernel without tiles -------------------------------------------------------------------
-// Values and interval bounds of the sort neuron.  A wavefront takes one batch row at a time against the tile's 128
-// weight rows (lane l holds the rows l and l + 64): it reads the row's table words 64 chunks at a time, lists the
-// marked inputs in LDS and walks the list four marks at a time with the loads of the next four in flight: lane l
-// fetches the number and the row's value(s) of mark l % 4 (read back lane by lane, so they are scalar operands of the
-// terms), every lane its two weights from the transposed copy (two coalesced 256-byte loads per mark).  No tile is
-// staged and no barrier is met, so a wavefront with many marks holds nobody up; the tile's transposed weights
-// (2.6 MB at 5120 inputs) stay in the cache of the die its workgroups are dealt to.  Every load is issued
-// unconditionally (groups past the end of the list repeat its last mark and are not used), so that the waits the
-// compiler places cover exactly the group that is used next.
+// A wavefront takes one batch row at a time against the tile's 128 weight rows (lane l holds the rows l and l + 64):
+// it reads the row's table words 64 chunks at a time, lists the marked inputs in LDS and walks the list four marks at
+// a time with the loads of the next four in flight: lane l fetches the number and the row's value(s) of mark l % 4
+// (read back lane by lane, so they are scalar operands of the terms), every lane its two weights from the transposed
+// copy (two coalesced 256-byte loads per mark).  No tile is staged and no barrier is met, so a wavefront with many
+// marks holds nobody up; a workgroup is eight wavefronts = eight batch rows, and the workgroups of a tile are dealt to
+// one die, so that the tile's transposed weights (2.6 MB at 5120 inputs) stay in that die's cache while its 64
+// resident workgroups walk them.  Every load is issued unconditionally (groups past the end of the list repeat its last
+// mark and are not used), so that the waits the compiler places cover exactly the group that is used next.
+// Forms: top-K lists of values (branch-free median insertion), of both interval bounds, of values with the input
+// numbers (the reference's ordered insertion: the marks go by in ascending input order), and the l-inf distance (the
+// difference of largest magnitude and, optionally, its input; under the factored mask the dropped weights of the
+// transposed copy are undefined, the table holds no input the batch row drops, and an output that ends below the bound
+// its marks were taken against is listed for rc_fix_kernel).
 constexpr int kRtWaves = 8;          // wavefronts of a workgroup
 constexpr int kRtRows = 1;           // batch rows a wavefront takes, one after the other
 constexpr int kRtBatch = 64;         // chunks whose table words a wavefront reads at a time, one per lane
@@ -718,16 +406,20 @@ constexpr int kRtListCap = 2304;     // entries of a wavefront's list of marked 
 
 struct RtArgs {
     const float* xl; const float* xu; const float* wt;
-    const uint32_t* bits;
-    const unsigned long long* count;
+    const uint32_t* bits; const float* low;
+    unsigned long long* count;
+    uint32_t* fix;
     int B, Bp, M, N;
     float q;
-    float* outL; float* outU;
+    float* outL; float* outU; int* pos;
 };
 
-template <int K, bool IV>
+template <int FORM, int K, bool POS, bool MASKED>
 __global__ void __launch_bounds__(64 * kRtWaves) rt_main_kernel(RtArgs a) {
     if (a.count[2] == 0ull) return;
+    constexpr bool IV = FORM == kRowsSortInterval;
+    constexpr bool LISTS = FORM != kRowsMax;
+    constexpr bool IDX = FORM == kRowsSortPos || (FORM == kRowsMax && POS);
     __shared__ uint16_t list[kRtWaves][kRtListCap];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -741,21 +433,34 @@ __global__ void __launch_bounds__(64 * kRtWaves) rt_main_kernel(RtArgs a) {
     uint16_t* mine = list[wave];
     float inf = __builtin_inff();
     asm volatile("" : "+v"(inf));                     // (see insert_value)
+    const size_t plane = (size_t)B * M;
 
     for (int rr = 0; rr < kRtRows; rr++) {
         const int b = (bg * kRtWaves + wave) * kRtRows + rr;
         if (b >= B) break;   // wave-uniform; the rows of a wavefront ascend
-        float hi[2][K], lo[IV ? 2 : 1][IV ? K : 1];
+        // state of the row x the lane's two weight rows: top-K lists (ascending), or the difference of largest magnitude
+        float hi[2][LISTS ? K : 1], lo[IV ? 2 : 1][IV ? K : 1];
+        int idx[IDX ? 2 : 1][FORM == kRowsSortPos ? K : 1];
         #pragma unroll
-        for (int k = 0; k < K; k++) {
-            hi[0][k] = hi[1][k] = 0.f;
-            if constexpr (IV) lo[0][k] = lo[1][k] = 0.f;
+        for (int j = 0; j < 2; j++) {
+            if constexpr (LISTS) {
+                #pragma unroll
+                for (int k = 0; k < K; k++) {
+                    hi[j][k] = 0.f;
+                    if constexpr (IV) lo[j][k] = 0.f;
+                    if constexpr (FORM == kRowsSortPos) idx[j][k] = 0;
+                }
+            } else {
+                hi[j][0] = kEps;
+                if constexpr (POS) idx[j][0] = 0;
+            }
         }
         const uint32_t* __restrict__ rowbits = a.bits + ((size_t)t * a.Bp + b) * NCH;
         const float* __restrict__ xlrow = a.xl + (size_t)b * N;
         const float* __restrict__ xurow = IV ? a.xu + (size_t)b * N : nullptr;
         int cnt = 0;   // marks in the list
         float xreg[2], ureg[IV ? 2 : 1];
+        int nreg[IDX ? 2 : 1];
         float wa[2][4], wb[2][4];
         auto load = [&](int buf, int k0, int total) __attribute__((always_inline)) {
             int k = k0 + (lane & 3);
@@ -768,6 +473,7 @@ __global__ void __launch_bounds__(64 * kRtWaves) rt_main_kernel(RtArgs a) {
                 ureg[buf] = u;
             }
             xreg[buf] = l;
+            if constexpr (IDX) nreg[buf] = nn;
             #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int n = __builtin_amdgcn_readlane(nn, i);
@@ -789,8 +495,31 @@ __global__ void __launch_bounds__(64 * kRtWaves) rt_main_kernel(RtArgs a) {
                         insert_value<K>(lo[1], -fminf(b1, b2), inf);
                         insert_value<K>(hi[1], fmaxf(b1, b2), inf);
                     } else {
-                        insert_value<K>(hi[0], fabsf(xi - wa[buf][i]), inf);
-                        insert_value<K>(hi[1], fabsf(xi - wb[buf][i]), inf);
+                        const float d0 = xi - wa[buf][i], d1 = xi - wb[buf][i];
+                        [[maybe_unused]] int n = 0;
+                        if constexpr (IDX) n = __builtin_amdgcn_readlane(nreg[IDX ? buf : 0], i);
+                        if constexpr (FORM == kRowsSortValues) {
+                            insert_value<K>(hi[0], fabsf(d0), inf);
+                            insert_value<K>(hi[1], fabsf(d1), inf);
+                        } else if constexpr (FORM == kRowsSortPos) {
+                            // the marks of a row go by in ascending input order: the ordered insertion of the scan
+                            // over all inputs (core/cuda/sort_neuron.cu:108-113, 176-185), ties included
+                            if (fabsf(d0) > hi[0][0]) topk_insert<K>(hi[0], idx[0], fabsf(d0), n | (d0 >= 0.f ? 0 : (int)kSign));
+                            if (fabsf(d1) > hi[1][0]) topk_insert<K>(hi[1], idx[1], fabsf(d1), n | (d1 >= 0.f ? 0 : (int)kSign));
+                        } else {
+                            // running maximum; only a larger term replaces it, so the first of equal terms keeps the
+                            // position (core/cuda/inf_dist_cuda.cu:176-190); an undefined term (a weight the row of
+                            // the mask drops) never compares greater
+                            // (the difference itself is kept: its magnitude is the maximum, its sign the flag of
+                            // the position)
+                            const bool g0 = fabsf(d0) > fabsf(hi[0][0]), g1 = fabsf(d1) > fabsf(hi[1][0]);
+                            hi[0][0] = g0 ? d0 : hi[0][0];
+                            hi[1][0] = g1 ? d1 : hi[1][0];
+                            if constexpr (POS) {
+                                idx[0][0] = g0 ? n : idx[0][0];
+                                idx[1][0] = g1 ? n : idx[1][0];
+                            }
+                        }
                     }
                 }
             }
@@ -833,22 +562,47 @@ __global__ void __launch_bounds__(64 * kRtWaves) rt_main_kernel(RtArgs a) {
                 __builtin_amdgcn_wave_barrier();   // the reads of the list come before the next marks
             }
         }
+        float bound = 0.f;
+        if constexpr (MASKED) bound = a.low[(size_t)t * a.Bp + b];   // wave-uniform
         #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int col = t * kTileW + lane + 64 * j;
             if (col < M) {
                 const size_t o = (size_t)b * M + col;
-                a.outU[o] = geo_sum<K>(hi[j], a.q);
-                if constexpr (IV) a.outL[o] = geo_sum<K>(lo[j], a.q);
+                if constexpr (LISTS) {
+                    a.outU[o] = geo_sum<K>(hi[j], a.q);
+                    if constexpr (IV) a.outL[o] = geo_sum<K>(lo[j], a.q);
+                    if constexpr (FORM == kRowsSortPos) {
+                        #pragma unroll
+                        for (int k = 0; k < K; k++) a.pos[(size_t)(K - 1 - k) * plane + o] = idx[j][k];   // plane 0 = largest
+                    }
+                } else {
+                    a.outU[o] = fabsf(hi[j][0]);
+                    if constexpr (POS) a.pos[o] = idx[j][0] | (hi[j][0] >= 0.f ? 0 : (int)kSign);
+                    if constexpr (MASKED) {
+                        // The bound rests on K inputs that the batch row keeps; a weight row that keeps none of them
+                        // may have its maximum at an unmarked input: such an output is recomputed from every input.
+                        if (!(fabsf(hi[j][0]) >= bound)) a.fix[atomicAdd(a.count + 4, 1ull)] = (uint32_t)o;
+                    }
+                }
             }
         }
     }
 }
 
+struct FixArgs {
+    const float* xl; const float* w;
+    const uint32_t* xkeep; const uint32_t* wkeep;
+    const unsigned long long* count;
+    const uint32_t* fix;
+    int M, N;
+    float* outU; int* pos;
+};
+
 // Outputs of the masked l-inf form whose maximum stayed below the bound their marks were taken against: one
 // wavefront per output over every input that both rows keep, lowest input first among equal terms.
 template <bool POS>
-__global__ void __launch_bounds__(256) rc_fix_kernel(MainArgs a) {
+__global__ void __launch_bounds__(256) rc_fix_kernel(FixArgs a) {
     if (a.count[2] == 0ull) return;
     const unsigned long long total = a.count[4];
     const int lane = threadIdx.x & 63;
@@ -881,68 +635,20 @@ __global__ void __launch_bounds__(256) rc_fix_kernel(MainArgs a) {
     }
 }
 
-// Batch rows of a workgroup (at most `cap`): the workgroups stay for their whole run, one per compute unit, so the
-// launch proceeds in rounds of num_cus() workgroups and a partly filled last round costs a whole one.  Among the group
-// counts from the fewest that `cap` allows up to twice as many, the one that wastes least is taken (more groups also
-// stage the weight tiles more often, so the fewest wins ties).
-inline int rows_per_group(int B, int T, int cap) {
-    const long long cus = num_cus();
-    const int g_min = (B + cap - 1) / cap;
-    int best_g = g_min;
-    double best = 0.0;
-    for (int g = g_min; g <= 2 * g_min && g <= B; g++) {
-        const long long wgs = (long long)g * T, rounds = (wgs + cus - 1) / cus;
-        const int rows = (B + g - 1) / g;
-        // time ~ rounds x rows of a group (+ a fixed share per round for staging the tiles)
-        const double cost = (double)rounds * (rows + 0.15 * cap);
-        if (g == g_min || cost < best * 0.98) { best = cost; best_g = g; }
-    }
-    return (B + best_g - 1) / best_g;
-}
-
-template <int FORM, int K, int TR, bool POS, bool MASKED>
-int launch_main(MainArgs a, hipStream_t st) {
-    constexpr int ROWS = kWaves * TR;
-    constexpr size_t lds = (size_t)(2 * kStage * kWRow + kSeg * ROWS) * 4 + (size_t)kWaves * TR * (kStage + 2) * 12;
-    static_assert(lds <= 160 * 1024, "LDS of the main kernel");
-    auto kern = rc_main_kernel<FORM, K, TR, POS, MASKED>;
-    static bool attr_done = false;   // once per instantiation (benign if two threads both set it)
-    if (!attr_done) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
-            (void)hipGetLastError();
-            set_error("row_cands: cannot reserve %zu bytes of LDS", lds);
-            return SD_ERR_HIP;
-        }
-        attr_done = true;
-    }
-    const int T = tiles_w(a.M);
-    a.rows = rows_per_group(a.B, T, ROWS);
-    const int BG = (a.B + a.rows - 1) / a.rows;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(T * BG)), dim3(64 * kWaves), lds, st, a);
-    return check_launch("rc_main_kernel");
-}
-
-// Batch rows per wavefront: as many as keep the top-K lists of its rows x the lane's two weight rows (2 K registers per
-// row for values, 4 K with the second list or the positions) within about 64 of the 128 registers that 16 wavefronts
-// per compute unit allow; the rest go to the 24 staging registers of the two chunks in flight, the operands of four
-// marks and addresses (checked with the compiler's resource report: no instantiation spills).
-constexpr int tr_for(int form, int K) {
-    const int per = (form == kRowsSortValues ? 2 : 4) * K;
-    // (the ordered insertion with positions needs the most temporaries, the two-list form a few more than the values)
-    const int tr = (form == kRowsSortValues ? 64 : form == kRowsSortInterval ? 80 : 40) / per;
-    if (form == kRowsSortInterval && tr >= 4) return tr > 5 ? 4 : 3;   // (four and five rows of two lists spill)
-    return tr > 5 ? 5 : tr < 1 ? 1 : tr;
+template <int FORM, int K, bool POS, bool MASKED>
+int launch_rt(const RtArgs& a, hipStream_t st) {
+    const int T = tiles_w(a.M), BG = (a.B + kRtWaves * kRtRows - 1) / (kRtWaves * kRtRows);
+    hipLaunchKernelGGL((rt_main_kernel<FORM, K, POS, MASKED>), dim3((unsigned)(T * BG)), dim3(64 * kRtWaves), 0, st, a);
+    return check_launch("rt_main_kernel");
 }
 
 template <int FORM, int K>
 int run(const float* xl, const float* xu, const float* w, int B, int M, int N, float q, float* outL, float* outU, int* pos,
         const Carve& c, unsigned long long limit, const float* col_stat, const unsigned long long* col_count, hipStream_t st) {
     constexpr bool IV = FORM == kRowsSortInterval;
-    constexpr bool WT = walks_transposed(FORM);
     const int T = tiles_w(M), Bp = bpad_of(B), NCH = N / kChunk, slices = slices_of(NCH), S = (B + 127) / 128;
     int rc;
-    hipLaunchKernelGGL((rc_range_kernel<false, WT>), dim3((N + 63) / 64, T), dim3(256), 0, st, w, nullptr, M, N, S, c.wr, col_stat,
-                       kProbeRatio, WT ? c.wt : nullptr);
+    hipLaunchKernelGGL((rc_range_kernel<false>), dim3((N + 63) / 64, T), dim3(256), 0, st, w, nullptr, M, N, S, c.wr, c.wt, col_stat, kProbeRatio);
     if ((rc = check_launch("rc_range_kernel"))) return rc;
     const dim3 tgrid(Bp / 64, slices, (T + 3) / 4);
     hipLaunchKernelGGL((rc_low_kernel<K, IV, false>), tgrid, dim3(256), 0, st, xl, xu, nullptr, c.wr, B, N, T, Bp, S, c.lists, col_stat, kProbeRatio);
@@ -950,19 +656,12 @@ int run(const float* xl, const float* xu, const float* w, int B, int M, int N, f
     constexpr int nw = IV ? 2 : 1;
     hipLaunchKernelGGL((rc_merge_kernel<K>), dim3((Bp + 255) / 256, T * nw), dim3(256), 0, st, c.lists, slices, Bp, nw, S, c.low, col_stat, kProbeRatio);
     if ((rc = check_launch("rc_merge_kernel"))) return rc;
-    hipLaunchKernelGGL((rc_bits_kernel<IV, false, WT>), tgrid, dim3(256), 0, st, xl, xu, nullptr, c.wr, c.low, B, N, T, Bp, S, c.bits, c.partial, col_stat, kProbeRatio);
+    hipLaunchKernelGGL((rc_bits_kernel<IV, false>), tgrid, dim3(256), 0, st, xl, xu, nullptr, c.wr, c.low, B, N, T, Bp, S, c.bits, c.partial, col_stat, kProbeRatio);
     if ((rc = check_launch("rc_bits_kernel"))) return rc;
     hipLaunchKernelGGL(rc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)tgrid.x * tgrid.y * tgrid.z * 4, c.count, col_count, col_stat, S, limit, kProbeRatio);
     if ((rc = check_launch("rc_sum_kernel"))) return rc;
-    if constexpr (WT) {
-        RtArgs a{xl, xu, c.wt, c.bits, c.count, B, Bp, M, N, q, outL, outU};
-        const int BG = (B + kRtWaves * kRtRows - 1) / (kRtWaves * kRtRows);
-        hipLaunchKernelGGL((rt_main_kernel<K, IV>), dim3((unsigned)(T * BG)), dim3(64 * kRtWaves), 0, st, a);
-        return check_launch("rt_main_kernel");
-    } else {
-        MainArgs a{xl, xu, w, nullptr, nullptr, c.bits, c.low, c.count, c.fix, B, Bp, M, N, 0, q, outL, outU, pos};
-        return launch_main<FORM, K, tr_for(FORM, K), false, false>(a, st);
-    }
+    RtArgs a{xl, xu, c.wt, c.bits, c.low, c.count, c.fix, B, Bp, M, N, q, outL, outU, pos};
+    return launch_rt<FORM, K, false, false>(a, st);
 }
 
 template <int K, bool MASKED>
@@ -971,7 +670,7 @@ int run_max(const float* x, const float* w, const uint32_t* xkeep, const uint32_
             float ratio, hipStream_t st) {
     const int T = tiles_w(M), Bp = bpad_of(B), NCH = N / kChunk, slices = slices_of(NCH), S = (B + 127) / 128;
     int rc;
-    hipLaunchKernelGGL((rc_range_kernel<MASKED>), dim3((N + 63) / 64, T), dim3(256), 0, st, w, wkeep, M, N, S, c.wr, col_stat, ratio);
+    hipLaunchKernelGGL((rc_range_kernel<MASKED>), dim3((N + 63) / 64, T), dim3(256), 0, st, w, wkeep, M, N, S, c.wr, c.wt, col_stat, ratio);
     if ((rc = check_launch("rc_range_kernel"))) return rc;
     const dim3 tgrid(Bp / 64, slices, (T + 3) / 4);
     hipLaunchKernelGGL((rc_low_kernel<K, false, MASKED>), tgrid, dim3(256), 0, st, x, nullptr, xkeep, c.wr, B, N, T, Bp, S, c.lists, col_stat, ratio);
@@ -982,13 +681,13 @@ int run_max(const float* x, const float* w, const uint32_t* xkeep, const uint32_
     if ((rc = check_launch("rc_bits_kernel"))) return rc;
     hipLaunchKernelGGL(rc_sum_kernel, dim3(1), dim3(1024), 0, st, c.partial, (size_t)tgrid.x * tgrid.y * tgrid.z * 4, c.count, col_count, col_stat, S, limit, ratio);
     if ((rc = check_launch("rc_sum_kernel"))) return rc;
-    MainArgs a{x, nullptr, w, xkeep, wkeep, c.bits, c.low, c.count, c.fix, B, Bp, M, N, 0, 0.f, nullptr, y, pos};
-    // (four rows per wavefront: their mark lists share the LDS with the weight tiles)
-    if (pos) rc = launch_main<kRowsMax, 1, 4, true, MASKED>(a, st);
-    else rc = launch_main<kRowsMax, 1, 4, false, MASKED>(a, st);
+    RtArgs a{x, nullptr, c.wt, c.bits, c.low, c.count, c.fix, B, Bp, M, N, 0.f, nullptr, y, pos};
+    if (pos) rc = launch_rt<kRowsMax, 1, true, MASKED>(a, st);
+    else rc = launch_rt<kRowsMax, 1, false, MASKED>(a, st);
     if (rc || !MASKED) return rc;
-    if (pos) hipLaunchKernelGGL((rc_fix_kernel<true>), dim3(256), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((rc_fix_kernel<false>), dim3(256), dim3(256), 0, st, a);
+    const FixArgs f{x, w, xkeep, wkeep, c.count, c.fix, M, N, y, pos};
+    if (pos) hipLaunchKernelGGL((rc_fix_kernel<true>), dim3(256), dim3(256), 0, st, f);
+    else hipLaunchKernelGGL((rc_fix_kernel<false>), dim3(256), dim3(256), 0, st, f);
     return check_launch("rc_fix_kernel");
 }
 
@@ -1002,8 +701,8 @@ size_t row_cands_workspace(int form, int B, int CO, int CI, int K) {
 bool row_cands_supported(int form, int K) {
     switch (form) {
         case kRowsSortValues: return K >= 2 && K <= 25;
-        case kRowsSortInterval: return K >= 2 && K <= 18;
-        case kRowsSortPos: return K >= 2 && K <= 12;
+        case kRowsSortInterval: return K >= 2 && K <= 25;
+        case kRowsSortPos: return K >= 2 && K <= 25;
         case kRowsMax: return K == 1 || K == 8 || K == 12 || K == 16 || K == 20 || K == 24;
     }
     return false;
@@ -1023,7 +722,7 @@ int row_cands_forward(int form, const float* xl, const float* xu, const float* w
         set_error("row_cands_forward: shape or form not supported");
         return SD_ERR_ARG;
     }
-    if (walks_transposed(form) && CI > 65536) {   // (16-bit input numbers in the lists of marks)
+    if (CI > 65536) {   // (16-bit input numbers in the lists of marks)
         set_error("row_cands_forward: rows of more than 65536 inputs");
         return SD_ERR_ARG;
     }
@@ -1042,14 +741,14 @@ int row_cands_forward(int form, const float* xl, const float* xu, const float* w
         case kRowsSortInterval:
             switch (K) {
 #define X(k) case k: return run<kRowsSortInterval, k>(xl, xu, w, B, CO, CI, q, outL, outU, nullptr, c, limit, col_stat, col_count, st);
-                SD_ROWS_K18(X)
+                SD_ROWS_K25(X)
 #undef X
             }
             break;
         case kRowsSortPos:
             switch (K) {
 #define X(k) case k: return run<kRowsSortPos, k>(xl, nullptr, w, B, CO, CI, q, outL, outU, pos, c, limit, col_stat, col_count, st);
-                SD_ROWS_K12(X)
+                SD_ROWS_K25(X)
 #undef X
             }
             break;

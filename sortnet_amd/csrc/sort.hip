@@ -161,14 +161,14 @@ static void sort_cols_report(const FwdArgs& a, int site, int B, int CO, int CI, 
 
 // Largest share of marked (tile of 128 weight rows, batch row, input) triples at which the kernel of the tables per
 // batch row runs.  Measured per 512 x 5120 x 5120 layer at K = 10 on inputs in [0, 1] against weights ~ N(0, 1/N)
-// (7.2 % marked): values 0.75 ms against 1.9 ms for every term, interval bounds 1.24 against 3.3, values with positions
-// 2.1 against 2.6; 0.2 ms of that are tables and staging, the rest grows with the marks.
-constexpr float kSortRowsCap = 0.12f;
-// Smallest layers (in terms) given tables per batch row under the built-in limit: a workgroup of their main kernel
-// takes a whole compute unit for 16 to 48 batch rows x 128 weight rows, so small layers leave most of the chip idle
-// (128 x 3072 x 1024, 0.4 G terms: values 0.22 ms from tables against 0.15 ms for every term, interval bounds 0.25
-// against 0.32; 256 x 4096 x 2048, 2.1 G terms: 0.27 against 0.38 and 0.32 against 0.87)
-constexpr long long kSortRowsMinTerms = 1ll << 30, kSortRowsMinTermsInterval = 1ll << 28;
+// (7.2 % marked): values 0.58 ms against 1.9 ms for every term, interval bounds 0.95 against 3.3, values with positions
+// 0.83 against 2.4; 0.16 ms of that are tables and the transposed copy of the weights, the rest grows with the marks
+// (the two would meet at 25 to 30 %).
+constexpr float kSortRowsCap = 0.22f;
+// Smallest layers (in terms) given tables per batch row under the built-in limit (128 x 3072 x 1024, 0.4 G terms:
+// values 0.12 ms from tables against 0.14 ms for every term, with positions 0.16 against 0.19, interval bounds 0.17
+// against 0.32)
+constexpr long long kSortRowsMinTerms = 1ll << 28;
 
 // bytes of both tables' workspace for one call: per weight row first (with the probe and the counter the per-batch-row
 // tables read), per batch row behind it
@@ -188,7 +188,7 @@ static int queue_sort_cols(FwdArgs& a, int form, const float* xl, const float* x
     a.gate_above = 1;
     const long long terms = (long long)B * CO * CI;
     const bool rows = row_cands_supported(form, K) &&
-                      (density > 0.f || terms >= (form == kRowsSortInterval ? kSortRowsMinTermsInterval : kSortRowsMinTerms));
+                      (density > 0.f || terms >= kSortRowsMinTerms);
     if (rc || !rows) {
         // the every-term kernels read the flag behind the counter, as with both tables
         if (!rc) { a.gate = a.gate + 1; a.gate_limit = 0ull; }
