@@ -24,12 +24,15 @@ size_t bound_cols_workspace(int B, int CO, int CI);
 // term with the opposite condition on the same counter (*gate, *gate_limit).  outL / outU must be zero-filled:
 // the slices of the input range merge by atomic maximum.  (*gate)[1] (the word behind the gate) is 1 when the marks
 // per weight row are so few (below a sixteenth of the limit) that a kernel without LDS staging would serve better.
-// With packedL / packedU (B x CO words each, zero-filled) instead of outL / outU the table kernel leaves (value bits
-// << 32 | ~chunk of 32 inputs) per output, merged by atomic maximum, as the every-term kernel with chunk tracking does
-// (fwd_tile.h: store_chunk_winner), for resolve_bound_kernel to take values and positions from.
+// With packedL / packedU (B x CO words each, zero-filled) and posL / posU: the forward with positions.  The kernel of
+// the tables per weight row leaves (value bits << 32 | ~chunk of 32 inputs) per output in packedL / packedU, merged by
+// atomic maximum, as the every-term kernel with chunk tracking does (fwd_tile.h: store_chunk_winner), for
+// resolve_bound_kernel to take values and positions from; the kernel of the tables per batch row stores final values
+// and positions in outL / outU / posL / posU itself and sets (*gate)[2], which the resolve pass must be given as
+// FwdArgs::resolved.
 int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float* outL,
-                       float* outU, unsigned long long* packedL, unsigned long long* packedU, void* ws, float density,
-                       float density_rows, const unsigned long long** gate, unsigned long long* gate_limit,
-                       hipStream_t st);
+                       float* outU, unsigned long long* packedL, unsigned long long* packedU, int* posL, int* posU,
+                       void* ws, float density, float density_rows, const unsigned long long** gate,
+                       unsigned long long* gate_limit, hipStream_t st);
 
 }  // namespace sd

@@ -667,7 +667,8 @@ __global__ void __launch_bounds__(256) table_kernel(const float* __restrict__ xl
 
 // count[0] = marks of the table per weight row, count[1] = of the table per batch row (the one that was not built
 // counts as full), count[2] = 1 when neither is below its limit, which is what the every-term kernel waits for,
-// count[3] = 1 when the per-weight-row marks are below a sixteenth of their limit (for the caller's choice of kernel)
+// count[3] = 1 when the per-weight-row marks are below a sixteenth of their limit (for the caller's choice of kernel),
+// count[4] = 1 when the kernel of the tables per batch row runs (with positions it stores the final results itself)
 __global__ void __launch_bounds__(1024) sum_tables_kernel(const uint32_t* __restrict__ partial, size_t n_col,
                                                           size_t n_row, unsigned long long* __restrict__ count,
                                                           const float* __restrict__ stat, int S,
@@ -690,6 +691,7 @@ __global__ void __launch_bounds__(1024) sum_tables_kernel(const uint32_t* __rest
         count[2] = (c > limit_col && r > limit_row) ? 1ull : 0ull;
         // so few marks per weight row that staging tiles through LDS is most of the main kernel's time
         count[3] = c <= limit_col / 16 ? 1ull : 0ull;
+        count[4] = (c > limit_col && r <= limit_row) ? 1ull : 0ull;
     }
 }
 
@@ -701,9 +703,10 @@ __global__ void __launch_bounds__(1024) sum_tables_kernel(const uint32_t* __rest
 // tile (eight wavefronts = eight batch rows each) are dealt to one die, whose cache then holds the tile's transposed
 // weights.  Every load is issued unconditionally (groups past the end of the list repeat its last mark and are not
 // used).  One wavefront sees every input of its outputs, so the results are stored, not merged.
-// POS: the chunk of the mark that last improved a bound strictly is the chunk of the first input attaining it (the
-// marks go by in input order, and every input that attains a bound is marked); the (value bits << 32 | ~chunk) pairs
-// are left as the every-term kernel with chunk tracking leaves them, for resolve_bound_kernel.
+// POS: the mark that last improved a bound strictly is the first input attaining it (the marks go by in input order,
+// and every input that attains a bound is marked), so values and positions are stored as they are
+// (core/cuda/bound_inf_dist_cuda.cu:176-212: position = input | bit 31 when w - l > u - w; a lower bound that never
+// left its floor keeps 0xffffffff) and the resolve pass is told to skip the call (count[4]).
 constexpr int kWalkWaves = 8;        // wavefronts of a workgroup
 constexpr int kWalkBatch = 64;       // chunks whose table words a wavefront reads at a time, one per lane
 constexpr int kWalkListCap = 2304;   // entries of a wavefront's list of marked inputs (16-bit input numbers)
@@ -713,8 +716,7 @@ __global__ void __launch_bounds__(64 * kWalkWaves)
 bound_rows_walk_kernel(const float* __restrict__ xl, const float* __restrict__ xu, const float* __restrict__ wt,
                        const uint32_t* __restrict__ bits, const unsigned long long* __restrict__ count,
                        unsigned long long limit_col, unsigned long long limit_row, int B, int Bp, int M, int N,
-                       float* __restrict__ yL, float* __restrict__ yU, unsigned long long* __restrict__ packedL,
-                       unsigned long long* __restrict__ packedU) {
+                       float* __restrict__ yL, float* __restrict__ yU, int* __restrict__ posL, int* __restrict__ posU) {
     if (count[0] <= limit_col || count[1] > limit_row) return;   // the other table's turn, or the every-term kernel's
     __shared__ uint16_t list[kWalkWaves][kWalkListCap];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -731,7 +733,7 @@ bound_rows_walk_kernel(const float* __restrict__ xl, const float* __restrict__ x
     const float* __restrict__ xlrow = xl + (size_t)b * N;
     const float* __restrict__ xurow = xu + (size_t)b * N;
     float lo[2] = {-kEps, -kEps}, hi[2] = {kEps, kEps};
-    int cl[2] = {-1, -1}, cu[2] = {-1, -1};   // POS: chunk of the input that last improved the bound (-1: none)
+    int pl[2] = {-1, -1}, pu[2] = {0, 0};   // POS: the input that last improved the bound, with its flag
     int cnt = 0;   // marks in the list
     float lreg[2], ureg[2];
     int nreg[2];
@@ -758,13 +760,14 @@ bound_rows_walk_kernel(const float* __restrict__ xl, const float* __restrict__ x
                 const float ui = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ureg[buf]), i));
                 const float a1 = wa[buf][i] - li, a2 = ui - wa[buf][i], b1 = wb[buf][i] - li, b2 = ui - wb[buf][i];
                 if constexpr (POS) {
-                    const int c = __builtin_amdgcn_readlane(nreg[buf], i) >> 5;
+                    const int n = __builtin_amdgcn_readlane(nreg[buf], i);
+                    const int p0 = a1 <= a2 ? n : n | (int)0x80000000, p1 = b1 <= b2 ? n : n | (int)0x80000000;
                     const float v0 = fminf(a1, a2), V0 = fmaxf(a1, a2), v1 = fminf(b1, b2), V1 = fmaxf(b1, b2);
                     const bool w0 = v0 < lo[0], w1 = v1 < lo[1], w2 = V0 > hi[0], w3 = V1 > hi[1];
                     lo[0] = w0 ? v0 : lo[0]; lo[1] = w1 ? v1 : lo[1];
                     hi[0] = w2 ? V0 : hi[0]; hi[1] = w3 ? V1 : hi[1];
-                    cl[0] = w0 ? c : cl[0]; cl[1] = w1 ? c : cl[1];
-                    cu[0] = w2 ? c : cu[0]; cu[1] = w3 ? c : cu[1];
+                    pl[0] = w0 ? p0 : pl[0]; pl[1] = w1 ? p1 : pl[1];
+                    pu[0] = w2 ? p0 : pu[0]; pu[1] = w3 ? p1 : pu[1];
                 } else {
                     lo[0] = fminf(fminf(lo[0], a1), a2);
                     hi[0] = fmaxf(fmaxf(hi[0], a1), a2);
@@ -816,12 +819,8 @@ bound_rows_walk_kernel(const float* __restrict__ xl, const float* __restrict__ x
         const int col = t * kTileW + lane + 64 * j;
         if (col < M) {
             const size_t o = (size_t)b * M + col;
-            if constexpr (POS) {
-                if (cl[j] >= 0)
-                    packedL[o] = ((unsigned long long)__float_as_uint(-lo[j]) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)cl[j]);
-                if (cu[j] >= 0)
-                    packedU[o] = ((unsigned long long)__float_as_uint(hi[j]) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)cu[j]);
-            } else { yL[o] = -lo[j]; yU[o] = hi[j]; }
+            yL[o] = -lo[j]; yU[o] = hi[j];
+            if constexpr (POS) { posL[o] = pl[j]; posU[o] = pu[j]; }
         }
     }
 }
@@ -846,9 +845,9 @@ size_t bound_cols_workspace(int B, int CO, int CI) {
 }
 
 int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, int CO, int CI, float* outL,
-                       float* outU, unsigned long long* packedL, unsigned long long* packedU, void* ws, float density,
-                       float density_rows, const unsigned long long** gate, unsigned long long* gate_limit,
-                       hipStream_t st) {
+                       float* outU, unsigned long long* packedL, unsigned long long* packedU, int* posL, int* posU,
+                       void* ws, float density, float density_rows, const unsigned long long** gate,
+                       unsigned long long* gate_limit, hipStream_t st) {
     const bool with_pos = packedL != nullptr;
     if (CI % kChunk != 0 || B < 1 || CO < 1) { set_error("bound_cols_forward: shape not supported"); return SD_ERR_ARG; }
     const Carve c = carve(ws, B, CO, CI);
@@ -900,10 +899,10 @@ int bound_cols_forward(const float* xl, const float* xu, const float* w, int B, 
         // chunk numbers within a slice take 8 bits (255 = none)
         while ((((NCH + 1) / 2 + nsplit - 1) / nsplit) * 2 > 254) nsplit++;
         hipLaunchKernelGGL(bound_table_kernel<true>, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, w, c.xt, c.bits,
-                           c.order, c.count, limit_col, B, CO, Mp, CI, nsplit, outL, outU, packedL, packedU);
+                           c.order, c.count, limit_col, B, CO, Mp, CI, nsplit, nullptr, nullptr, packedL, packedU);
         if ((rc = check_launch("bound_table_kernel"))) return rc;
         hipLaunchKernelGGL(bound_rows_walk_kernel<true>, dim3((unsigned)(T * BG)), dim3(64 * kWalkWaves), 0, st, xl, xu, c.wt,
-                           c.bits, c.count, limit_col, limit_row, B, Bp, CO, CI, outL, outU, packedL, packedU);
+                           c.bits, c.count, limit_col, limit_row, B, Bp, CO, CI, outL, outU, posL, posU);
         return check_launch("bound_rows_walk_kernel");
     }
     hipLaunchKernelGGL(bound_table_kernel<false>, dim3((unsigned)(wgs * nsplit)), dim3(1024), 0, st, w, c.xt, c.bits, c.order,

@@ -62,6 +62,9 @@ struct FwdArgs {
     const unsigned long long* gate;
     unsigned long long gate_limit;
     int gate_above;
+    // interval forward with positions: non-null and non-zero on the device when a table kernel has already stored the
+    // final values and positions, so that resolve_bound_kernel has nothing to do
+    const unsigned long long* resolved;
 };
 
 __device__ __forceinline__ bool gate_closed(const unsigned long long* gate, unsigned long long limit, int above) {

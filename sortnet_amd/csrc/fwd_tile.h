@@ -1329,6 +1329,7 @@ struct ResolveBoundSlot { int cl, cu; float vl, vu; unsigned long long xoff, wof
 template <bool PACKED>
 __global__ void __launch_bounds__(256) resolve_bound_kernel(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) ResolveBoundSlot slots[4][64];
+    if (a.resolved != nullptr && *a.resolved != 0ull) return;   // (uniform over the launch)
     const long long total = (long long)a.R * a.G * a.COg;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const long long o_base = ((long long)blockIdx.x * 4 + wave) * 64;

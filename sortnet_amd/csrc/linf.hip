@@ -403,7 +403,7 @@ extern "C" int sd_bound_inf_dist_forward_nograd(const float* inputL, const float
     }
     if (cols) {
         void* ws = wsbase;
-        if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, outputL, outputU, nullptr, nullptr, ws, cap,
+        if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, outputL, outputU, nullptr, nullptr, nullptr, nullptr, ws, cap,
                                      bound_density >= 0.f ? bound_density : kBoundRowsCap, &a.gate, &a.gate_limit, st)))
             return rc;
         a.gate_above = 1;
@@ -464,10 +464,11 @@ extern "C" int sd_bound_inf_dist_forward(const float* inputL, const float* input
         a.packed1 = a.packed0 + n;
         if (a.nsplit > 1 && (rc = fill_zero(a.packed0, n * 4, st))) return rc;
         if (cols) {
-            if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, nullptr, nullptr, a.packed0, a.packed1,
+            if ((rc = bound_cols_forward(inputL, inputU, weight, B, CO, CI, outputL, outputU, a.packed0, a.packed1, posL, posU,
                                          ws + pairs, cap, cap, &a.gate, &a.gate_limit, st)))
                 return rc;
             a.gate_above = 1;
+            a.resolved = a.gate + 2;   // the tables per batch row store final values and positions themselves
         }
     }
     // exact dense tiles: the LDS-direct kernel with the chunk numbers packed (same (value, chunk) pairs, same resolve)
