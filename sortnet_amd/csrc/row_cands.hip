@@ -1,7 +1,5 @@
 // Sort neuron, its interval bounds and the l-inf forward from candidate tables per batch row (see row_cands.h).
 #include "row_cands.h"
-#include <type_traits>
-#include <utility>
 #include "fwd_tile.h"
 
 namespace sd {
@@ -97,11 +95,6 @@ __device__ __forceinline__ void insert_value(float (&res)[K], float v, float inf
     #pragma unroll
     for (int k = 0; k < K - 1; k++) res[k] = __builtin_amdgcn_fmed3f(res[k], v, res[k + 1]);
     res[K - 1] = __builtin_amdgcn_fmed3f(res[K - 1], v, inf);
-}
-
-template <class F, int... R>
-__device__ __forceinline__ void static_for(F&& f, std::integer_sequence<int, R...>) {
-    (f(std::integral_constant<int, R>{}), ...);
 }
 
 // ---- tables ----------------------------------------------------------------------------------
