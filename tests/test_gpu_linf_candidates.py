@@ -145,6 +145,36 @@ def test_linf_candidate_kernels_at_layer_size(knobs):
             assert torch.equal(a, b), dens
 
 
+def test_linf_row_tables_at_layer_size_with_built_in_limits(knobs):
+    """B = 512, 3072 -> 5120 (the first layer of the benchmark net): images against small weights.  With the built-in
+    limits the tables per batch row serve the plain and the masked forward, and values and positions are the
+    every-term kernels' bits."""
+    from sortnet_amd import ext, _lib
+    dev = _dev()
+    B, N, M = 512, 3072, 5120
+    g = torch.Generator().manual_seed(5)
+    x = torch.rand(B, N, 1, generator=g).contiguous().to(dev)
+    w = (torch.randn(M, N, generator=g) * N ** -0.5).contiguous().to(dev)
+    out = {}
+    for dens in (0.0, -1.0):
+        knobs(dens)
+        y, yn, ym = (torch.empty(B, M, 1, device=dev) for _ in range(3))
+        p = torch.empty(B, M, 1, device=dev, dtype=torch.int32)
+        pm = torch.empty_like(p)
+        ext.inf_dist_forward(x, w, y, p, 1)
+        share = _lib.last_forward_term_share()
+        ext.inf_dist_forward_nograd(x, w, yn, 1)
+        ext.masked_inf_dist_forward(x, w, ym, pm, 1, 0.3, 9, ext.MASK_FACTORED)
+        share_masked = _lib.last_forward_term_share()
+        out[dens] = (y, p, yn, ym, pm)
+        if dens < 0:
+            assert share < 0.15 and share_masked < 0.15, (share, share_masked)
+        else:
+            assert share == 1.0 and share_masked == 1.0, (share, share_masked)
+    for a, b in zip(out[-1.0], out[0.0]):
+        assert torch.equal(a, b)
+
+
 def test_linf_candidate_arguments(knobs):
     from sortnet_amd import _lib
     with pytest.raises(RuntimeError):
