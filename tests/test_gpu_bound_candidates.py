@@ -102,6 +102,29 @@ def test_bound_candidate_kernel_with_positions_matches_oracle(oracle, density, d
             assert np.array_equal(pu.cpu().numpy(), rpu), tag
 
 
+@pytest.mark.parametrize("kind", ["images", "rows_alike"])
+def test_bound_candidate_kernels_with_rows_longer_than_the_mark_lists(oracle, density, kind):
+    """The kernel of the tables per batch row lists marked inputs as 16-bit numbers: a layer with more than 65536 inputs
+    per row, forced into the tables, still gives the oracle's values and positions (from the tables per weight row or
+    from every term)."""
+    from sortnet_amd import ext
+    dev = _dev()
+    B, CI, CO = 8, 65568, 32
+    density(1.0)
+    xl, xu = _intervals(B, CI, kind, 11)
+    g = torch.Generator().manual_seed(12)
+    w = (torch.randn(CO, CI, generator=g) * 0.02).contiguous()
+    rl, ru, rpl, rpu = oracle.bound_inf_dist_forward(xl.numpy(), xu.numpy(), w.numpy(), 1, need_pos=True)
+    yl, yu = (torch.full((B, CO, 1), float("nan"), device=dev) for _ in range(2))
+    pl, pu = (torch.full((B, CO, 1), -7, device=dev, dtype=torch.int32) for _ in range(2))
+    ext.bound_inf_dist_forward(xl.to(dev), xu.to(dev), w.to(dev), yl, yu, pl, pu, 1)
+    assert np.array_equal(yl.cpu().numpy(), rl) and np.array_equal(yu.cpu().numpy(), ru)
+    assert np.array_equal(pl.cpu().numpy(), rpl) and np.array_equal(pu.cpu().numpy(), rpu)
+    yl2, yu2 = (torch.full((B, CO, 1), float("nan"), device=dev) for _ in range(2))
+    ext.bound_inf_dist_forward_nograd(xl.to(dev), xu.to(dev), w.to(dev), yl2, yu2, 1)
+    assert np.array_equal(yl2.cpu().numpy(), rl) and np.array_equal(yu2.cpu().numpy(), ru)
+
+
 def test_bound_candidate_kernel_with_positions_at_layer_size(density):
     """B = 512, N = M = 5120 with rows that are nearly alike: table kernel, every-term kernel and the built-in choice
     give the same values and positions."""
