@@ -146,12 +146,11 @@ def test_linf_candidate_kernels_at_layer_size(knobs):
 
 
 def test_linf_row_tables_at_layer_size_with_built_in_limits(knobs):
-    """B = 512, 3072 -> 5120 (the first layer of the benchmark net): images against small weights.  With the built-in
-    limits the tables per batch row serve the plain and the masked forward, and values and positions are the
-    every-term kernels' bits."""
+    """B = 512, N = M = 5120: images against small weights.  With the built-in limits the tables per batch row serve the
+    plain and the masked forward, and values and positions are the every-term kernels' bits."""
     from sortnet_amd import ext, _lib
     dev = _dev()
-    B, N, M = 512, 3072, 5120
+    B, N, M = 512, 5120, 5120
     g = torch.Generator().manual_seed(5)
     x = torch.rand(B, N, 1, generator=g).contiguous().to(dev)
     w = (torch.randn(M, N, generator=g) * N ** -0.5).contiguous().to(dev)
