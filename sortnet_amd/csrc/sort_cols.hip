@@ -75,7 +75,8 @@ __device__ __forceinline__ void repair(float& l, float& u) {
 
 // Top-K lists are kept as the bit patterns of their values (all >= 0, where signed integers order like the
 // floats): new[k] = max(res[k], min(res[k+1], v)) (core/cuda/sort_neuron.cu:76-77) = the median of the three, one integer
-// instruction per slot.  A negative v (sign bit set: a negative integer) is below every entry and changes nothing.
+// instruction per slot.  A negative v (sign bit set: a negative integer) is below every entry and changes nothing;
+// an undefined v with a clear sign bit would order above every number, so callers hand over defined values only.
 __device__ __forceinline__ int imed3(int a, int b, int c) {
     int r;
     asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
@@ -487,13 +488,18 @@ sc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
                     } else if constexpr (IV) {
                         const float a1 = wi - xa[buf][i].x, a2 = xa[buf][i].y - wi;
                         const float b1 = wi - xb[buf][i].x, b2 = xb[buf][i].y - wi;
-                        insert_bits<K>(lo[0], -fminf(a1, a2));
-                        insert_bits<K>(hi[0], fmaxf(a1, a2));
-                        insert_bits<K>(lo[1], -fminf(b1, b2));
-                        insert_bits<K>(hi[1], fmaxf(b1, b2));
+                        // (the maximum with -1 turns a term that is undefined altogether, whose bit pattern would
+                        // order above every number, into a negative one, which the lists ignore; three-operand
+                        // maxima, so it costs no instruction)
+                        insert_bits<K>(lo[0], fmaxf(fmaxf(-a1, -a2), -1.f));
+                        insert_bits<K>(hi[0], fmaxf(fmaxf(a1, a2), -1.f));
+                        insert_bits<K>(lo[1], fmaxf(fmaxf(-b1, -b2), -1.f));
+                        insert_bits<K>(hi[1], fmaxf(fmaxf(b1, b2), -1.f));
                     } else {
-                        insert_bits<K>(hi[0], fabsf(xa[buf][i] - wi));
-                        insert_bits<K>(hi[1], fabsf(xb[buf][i] - wi));
+                        // (the same for the value form: the maximum stands where the absolute value's own
+                        // instruction stood)
+                        insert_bits<K>(hi[0], fmaxf(fabsf(xa[buf][i] - wi), -1.f));
+                        insert_bits<K>(hi[1], fmaxf(fabsf(xb[buf][i] - wi), -1.f));
                     }
                 }
             }

@@ -144,6 +144,35 @@ def test_sort_candidate_kernels_at_layer_size(density):
             assert torch.equal(a, b), dens
 
 
+@pytest.mark.parametrize("kind", ["rows_alike", "pixels", "ties"])
+def test_sort_candidate_kernels_drop_undefined_terms(oracle, density, kind):
+    """Undefined and infinite inputs and weights: a term with an undefined operand is left out of the K largest
+    (include/sortdist.h), an infinite one counts.  The table kernels keep some of their lists as bit patterns, where an
+    undefined value would order above every number: they must agree with the every-term kernels and the oracle, in
+    both orientations of the tables (rows alike / pixels) and on ties."""
+    B, CI, CO, q, K = 150, 1024, 200, 0.4, 10
+    x, xl, xu, w = _data(B, CI, CO, kind, 11)
+    g = torch.Generator().manual_seed(12)
+    mx, mw = torch.rand(x.shape, generator=g), torch.rand(w.shape, generator=g)
+    for t in (x, xl, xu):
+        t[mx < 0.002] = float("nan")
+        t[(mx >= 0.002) & (mx < 0.003)] = float("inf")
+        t[(mx >= 0.003) & (mx < 0.004)] = float("-inf")
+    w[mw < 0.0005] = float("nan")
+    w[(mw >= 0.0005) & (mw < 0.001)] = float("inf")
+    w[(mw >= 0.001) & (mw < 0.0015)] = float("-inf")
+    ry, rpos = oracle.sort_neuron_forward(x.numpy(), w.numpy(), q, K)
+    rl, ru = oracle.bound_sort_neuron_forward(xl.numpy(), xu.numpy(), w.numpy(), q, K)
+    density(0.0)
+    every = _run(x, xl, xu, w, q, K)
+    for got, want in zip(every[:4], (ry, rl, ru, ry)):
+        np.testing.assert_allclose(got, want, rtol=RTOL, err_msg=kind)   # (infinities and undefined sums compare equal)
+    assert np.array_equal(every[4], rpos), kind
+    density(1.0)
+    for got, want in zip(_run(x, xl, xu, w, q, K), every):
+        assert np.array_equal(got, want, equal_nan=got.dtype.kind == "f"), kind
+
+
 def test_rows_longer_than_the_mark_lists_take_the_every_term_kernels(oracle, density):
     """The table kernels list marked inputs as 16-bit numbers: a dense layer with more than 65536 inputs per row
     (a multiple of 32, enough terms for the tables, density forced on) must fall back to the every-term kernels
