@@ -207,7 +207,13 @@ int sd_bound_sort_neuron_forward(const float* inputL, const float* inputU, const
                                  float q, int K, sd_stream_t stream);
 
 /* ---- l-p norm distance: template struct norm_dist<ip>, norm_dist.h:4-18.  The dispatch on p
- * that the reference does in its pybind layer (norm_dist.cpp:4,17-38,51-60) happens inside. ---- */
+ * that the reference does in its pybind layer (norm_dist.cpp:4,17-38,51-60) happens inside.
+ * Undefined (NaN) and infinite operands: the reference sums every term, so an output that meets such an operand is
+ * undefined there.  Here the forward never returns a finite value for such an output, whichever kernel serves the
+ * call (undefined, or infinite where a kernel leaves out the undefined term inf / inf), and every other output is
+ * unaffected.  The backward kernels leave out terms whose ratio to the output does not compare as significant, an
+ * undefined ratio among them, so the gradients that belong to a non-finite output are only partly undefined:
+ * callers detect such a state from the forward's output. ---- */
 
 /* norm_dist<ip>::forward / forward_with_max(max_output = nullptr) as selected by
  * norm_dist_forward (core/cuda/norm_dist.cpp:43-61; norm_dist_cuda.cu:512-552). */

@@ -68,18 +68,22 @@ __global__ void __launch_bounds__(256) tile_rowmin_kernel(const float* __restric
     if (wave >= B * T) return;
     const int b = wave / T, t = wave - b * T;
     float r = __builtin_inff();
+    float odd = 0.f;   // stays 0 while every scale of the tile is finite
     #pragma unroll
     for (int j = 0; j < kTileM / 64; j++) {
         const int m = t * kTileM + lane + 64 * j;
         if (m < M) {
             const float y = v[(size_t)b * M + m];
             r = fminf(r, y);
+            odd += y - y;
             if (RECIP) rv[(size_t)b * M + m] = 1.f / y;
         }
     }
     #pragma unroll
-    for (int o = 32; o; o >>= 1) r = fminf(r, __shfl_xor(r, o));
-    if (lane == 0) ymin[(size_t)t * Bp + b] = r;
+    for (int o = 32; o; o >>= 1) { r = fminf(r, __shfl_xor(r, o)); odd += __shfl_xor(odd, o); }
+    // an undefined or infinite scale makes the row's terms of the tile undefined: the bound becomes undefined, which
+    // cand_bits_kernel takes for a candidate at every input
+    if (lane == 0) ymin[(size_t)t * Bp + b] = r + odd;
 }
 
 // one wavefront per (row, tile): a lower bound of the largest |x[b,n] - w[m,n]| of every output channel m of the
@@ -116,7 +120,10 @@ __global__ void __launch_bounds__(256) cand_bits_kernel(const float* __restrict_
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int marks = 0;
     for (int t = wave; t < T; t += 4) {
-        const float lim = b < B ? thr * ymin[(size_t)t * Bp + b] : __builtin_inff();
+        // (an infinite bound - an infinite input - becomes undefined: every input of the row is a candidate, so the
+        // outputs come out undefined as they do when every term is formed)
+        const float s = ymin[(size_t)t * Bp + b];
+        const float lim = b < B ? thr * ((s - s) + s) : __builtin_inff();
         const float* __restrict__ wa = wabs + (size_t)t * N + c * kChunk;
         uint32_t word = 0;
         #pragma unroll

@@ -104,6 +104,35 @@ def test_candidate_kernels_undefined_entries_reach_their_outputs(oracle, density
     np.testing.assert_allclose(got[ok], ry[ok], rtol=RTOL)
 
 
+@pytest.mark.parametrize("dens", [1.0, 0.0])
+@pytest.mark.parametrize("p", [24.0, 256.0])
+def test_candidate_kernels_infinite_entries_reach_their_outputs(oracle, density, dens, p):
+    """An infinite input or weight makes the distance of every output it meets infinite and its scaled terms
+    undefined in the reference (inf / inf); here such an output is never finite either (undefined, or infinite where
+    the kernel skips the undefined term), and every other output is unchanged.  The scale of the affected rows is
+    infinite, which must not unmark the row's inputs in the table."""
+    from sortnet_amd import ext
+    dev = _dev()
+    density(dens)
+    B, CI, CO = 70, 352, 300
+    x, w = _gen((B, CI, 1), 31), _gen((CO, CI), 32, 0.3)
+    x[5, 100, 0] = float("inf")
+    x[40, 7, 0] = float("-inf")
+    w[17, 3] = float("inf")
+    w[280, 200] = float("-inf")
+    w[281, 7] = float("nan")
+    with np.errstate(invalid="ignore", over="ignore"):
+        ry = oracle.norm_dist_forward(x.numpy(), w.numpy(), p, 1)
+    bad = ~np.isfinite(ry)
+    assert bad[5].all() and bad[40].all() and bad[:, 17].all() and bad[:, 280].all() and bad[:, 281].all()
+    assert bad.sum() == 2 * CO + 3 * (B - 2)
+    y = torch.zeros(B, CO, 1, device=dev)
+    ext.norm_dist_forward(x.to(dev), w.to(dev), y, 1, p)
+    got = y.cpu().numpy()
+    assert np.array_equal(~np.isfinite(got), bad)
+    np.testing.assert_allclose(got[~bad], ry[~bad], rtol=RTOL)
+
+
 def test_candidate_density_argument(density):
     from sortnet_amd import _lib
     with pytest.raises(RuntimeError):
