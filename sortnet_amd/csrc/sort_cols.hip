@@ -594,6 +594,8 @@ mc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
     const int m = mb * kMainTile + wave;
     if (m < M) {   // wave-uniform
         const float* __restrict__ wrow = w + (size_t)m * N;
+        // per batch row of the lane: the difference of largest magnitude so far (its sign is the position's flag)
+        // and the input it sits at; without positions only the magnitude
         float best[2];
         int where[2];
         float wreg[2];
@@ -620,8 +622,14 @@ mc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
                     const int n = __builtin_amdgcn_readlane(nreg[buf], i);
                     const float d0 = xa[buf][i] - wi, d1 = xb[buf][i] - wi;
                     // an undefined difference (an input the row does not keep) never compares greater
-                    if (fabsf(d0) > best[0]) { best[0] = fabsf(d0); if (POS) where[0] = n | (d0 >= 0.f ? 0 : (int)kSign); }
-                    if (fabsf(d1) > best[1]) { best[1] = fabsf(d1); if (POS) where[1] = n | (d1 >= 0.f ? 0 : (int)kSign); }
+                    if constexpr (POS) {
+                        const bool g0 = fabsf(d0) > fabsf(best[0]), g1 = fabsf(d1) > fabsf(best[1]);
+                        best[0] = g0 ? d0 : best[0]; where[0] = g0 ? n : where[0];
+                        best[1] = g1 ? d1 : best[1]; where[1] = g1 ? n : where[1];
+                    } else {
+                        best[0] = fmaxf(best[0], fabsf(d0));
+                        best[1] = fmaxf(best[1], fabsf(d1));
+                    }
                 }
             }
         };
@@ -669,12 +677,12 @@ mc_main_kernel(const float* __restrict__ xT, const float* __restrict__ w, const 
         pass(bits + ((size_t)s * Mp + m) * NCH);
         const float bound = low[(size_t)(s * 2) * Mp + m];
         const int b0 = s * kTileB + lane;
-        const bool short0 = b0 < B && best[0] < bound, short1 = b0 + 64 < B && best[1] < bound;
+        const bool short0 = b0 < B && fabsf(best[0]) < bound, short1 = b0 + 64 < B && fabsf(best[1]) < bound;
         if (__builtin_amdgcn_ballot_w64(short0 || short1) != 0ull) pass(wkeep ? wkeep + (size_t)m * NCH : nullptr);
         #pragma unroll
         for (int j = 0; j < 2; j++) {
-            stage_y[lane + 64 * j][wave] = best[j];
-            if (POS) stage_p[lane + 64 * j][wave] = where[j];
+            stage_y[lane + 64 * j][wave] = fabsf(best[j]);
+            if (POS) stage_p[lane + 64 * j][wave] = where[j] | (best[j] >= 0.f ? 0 : (int)kSign);
         }
     }
     __syncthreads();
