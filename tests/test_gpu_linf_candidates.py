@@ -122,6 +122,26 @@ def test_masked_candidate_kernels_match_oracle(oracle, knobs, dens, depth, B, CI
             _check_masked(oracle, x, w, q, seed, "dens=%g depth=%d %s q=%g" % (dens, depth, kind, q), expect)
 
 
+@pytest.mark.parametrize("dens", [1.0, 0.0])
+@pytest.mark.parametrize("kind", ["rows_alike", "images", "ties"])
+def test_linf_candidate_kernels_with_undefined_and_infinite_operands(oracle, knobs, dens, kind):
+    """NaN and +-inf sprinkled into inputs and weights: an undefined difference never becomes the maximum (strict
+    comparisons, core/cuda/inf_dist_cuda.cu:176-190), an infinite one does, lowest input first.  Both table
+    orientations (rows alike / images) and the every-term kernels against the oracle, plain and under the mask."""
+    knobs(dens)
+    B, CI, CO = 150, 1024, 200
+    x, w = _data(B, CI, CO, kind, 41)
+    g = torch.Generator().manual_seed(42)
+    for t, frac in ((x, 0.002), (w, 0.0005)):
+        m = torch.rand(t.shape, generator=g)
+        t[m < frac] = float("nan")
+        t[(m >= frac) & (m < 2 * frac)] = float("inf")
+        t[(m >= 2 * frac) & (m < 3 * frac)] = float("-inf")
+    _check_plain(oracle, x, w, "dens=%g %s" % (dens, kind))
+    for q, seed in ((0.3, 5), (1.0, 3)):
+        _check_masked(oracle, x, w, q, seed, "dens=%g %s q=%g" % (dens, kind, q))
+
+
 def test_linf_candidate_kernels_at_layer_size(knobs):
     """B = 512, N = M = 5120, unit-scale weights against rows that are nearly alike: table kernels and every-term
     kernels give the same values and positions, plain and masked, and the built-in limit picks the table."""
