@@ -65,9 +65,10 @@ static int max_cols_wanted(const FwdArgs& a, int K, int site, int B, int CO, int
 // of it tables and the transposed copy of the weights) against 0.49 (0.61) for every term, 256 x 12288 x 10240 0.86
 // (0.89) against 1.28 (1.30), 512 x 3072 x 5120 0.26 (0.27) against 0.27 (0.43), 256 x 4096 x 2048 0.13 (0.13)
 // against 0.09 (0.12): the main kernel's time grows with the marks, so the limit sits where the two would meet at the
-// large sizes.  The path is a chain of fifteen launches where the every-term path has three, and a training step that
-// runs other streams beside it pays for every launch boundary: with the 512 x 3072 x 5120 layer served from tables the
-// benchmark step gained 0.1 ms on one stream and lost 0.05 ms on three, so the size limit sits above that layer.
+// large sizes.  With the 512 x 3072 x 5120 layer served from tables the benchmark step gained 0.1 ms on one stream and
+// lost 0.05 ms on three (presumably the table passes and the transposed copy, which stream the operands through
+// memory, meet the traffic of the optimizer and the backward on the other streams), so the size limit sits above
+// that layer.
 constexpr float kMaxRowsCap = 0.10f;
 constexpr long long kMaxRowsMinTerms = 1ll << 33;
 
