@@ -19,6 +19,8 @@ def _built_in_limits_afterwards():
     yield
     from sortnet_amd import _lib
     _lib.set_bound_candidate_density(-1.0)
+    _lib.set_linf_candidate_density(-1.0)
+    _lib.set_sort_candidate_density(-1.0)
 
 
 def _dev():
@@ -270,6 +272,76 @@ def test_graph_replays_of_the_candidate_table_kernels(oracle):
         # the kernels differentiated their own y, which agrees with the oracle's to rel 1e-5: (d/y)^(p-1) moves by p times that
         for got, ref in ((captured["gx"], rgx), (captured["gw"], rgw), (captured["gx2"], rgx)):
             np.testing.assert_allclose(got.cpu().numpy(), ref, rtol=2e-3, atol=2e-3 * float(np.abs(ref).max()))
+
+
+def test_graph_replays_of_both_table_orientations():
+    """The l-inf forward, the masked neuron, the sort neuron with positions and the interval forward with positions
+    queue the kernels of the tables per weight row, of the tables per batch row and the every-term kernels for one
+    result, and counts taken on the device pick one.  ONE captured graph must therefore serve batch rows that are alike
+    against weights of unit scale (tables per weight row), images against small weights (tables per batch row) and
+    unrelated rows (every term): every replay reproduces the eager calls and the calls with every table switched off,
+    bit for bit, values and positions."""
+    from sortnet_amd import ext, _lib
+    dev = _dev()
+    B, CI, CO, K = 160, 1024, 300, 6
+    g = torch.Generator().manual_seed(31)
+    x = torch.empty(B, CI, 1, device=dev); w = torch.empty(CO, CI, device=dev)
+
+    def limits(d):
+        _lib.set_bound_candidate_density(d); _lib.set_linf_candidate_density(d); _lib.set_sort_candidate_density(d)
+
+    def outputs():
+        f = lambda: torch.empty(B, CO, 1, device=dev)
+        i = lambda: torch.empty(B, CO, 1, device=dev, dtype=torch.int32)
+        return dict(y=f(), pos=i(), ym=f(), pm=i(), ys=f(), pk=torch.empty(K, B, CO, 1, device=dev, dtype=torch.int32),
+                    zl=f(), zu=f(), pl=i(), pu=i(), ysl=f(), ysu=f())
+
+    def run(o):
+        ext.inf_dist_forward(x, w, o["y"], o["pos"], 1)
+        ext.masked_inf_dist_forward(x, w, o["ym"], o["pm"], 1, 0.3, 9, ext.MASK_FACTORED)
+        ext.sort_neuron_forward(x, w, o["ys"], o["pk"], 1, 0.5, K)
+        ext.bound_inf_dist_forward(x - 0.03, x + 0.03, w, o["zl"], o["zu"], o["pl"], o["pu"], 1)
+        ext.bound_sort_neuron_forward(x - 0.03, x + 0.03, w, o["ysl"], o["ysu"], 1, 0.5, K)
+
+    def new_inputs(kind):
+        if kind == "alike":
+            x.copy_(torch.randn(1, CI, 1, generator=g) * 0.3 + torch.randn(B, CI, 1, generator=g) * 0.02)
+            w.copy_(torch.randn(CO, CI, generator=g))
+        elif kind == "images":
+            x.copy_(torch.rand(B, CI, 1, generator=g))
+            w.copy_(torch.randn(CO, CI, generator=g) * CI ** -0.5)
+        else:
+            x.copy_(torch.randn(B, CI, 1, generator=g))
+            w.copy_(torch.randn(CO, CI, generator=g))
+
+    limits(0.5)   # a limit set by hand applies at any size; the counts on the device still decide
+    new_inputs("images")
+    eager, captured, plain = outputs(), outputs(), outputs()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(captured)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run(captured)
+    served = {}
+    for replay, kind in enumerate(("images", "alike", "random", "images", "alike")):
+        new_inputs(kind)
+        run(eager)
+        served[kind] = _lib.last_forward_term_share()    # of the last call, the interval sort neuron
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        limits(0.0)
+        run(plain)
+        torch.cuda.synchronize()
+        limits(0.5)
+        for name in eager:
+            assert torch.equal(captured[name], eager[name]), "%s, replay %d (%s): graph against eager" % (name, replay, kind)
+            assert torch.equal(captured[name], plain[name]), "%s, replay %d (%s): tables against every term" % (name, replay, kind)
+    assert served["images"] < 1.0 and served["alike"] < 1.0 and served["random"] == 1.0, served
 
 
 def test_two_host_threads_on_one_stream_leave_results_unchanged():
